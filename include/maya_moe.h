@@ -1,0 +1,168 @@
+/* maya_moe.h - C ABI of the MI355X (gfx950) routed-MoE expert block.
+ *
+ * The library (libmaya_moe.so) replaces the reference engine's expert-rows operators on one GPU: router top-k, the
+ * per-expert grouping of a token batch, the activation quantizers, the fused dequant gate/up GLU mat-vec, the down
+ * mat-vec, the weighted combine, and the prefill grouped int8 GEMM.  Each entry point names the reference interface it
+ * stands in for (paths relative to the reference tree).
+ *
+ * Conventions (the reference's operator contract, include/strata/kernels/glm_fast.hpp:496-501, src/ds4/ds4_iq.cuh:60-91,
+ * include/strata/kernels/s2_expert_grouped.hpp:36-38):
+ *   - every pointer is DEVICE memory unless it says "host"; the caller owns every buffer, scratch included
+ *     (maya_moe_workspace_bytes gives the size); no entry point allocates, synchronizes or calls back to the host;
+ *   - `stream` is a hipStream_t passed as void*; work is asynchronous and ordered on it; calls on different streams
+ *     may overlap as long as they use different workspaces;
+ *   - routing results stay on the device: kernels read plans, groups and counts from device memory, so a launch
+ *     sequence does not depend on routing and can be captured in a HIP graph;
+ *   - a plan slot whose blob address is 0 is skipped (the expert is not resident here; its part is left out);
+ *   - weights are raw GGUF rows, row-major, [gate rows | up rows | down rows] per expert (offsets in maya_moe_layout),
+ *     aligned to 2 bytes or better;
+ *   - return value: 0 ok; > 0 "not covered, nothing launched" (MAYA_E_*); < 0 a HIP error (-hipError_t).
+ *     maya_last_error() returns a thread-local message for the last non-zero return.
+ */
+#ifndef MAYA_MOE_H
+#define MAYA_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids of the weight formats (src/ds4/ds4_iq.cuh:27-31) */
+#define MAYA_TYPE_Q8_0 8
+#define MAYA_TYPE_Q4_K 12
+#define MAYA_TYPE_IQ1_S 19
+#define MAYA_TYPE_IQ2_S 22
+#define MAYA_TYPE_IQ1_M 29
+
+/* element types of activations handed in by the caller */
+#define MAYA_DT_F32 0
+#define MAYA_DT_BF16 1
+#define MAYA_DT_F16 2
+
+#define MAYA_OK 0
+#define MAYA_E_UNSUPPORTED 1 /* a weight type, dtype or codebook this library has no kernel for */
+#define MAYA_E_SHAPE 2       /* a size outside what the kernels assume (not whole blocks, too many tokens, ...) */
+#define MAYA_E_ARG 3         /* a null pointer or a workspace that is too small */
+#define MAYA_E_NOGPU 4       /* no gfx950 device / the library's device code is not loadable */
+
+#define MAYA_MAX_K 16          /* experts per token */
+#define MAYA_MAX_TOKENS 16     /* tokens of one decode / verify-window call */
+#define MAYA_MAX_EXPERTS 1024  /* router width */
+
+/* One layer's expert geometry: strata::kernels::cpu::NativeFmt (include/strata/kernels/cpu/native_expert.hpp:26-39),
+ * iq::Args::tr / tg / td (src/ds4/ds4_iq.cuh:72-84). */
+typedef struct maya_moe_layout {
+    int32_t gate_type, up_type, down_type; /* ggml ids; gate and up must share the activation format */
+    int32_t n_embd, n_ff;                  /* multiples of 256 */
+    uint64_t gate_off, up_off, down_off;   /* byte offsets of the three row arrays inside an expert blob */
+} maya_moe_layout;
+
+/* A quantized activation batch in device memory (rows x k): int8 codes, an F32 scale per 32 values (a 256-value
+ * Q8_K block's scale is written 8 times, as ds4's xd / hd hold it: src/ds4/ds4_lane_parity.hpp:40-42) and ggml's
+ * bsums (the sum of every 16 codes, third_party/ggml/ggml-common.h:371-376). */
+typedef struct maya_act {
+    int8_t* q;      /* [rows][k] */
+    float* d;       /* [rows][k/32] */
+    int16_t* bsums; /* [rows][k/16] */
+} maya_act;
+
+/* The token / window experts: iq::Args (src/ds4/ds4_iq.cuh:66-87), glmf::MoeDev's plan_ptr / plan_w / skip / cpu_part /
+ * cpu_flag (include/strata/kernels/glm_fast.hpp:293-318).  Entry e = token e / k, slot e % k.  Group g = one distinct
+ * expert and the entries routed to it; with grp_ptr == NULL the groups are the plan itself (group g = entry g). */
+typedef struct maya_moe_args {
+    maya_moe_layout layout;
+    int32_t n_tokens, k;
+    const uint64_t* plan_ptr;  /* [n_tokens*k] blob address of each entry's expert (0: skipped) */
+    const float* plan_w;       /* [n_tokens*k] combine weights */
+    const uint64_t* grp_ptr;   /* [<= n_tokens*k] or NULL */
+    const int32_t* grp_start;  /* [groups+1] */
+    const int32_t* grp_ent;    /* [n_tokens*k] */
+    const int32_t* n_groups;   /* device count of groups (NULL: n_tokens*k) */
+    const int32_t* skip;       /* NULL or a device flag: non-zero makes every kernel of the call a no-op */
+    float limit;               /* SwiGLU clamp; +inf or <= 0: none */
+    maya_act x;                /* gate/up input, rows = tokens (maya_quant_act of the hidden state) */
+    float* h;                  /* [n_tokens*k][n_ff] SwiGLU output */
+    maya_act hq;               /* down input, rows = entries (maya_quant_act of h) */
+    float* part;               /* [n_tokens*k][n_embd] each entry's down output (NULL in the fused 1-token form) */
+    const float* add;          /* NULL or [n_tokens][n_embd] added to the combined output (shared expert, CPU lane part) */
+    const int32_t* add_flag;   /* NULL or a device flag: `add` is added only when it is non-zero */
+    float* out;                /* [n_tokens][n_embd] */
+} maya_moe_args;
+
+/* ---- probes: glmf::moe_supported, iq::supported / block_bytes / row_bytes (src/ds4/ds4_iq.cuh:40-52) */
+int maya_moe_supported(int ggml_type);
+int maya_moe_block_bytes(int ggml_type);
+int maya_moe_block_values(int ggml_type);
+size_t maya_moe_row_bytes(int ggml_type, int64_t k);
+/* fills off/sizes for the contiguous [gate|up|down] blob: native_fmt / native_fmt_mixed
+ * (src/kernels/cpu/native_expert.cpp:195-260); returns the blob's bytes (0: unsupported) */
+size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int down_type, int n_embd, int n_ff);
+
+const char* maya_last_error(void);
+/* Device and library identification: "gfx950 ..." (host string, valid until the next call on this thread). */
+const char* maya_device_info(void);
+/* Loads the device code and uploads the codebooks on the current device; idempotent.  Every other entry point calls it. */
+int maya_init(void);
+
+/* ---- dequantization to F32, bit-exact with the block formats' reference decode:
+ * dequantize_q4_K / dequantize_q8_0 (include/strata/artifact/dequant.hpp:81-85, 162-190), dq_iq2_s / dq_iq1_s /
+ * dq_iq1_m + iq_dequant_f32 (src/kernels/cuda/iq_kernels.cu:686-695, 825-855, 1038-1075), iq::decode_values
+ * (src/ds4/ds4_iq.cuh:171-175).  w: n_rows rows of k values, row_stride bytes apart (0: the type's own row size). */
+int maya_dequant_rows(int ggml_type, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out,
+                      void* stream);
+
+/* ---- activation quantizers.  act_type = the WEIGHT type whose dot will consume the activation:
+ * Q8_K rounding for the 256-value types - quantize_q8_K (src/kernels/cuda/quantize_act.cu:161-207), q8k_quant_kernel
+ * (src/ds4/ds4_gguf.cu:299-336), native_quant_act / native_quant_h (src/kernels/cpu/native_expert.cpp:262-268);
+ * Q8_0 rounding for Q8_0 weights - quantize_q8_0 (include/strata/kernels/quantize_act.hpp:28-31).
+ * x: rows x k of x_dtype, x_stride elements apart (0: k). */
+int maya_quant_act(int act_type, const void* x, int x_dtype, int64_t x_stride, int rows, int64_t k, maya_act out,
+                   void* stream);
+/* per-32 int8 + F32 scale, the prefill form: quant_act_nat_kernel (src/prefill/moe_fused_rdna4.cu:87-109),
+ * q8_quant_kernel (src/ds4/ds4_gguf.cu:219-227), mmq::quantize (src/prefill/moe_mmq.cu:120-157).
+ * row_idx: NULL or a gather table (row r reads x[row_idx[r]]). */
+int maya_quant_i8x32(const void* x, int x_dtype, int64_t x_stride, const int32_t* row_idx, int rows, int64_t k,
+                     int8_t* q, float* d, void* stream);
+
+/* ---- router: strata::kernels::router_top10 (src/kernels/cuda/router_top10.cu:191-224): softmax over all experts in
+ * double, stable top-k (strict >, lower index on ties) on the float probabilities, renormalised by max(sum, 2^-14). */
+int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights,
+                        void* stream);
+/* ids -> plan: plan_ptr[e] = expert_table[ids[e]] (0 stays 0: not resident), the plan part of moe_route_kernel
+ * (src/kernels/cuda/glm_fast.cu:3998-4545) without its residency tiers. */
+int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,
+                  void* stream);
+/* plan -> groups of distinct experts, in first-appearance order, entries of a group ascending:
+ * moe_win_group_kernel (src/kernels/cuda/glm_fast.cu:7545-7625), MoeWin (include/strata/kernels/glm_fast.hpp:439-458).
+ * grp_ptr / grp_ent: [n_entries]; grp_start: [n_entries+1]; n_groups: [1]. */
+int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, int32_t* grp_start, int32_t* grp_ent,
+                   int32_t* n_groups, void* stream);
+
+/* ---- the expert rows.
+ * maya_moe_gate_up: h[e][r] = swiglu(gate_r . x[token(e)], up_r . x[token(e)]) for every entry:
+ *   glmf::moe_gate_up (include/strata/kernels/glm_fast.hpp:496-498), iq::gate_up (src/ds4/ds4_iq.cuh:88-89),
+ *   native_gu_rows_split (src/kernels/cpu/native_expert.cpp:343-393).
+ * maya_moe_down: part[e][r] = down_r . hq[e], then out[t] = sum_i plan_w[t*k+i] * part[t*k+i] (+ add[t]) in slot order:
+ *   glmf::moe_down (glm_fast.hpp:499-501), iq::down (ds4_iq.cuh:90-91), native_down_rows_split
+ *   (native_expert.cpp:395-417), native_moe_combine (src/kernels/cuda/native_moe.cu:36-52). */
+int maya_moe_gate_up(const maya_moe_args* a, void* stream);
+int maya_moe_down(const maya_moe_args* a, void* stream);
+
+/* ---- the whole routed layer for a decode step / verify window of n_tokens <= MAYA_MAX_TOKENS tokens:
+ * route -> plan -> group -> quantize x -> gate/up -> quantize h -> down -> combine, every step on `stream`, nothing on
+ * the host (the sequence of glm_fast_path.cu:2688-2691 and ds4_gguf.cu:1903-1971).
+ *   expert_table: [n_expert] device array of blob addresses (0: not resident);
+ *   x: [n_tokens][n_embd] of x_dtype; out: [n_tokens][n_embd] F32; ids / weights: [n_tokens][k] results of the router;
+ *   workspace: maya_moe_workspace_bytes(layout, n_tokens, k) bytes, 256-byte aligned. */
+size_t maya_moe_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k);
+int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                          const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                          int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

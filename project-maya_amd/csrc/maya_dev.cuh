@@ -1,0 +1,196 @@
+// maya_dev.cuh - device-side building blocks shared by the kernels: scalar conversions, unaligned loads, wave64
+// reductions and the per-format decoders of a quantized block into int8 codes and integer scales.
+//
+// One decoded "unit" of a row is the work of one lane for one step.  Every format reduces to
+//     w_i = D * s_h * q_i  (- M_j for Q4_K)          q_i an int8 code, s_h an integer scale per 16 or 32 values
+// so a unit's contribution to a row sum against an int8 activation (codes y, F32 scale dy per 32) is
+//     D * dy * sum_h s_h * dot(q_h, y_h)   [ - Dmin * dy * sum_j m_j * sum(y_j) ]
+// with every dot an exact integer (v_dot4_i32_i8).  This is the arithmetic of the reference's exact-decode kernels
+// (src/ds4/ds4_iq.cu:178-184, 285-297, 347-361, 426-432; ds4_iq.cuh:7-13) and of its CPU contract
+// (src/kernels/cpu/iq_avx2.cpp:225-250, 332-394): exact block integers, F32 scales, no integer division.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace maya {
+
+constexpr int kQ8_0 = 8, kQ4_K = 12, kIQ1_S = 19, kIQ2_S = 22, kIQ1_M = 29;
+constexpr int kWave = 64;
+
+// ------------------------------------------------------------------------------------------------ scalars
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    // exact for every bit pattern (subnormals, infinities): the hardware conversion
+    return __half2float(__ushort_as_half((unsigned short) h));
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+typedef uint32_t __attribute__((aligned(2))) u32_a2;
+typedef uint16_t __attribute__((aligned(1))) u16_a1;
+// 4 bytes from a 2-byte aligned address (GGUF blocks are 2-byte aligned: their sizes are not multiples of 4)
+__device__ __forceinline__ uint32_t ld32_a2(const uint8_t* p) { return *(const u32_a2*) p; }
+__device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *(const uint16_t*) p; }
+
+__device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+
+// sum over the lanes of an aligned group of `width` lanes (a power of two <= 64); every lane gets the sum
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+    for (int o = WIDTH / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------ codebooks
+
+// Expanded on the host at init (maya_init) into device memory; kernels stage what they need into LDS.
+struct Codebooks {
+    const uint64_t* iq2s;  // 1024 x 8 magnitudes
+    const uint64_t* iq1s;  // 2048 x 8 values -1 / 0 / +1
+};
+
+// four sign bits -> 0x01 in the bytes of the set bits (bit i -> byte i); the 16 partial products land on distinct bits
+__device__ __forceinline__ uint32_t spread4(uint32_t nib) { return (nib * 0x00204081u) & 0x01010101u; }
+// negate the bytes of g that c marks with 0x01 (g's bytes in 1..127): (g ^ 0xff) + 1 per byte, no carry across bytes
+__device__ __forceinline__ uint32_t neg_bytes(uint32_t g, uint32_t c) {
+    const uint32_t m = (c << 8) - c;  // 0xff in the marked bytes
+    return (g ^ m) + c;
+}
+
+// ------------------------------------------------------------------------------------------------ decoders
+//
+// Fmt<TYPE>: kBytes / kValues of a block; kUnit values a lane takes a step; decode(blk, u, cb) fills codes and scales.
+
+struct Unit32 {
+    int q[8];    // 32 int8 codes in value order
+    int s0, s1;  // integer scales of values 0..15 / 16..31
+};
+
+template <int TYPE> struct Fmt;
+
+template <> struct Fmt<kIQ2_S> {
+    static constexpr int kBytes = 82, kValues = 256, kUnit = 32, kLdsWords = 2048;  // codebook: 1024 x u64
+    static constexpr bool kMin = false;
+    __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
+    // third_party/ggml/ggml-common.h:396-402; decode: src/kernels/cuda/iq_kernels.cu:686-695
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
+        const uint32_t i4 = ld32_a2(blk + 2 + 4 * ib), sg4 = ld32_a2(blk + 34 + 4 * ib);
+        const uint32_t h = blk[66 + ib], sc = blk[74 + ib];
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint32_t idx = ((i4 >> (8 * l)) & 255u) | ((h << (8 - 2 * l)) & 0x300u);
+            const uint2 g = grid[idx];
+            const uint32_t sb = (sg4 >> (8 * l)) & 255u;
+            u.q[2 * l] = (int) neg_bytes(g.x, spread4(sb & 15u));
+            u.q[2 * l + 1] = (int) neg_bytes(g.y, spread4(sb >> 4));
+        }
+        u.s0 = 2 * (int) (sc & 15u) + 1;
+        u.s1 = 2 * (int) (sc >> 4) + 1;
+    }
+};
+
+// IQ1_S / IQ1_M: the +-1/8 shift of each grid value rides in the integer dot: codes 8 g +- 1, scale d / 8
+// (src/ds4/ds4_iq.cuh:11-13).  Grid bytes are -1 / 0 / +1: 8 g as bytes is (g << 3) per byte, done on the u32 with the
+// sign bytes handled by two's complement: 8 * 0xff = 0xf8 (= -8) needs no carry when done per byte via a multiply of the
+// separated positive / negative masks.
+__device__ __forceinline__ uint32_t iq1_codes(uint32_t g, uint32_t delta_byte) {
+    // g bytes in {0xff, 0x00, 0x01}.  pos = bytes equal to 1, neg = bytes equal to 0xff (bit 1 set only there)
+    const uint32_t neg = (g >> 1) & 0x01010101u, pos = g & ~(g >> 1) & 0x01010101u;
+    // 8 g + delta per byte, delta = +1 (0x01) or -1 (0xff): bytes stay within -9..9, assembled without cross-byte carries
+    // as (pos*8) | (neg * 0xf8) then a per-byte add of delta through the carry-free form below
+    const uint32_t v = (pos << 3) | ((neg << 8) - (neg << 3));  // 0x08 / 0xf8 / 0x00
+    // per-byte add of delta_byte (0x01010101 or 0xffffffff): add the low 7 bits, fix the top bit by xor
+    const uint32_t lo = (v & 0x7f7f7f7fu) + (delta_byte & 0x7f7f7f7fu);
+    return lo ^ ((v ^ delta_byte) & 0x80808080u);
+}
+
+template <> struct Fmt<kIQ1_S> {
+    static constexpr int kBytes = 50, kValues = 256, kUnit = 32, kLdsWords = 4096;  // codebook: 2048 x u64
+    static constexpr bool kMin = false;
+    __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
+    // third_party/ggml/ggml-common.h:425-430; decode: src/kernels/cuda/iq_kernels.cu:825-837
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
+        const uint32_t q4 = ld32_a2(blk + 2 + 4 * ib), qh = ld16(blk + 34 + 2 * ib);
+        const uint32_t delta = (qh & 0x8000u) ? 0xffffffffu : 0x01010101u;
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint2 g = grid[((q4 >> (8 * l)) & 255u) | (((qh >> (3 * l)) & 7u) << 8)];
+            u.q[2 * l] = (int) iq1_codes(g.x, delta);
+            u.q[2 * l + 1] = (int) iq1_codes(g.y, delta);
+        }
+        u.s0 = u.s1 = 2 * (int) ((qh >> 12) & 7u) + 1;
+    }
+};
+
+template <> struct Fmt<kIQ1_M> {
+    static constexpr int kBytes = 56, kValues = 256, kUnit = 32, kLdsWords = 4096;
+    static constexpr bool kMin = false;
+    // the FP16 super-scale sits in the top nibbles of the four u16 scale words (src/kernels/cpu/iq_avx2.cpp:471-475)
+    __device__ static __forceinline__ float scale(const uint8_t* blk) {
+        const uint32_t s0 = ld16(blk + 48), s1 = ld16(blk + 50), s2 = ld16(blk + 52), s3 = ld16(blk + 54);
+        return f16_bits_to_f32((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u)) * 0.125f;
+    }
+    // third_party/ggml/ggml-common.h:433-438; decode: src/kernels/cuda/iq_kernels.cu:839-855
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
+        const uint32_t q4 = ld32_a2(blk + 4 * ib), qh = ld16(blk + 32 + 2 * ib);
+        const uint32_t sc = ld16(blk + 48 + 2 * (ib >> 1)) >> (6 * (ib & 1));
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint32_t nib = (qh >> (4 * l)) & 15u;
+            const uint32_t delta = (nib & 8u) ? 0xffffffffu : 0x01010101u;
+            const uint2 g = grid[((q4 >> (8 * l)) & 255u) | ((nib & 7u) << 8)];
+            u.q[2 * l] = (int) iq1_codes(g.x, delta);
+            u.q[2 * l + 1] = (int) iq1_codes(g.y, delta);
+        }
+        u.s0 = 2 * (int) (sc & 7u) + 1;
+        u.s1 = 2 * (int) ((sc >> 3) & 7u) + 1;
+    }
+};
+
+template <> struct Fmt<kQ8_0> {
+    static constexpr int kBytes = 34, kValues = 32, kUnit = 32, kLdsWords = 0;
+    static constexpr bool kMin = false;
+    __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)); }
+    // third_party/ggml/ggml-common.h:252-256; a unit is one block
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int, const uint2*, Unit32& u) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u.q[i] = (int) ld32_a2(blk + 2 + 4 * i);
+        u.s0 = u.s1 = 1;
+    }
+};
+
+// Q4_K: a unit is a pair of sub-blocks (64 values) sharing 32 bytes of nibbles
+// (third_party/ggml/ggml-common.h:327-338; include/strata/artifact/dequant.hpp:152-190)
+struct UnitQ4K {
+    int lo[8], hi[8];  // sub-block 2p (low nibbles), 2p+1 (high nibbles)
+    int sc0, sc1, m0, m1;
+};
+__device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, int& m) {
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
+        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+}
+template <> struct Fmt<kQ4_K> {
+    static constexpr int kBytes = 144, kValues = 256, kUnit = 64, kLdsWords = 0;
+    static constexpr bool kMin = true;
+    __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)); }
+    __device__ static __forceinline__ float scale_min(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk + 2)); }
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int p, UnitQ4K& u) {
+        const uint8_t* q = blk + 16 + 32 * p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t w = ld32_a2(q + 4 * i);
+            u.lo[i] = (int) (w & 0x0f0f0f0fu);
+            u.hi[i] = (int) ((w >> 4) & 0x0f0f0f0fu);
+        }
+        q4k_scale_min(blk + 4, 2 * p, u.sc0, u.m0);
+        q4k_scale_min(blk + 4, 2 * p + 1, u.sc1, u.m1);
+    }
+};
+
+}  // namespace maya

@@ -1,0 +1,1001 @@
+// maya_kernels.hip - gfx950 kernels of the routed-MoE expert block and their C ABI (include/maya_moe.h).
+//
+// Data layout in HBM: expert weights stay in their GGUF rows (row-major, [gate | up | down] per expert); activations
+// are int8 codes with an F32 scale per 32 values (maya_act); routing state (ids, weights, plan, groups) lives in device
+// arrays that only kernels read.  All kernels are HBM-bound integer work: a lane streams quantized blocks, expands them to
+// int8 codes in registers (codebooks staged in LDS), takes exact v_dot4_i32_i8 sums against the int8 activation held in
+// LDS and scales them in F32; rows are reduced across the lanes of a wavefront-64 with shuffles.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "../../include/maya_moe.h"
+#include "maya_dev.cuh"
+#include "maya_iq_grids.h"
+
+namespace maya {
+
+// ------------------------------------------------------------------------------------------------ host state
+
+thread_local char g_err[512] = "";
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+int hip_fail(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof g_err, "%s: %s", what, hipGetErrorString(e));
+    return -(int) e;
+}
+#define MAYA_HIP(call)                                         \
+    do {                                                       \
+        const hipError_t e_ = (call);                          \
+        if (e_ != hipSuccess) return hip_fail(e_, #call);      \
+    } while (0)
+#define MAYA_LAUNCHED(name)                                    \
+    do {                                                       \
+        const hipError_t e_ = hipGetLastError();               \
+        if (e_ != hipSuccess) return hip_fail(e_, name);       \
+    } while (0)
+
+constexpr int kMaxDevices = 16;
+struct DeviceState {
+    bool ready = false;
+    Codebooks cb{};
+    int lds_limit = 65536;
+};
+DeviceState g_dev[kMaxDevices];
+std::mutex g_init_mu;
+
+int current_state(DeviceState** out) {
+    int dev = 0;
+    MAYA_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(MAYA_E_NOGPU, "device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    DeviceState& s = g_dev[dev];
+    if (!s.ready) {
+        std::lock_guard<std::mutex> lock(g_init_mu);
+        if (!s.ready) {
+            hipDeviceProp_t p;
+            MAYA_HIP(hipGetDeviceProperties(&p, dev));
+            if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+                return fail(MAYA_E_NOGPU, "device %d is %s; this library holds gfx950 code only", dev, p.gcnArchName);
+            static const uint8_t m2[4] = {8, 25, 43, 0}, m1[4] = {0xff, 0x00, 0x01, 0};
+            uint64_t* host = new uint64_t[1024 + 2048];
+            for (int i = 0; i < 1024; ++i) {
+                uint64_t v = 0;
+                for (int j = 0; j < 8; ++j) v |= (uint64_t) m2[(maya_iq2s_packed[i] >> (2 * j)) & 3] << (8 * j);
+                host[i] = v;
+            }
+            for (int i = 0; i < 2048; ++i) {
+                uint64_t v = 0;
+                for (int j = 0; j < 8; ++j) v |= (uint64_t) m1[(maya_iq1s_packed[i] >> (2 * j)) & 3] << (8 * j);
+                host[1024 + i] = v;
+            }
+            uint64_t* d = nullptr;
+            hipError_t e = hipMalloc((void**) &d, sizeof(uint64_t) * (1024 + 2048));
+            if (e == hipSuccess) e = hipMemcpy(d, host, sizeof(uint64_t) * (1024 + 2048), hipMemcpyHostToDevice);
+            delete[] host;
+            if (e != hipSuccess) return hip_fail(e, "codebook upload");
+            s.cb.iq2s = d;
+            s.cb.iq1s = d + 1024;
+            s.lds_limit = (int) p.sharedMemPerBlock;
+            s.ready = true;
+        }
+    }
+    *out = &s;
+    return MAYA_OK;
+}
+
+inline hipStream_t as_stream(void* s) { return (hipStream_t) s; }
+
+// ------------------------------------------------------------------------------------------------ dequantize
+//
+// One thread a value; the float steps are the reference decode's, each rounded once (no contraction), so the output is
+// the block format's value to the bit.
+
+template <int TYPE>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, size_t row_stride, int64_t k,
+                                                      float* __restrict__ out, Codebooks cb) {
+    const int64_t row = blockIdx.y;
+    const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;  // value index in the row
+    if (v >= k) return;
+    const uint8_t* rp = w + (size_t) row * row_stride;
+    float r;
+    if constexpr (TYPE == kQ8_0) {
+        const uint8_t* blk = rp + (size_t) (v >> 5) * 34;
+        r = __fmul_rn((float) (int8_t) blk[2 + (v & 31)], f16_bits_to_f32(ld16(blk)));
+    } else if constexpr (TYPE == kQ4_K) {
+        const uint8_t* blk = rp + (size_t) (v >> 8) * 144;
+        const int i = (int) (v & 255), j = i >> 5, l = i & 31;
+        int sc, m;
+        q4k_scale_min(blk + 4, j, sc, m);
+        const float d1 = __fmul_rn(f16_bits_to_f32(ld16(blk)), (float) sc);
+        const float m1 = __fmul_rn(f16_bits_to_f32(ld16(blk + 2)), (float) m);
+        const uint8_t qb = blk[16 + 32 * (j >> 1) + l];
+        const int q = (j & 1) ? (qb >> 4) : (qb & 15);
+        r = __fsub_rn(__fmul_rn(d1, (float) q), m1);
+    } else if constexpr (TYPE == kIQ2_S) {
+        const uint8_t* blk = rp + (size_t) (v >> 8) * 82;
+        const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
+        const uint32_t idx = blk[2 + 4 * ib + il] | (((uint32_t) blk[66 + ib] << (8 - 2 * il)) & 0x300u);
+        const uint64_t g = cb.iq2s[idx];
+        const int ls = (blk[74 + ib] >> (4 * (il >> 1))) & 15;
+        const float dl = __fmul_rn(__fmul_rn(f16_bits_to_f32(ld16(blk)), __fadd_rn(0.5f, (float) ls)), 0.25f);
+        const float mag = __fmul_rn(dl, (float) (uint32_t) ((g >> (8 * j)) & 255u));
+        r = (blk[34 + 4 * ib + il] >> j) & 1 ? -mag : mag;
+    } else if constexpr (TYPE == kIQ1_S) {
+        const uint8_t* blk = rp + (size_t) (v >> 8) * 50;
+        const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
+        const uint32_t qh = ld16(blk + 34 + 2 * ib);
+        const uint64_t g = cb.iq1s[blk[2 + 4 * ib + il] | (((qh >> (3 * il)) & 7u) << 8)];
+        const float dl = __fmul_rn(f16_bits_to_f32(ld16(blk)), (float) (2 * (int) ((qh >> 12) & 7u) + 1));
+        const float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
+        r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
+    } else {  // IQ1_M
+        const uint8_t* blk = rp + (size_t) (v >> 8) * 56;
+        const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
+        const uint32_t nib = (blk[32 + 2 * ib + (il >> 1)] >> (4 * (il & 1))) & 15u;
+        const int ib16 = 2 * ib + (il >> 1);
+        const int s = (ld16(blk + 48 + 2 * (ib16 >> 2)) >> (3 * (ib16 & 3))) & 7;
+        const uint64_t g = cb.iq1s[blk[4 * ib + il] | ((nib & 7u) << 8)];
+        const float d = Fmt<kIQ1_M>::scale(blk) * 8.0f;  // scale() carries the 1/8 of the integer-code form
+        const float dl = __fmul_rn(d, (float) (2 * s + 1));
+        const float delta = (nib & 8u) ? -0.125f : 0.125f;
+        r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
+    }
+    out[(size_t) row * k + v] = r;
+}
+
+// ------------------------------------------------------------------------------------------------ activation quantizers
+
+template <int DT> __device__ __forceinline__ float load_x(const void* x, int64_t i) {
+    if constexpr (DT == MAYA_DT_F32) return ((const float*) x)[i];
+    else if constexpr (DT == MAYA_DT_BF16) return bf16_bits_to_f32(((const uint16_t*) x)[i]);
+    else return f16_bits_to_f32(((const uint16_t*) x)[i]);
+}
+
+// ggml's nearest_int: the magic-number round (ties to even) of a product already rounded to F32
+__device__ __forceinline__ int nearest_int(float f) {
+    const float v = __fadd_rn(f, 12582912.0f);
+    return (__float_as_int(v) & 0x007fffff) - 0x00400000;
+}
+
+// Q8_K: one workgroup of 256 threads a 256-value block (src/kernels/cuda/quantize_act.cu:161-207).  The block's signed
+// maximum is the value at the FIRST largest magnitude: the reduction keeps (|x|, index) and prefers the lower index.
+template <int DT>
+__global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__ x, int64_t x_stride, int64_t k,
+                                                        maya_act out) {
+    const int row = blockIdx.y, b = blockIdx.x, j = threadIdx.x;
+    const float xv = load_x<DT>(x, (int64_t) row * x_stride + (int64_t) b * 256 + j);
+    float am = fabsf(xv);
+    int ix = j;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float oa = __shfl_xor(am, o, kWave);
+        const int oi = __shfl_xor(ix, o, kWave);
+        if (oa > am || (oa == am && oi < ix)) {
+            am = oa;
+            ix = oi;
+        }
+    }
+    __shared__ float s_am[4];
+    __shared__ int s_ix[4];
+    __shared__ float s_x[256];
+    s_x[j] = xv;
+    if ((j & 63) == 0) {
+        s_am[j >> 6] = am;
+        s_ix[j >> 6] = ix;
+    }
+    __syncthreads();
+    am = s_am[0];
+    ix = s_ix[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+        if (s_am[w] > am) {  // later waves hold higher indices: only a strictly larger magnitude replaces
+            am = s_am[w];
+            ix = s_ix[w];
+        }
+    int q = 0;
+    float d = 0.0f;
+    if (am > 0.0f) {
+        const float iscale = __fdiv_rn(-127.0f, s_x[ix]);
+        q = min(127, nearest_int(__fmul_rn(iscale, xv)));
+        d = __fdiv_rn(1.0f, iscale);
+    }
+    const size_t base = (size_t) row * k + (size_t) b * 256;
+    out.q[base + j] = (int8_t) q;
+    int s = q;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+    if ((j & 15) == 0) out.bsums[(base >> 4) + (j >> 4)] = (int16_t) s;
+    if (j < 8) out.d[(base >> 5) + j] = d;
+}
+
+// Q8_0: 32-value blocks, d = amax / 127 kept as FP16, q = roundf(x / d) with the unrounded F32 d
+// (include/strata/kernels/quantize_act.hpp:28-31).  256 threads = 8 blocks.
+template <int DT>
+__global__ __launch_bounds__(256) void quant_q80_kernel(const void* __restrict__ x, int64_t x_stride, int64_t k,
+                                                        maya_act out) {
+    const int row = blockIdx.y, j = threadIdx.x;
+    const int64_t v = (int64_t) blockIdx.x * 256 + j;
+    const float xv = load_x<DT>(x, (int64_t) row * x_stride + v);
+    float am = fabsf(xv);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, kWave));
+    const float d = __fdiv_rn(am, 127.0f);
+    const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+    const int q = (int) roundf(__fmul_rn(xv, id));
+    const size_t base = (size_t) row * k + v;
+    out.q[base] = (int8_t) q;
+    int s = q;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+    if ((j & 15) == 0) out.bsums[base >> 4] = (int16_t) s;
+    if ((j & 31) == 0) out.d[base >> 5] = __half2float(__float2half_rn(d));
+}
+
+// per-32 int8 with an F32 scale: c = rint(x * (127 / amax)), d = amax / 127 (src/prefill/moe_fused_rdna4.cu:87-109)
+template <int DT>
+__global__ __launch_bounds__(256) void quant_i8x32_kernel(const void* __restrict__ x, int64_t x_stride,
+                                                          const int32_t* __restrict__ row_idx, int64_t k,
+                                                          int8_t* __restrict__ q, float* __restrict__ d) {
+    const int row = blockIdx.y, j = threadIdx.x;
+    const int64_t v = (int64_t) blockIdx.x * 256 + j;
+    const int64_t src = row_idx ? row_idx[row] : row;
+    const float xv = load_x<DT>(x, src * x_stride + v);
+    float am = fabsf(xv);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, kWave));
+    const float inv = am > 0.0f ? __fdiv_rn(127.0f, am) : 0.0f;
+    q[(size_t) row * k + v] = (int8_t) nearest_int(__fmul_rn(xv, inv));
+    if ((j & 31) == 0) d[((size_t) row * k + v) >> 5] = __fdiv_rn(am, 127.0f);
+}
+
+// ------------------------------------------------------------------------------------------------ router
+
+// One workgroup a token (src/kernels/cuda/router_top10.cu:68-187): the maximum (exact in any order), the exponentials in
+// double in parallel, their sum ascending on one thread, p = (float)(ex * inv) with inv a float, k rounds of a
+// workgroup-wide arg-max with a strict > and the lower index on ties, renormalisation by max(sum, 2^-14) in double.
+__global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k,
+                                                     int32_t* __restrict__ ids, float* __restrict__ weights) {
+    __shared__ double s_ex[MAYA_MAX_EXPERTS];
+    __shared__ float s_p[MAYA_MAX_EXPERTS];
+    __shared__ float s_rv[4];
+    __shared__ int s_ri[4];
+    __shared__ double s_sum;
+    __shared__ float s_w[MAYA_MAX_K];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const float* l = logits + (size_t) t * n_expert;
+    float mx = -INFINITY;
+    for (int e = tid; e < n_expert; e += 256) mx = fmaxf(mx, l[e]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    if ((tid & 63) == 0) s_rv[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_rv[0], s_rv[1]), fmaxf(s_rv[2], s_rv[3]));
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += 256) s_ex[e] = exp((double) l[e] - (double) mx);
+    __syncthreads();
+    if (tid == 0) {
+        double sum = 0.0;
+        for (int e = 0; e < n_expert; ++e) sum += s_ex[e];
+        s_sum = sum;
+    }
+    __syncthreads();
+    const float inv = (float) (1.0 / s_sum);
+    for (int e = tid; e < n_expert; e += 256) s_p[e] = (float) (s_ex[e] * (double) inv);
+    __syncthreads();
+    for (int i = 0; i < k; ++i) {
+        float bv = -INFINITY;
+        int bi = n_expert;
+        for (int e = tid; e < n_expert; e += 256) {
+            const float pe = s_p[e];
+            if (pe > bv) {
+                bv = pe;
+                bi = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, kWave);
+            const int oi = __shfl_xor(bi, o, kWave);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if ((tid & 63) == 0) {
+            s_rv[tid >> 6] = bv;
+            s_ri[tid >> 6] = bi;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float v = s_rv[0];
+            int ix = s_ri[0];
+            for (int w = 1; w < 4; ++w)
+                if (s_rv[w] > v || (s_rv[w] == v && s_ri[w] < ix)) {
+                    v = s_rv[w];
+                    ix = s_ri[w];
+                }
+            if (ix >= n_expert) ix = 0;  // only when every remaining probability is NaN
+            ids[(size_t) t * k + i] = ix;
+            s_w[i] = s_p[ix];
+            s_p[ix] = -INFINITY;  // taken: never selected again (a probability is >= 0)
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        double s = 0.0;
+        for (int i = 0; i < k; ++i) s += (double) s_w[i];
+        const double sc = fmax(s, 6.103515625e-05);
+        for (int i = 0; i < k; ++i) weights[(size_t) t * k + i] = (float) ((double) s_w[i] / sc);
+    }
+}
+
+__global__ void plan_kernel(const int32_t* __restrict__ ids, int n, const uint64_t* __restrict__ table, int n_expert,
+                            uint64_t* __restrict__ plan) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const int id = ids[e];
+    plan[e] = (id >= 0 && id < n_expert) ? table[id] : 0ull;
+}
+
+// Groups of distinct experts in first-appearance order, a group's entries ascending (what the reference's one-thread
+// grouping produces, src/kernels/cuda/glm_fast.cu:7545-7590).  n <= 256 entries: one workgroup, entry e's thread finds the
+// first entry with its blob (its group's leader); leaders are ranked by a prefix count; members are ranked inside their
+// group the same way.  Entries with a null blob belong to no group.
+__global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__ plan, int n,
+                                                    uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
+                                                    int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups) {
+    __shared__ uint64_t s_ptr[256];
+    __shared__ int s_leader[256];   // the first entry with the same blob, -1 for a null blob
+    __shared__ int s_gidx[256];     // leader entry -> group index
+    __shared__ int s_count[256];    // group -> entries
+    __shared__ int s_start[257];
+    __shared__ int s_ng;
+    const int e = threadIdx.x;
+    s_ptr[e] = e < n ? plan[e] : 0ull;
+    s_count[e] = 0;
+    __syncthreads();
+    int leader = -1;
+    if (e < n && s_ptr[e] != 0ull) {
+        leader = e;
+        for (int f = 0; f < e; ++f)
+            if (s_ptr[f] == s_ptr[e]) {
+                leader = f;
+                break;
+            }
+    }
+    s_leader[e] = leader;
+    __syncthreads();
+    if (leader == e) {
+        int g = 0;
+        for (int f = 0; f < e; ++f) g += s_leader[f] == f;
+        s_gidx[e] = g;
+    }
+    __syncthreads();
+    int rank = 0, g = -1;
+    if (leader >= 0) {
+        g = s_gidx[leader];
+        for (int f = 0; f < e; ++f) rank += s_leader[f] == leader;
+        atomicAdd(&s_count[g], 1);
+        if (leader == e) grp_ptr[g] = s_ptr[e];
+    }
+    __syncthreads();
+    if (e == 0) {
+        int ng = 0, acc = 0;
+        for (int f = 0; f < n; ++f) ng += s_leader[f] == f;
+        for (int i = 0; i < ng; ++i) {
+            s_start[i] = acc;
+            acc += s_count[i];
+        }
+        s_start[ng] = acc;
+        *n_groups = ng;
+        s_ng = ng;
+    }
+    __syncthreads();
+    const int ng = s_ng;
+    if (e <= ng) grp_start[e] = s_start[e];
+    if (g >= 0) grp_ent[s_start[g] + rank] = e;
+}
+
+// ------------------------------------------------------------------------------------------------ expert rows
+
+// LDS view of up to NT staged activation rows of k values
+struct ActLds {
+    const int* q;          // [NT][k/4]
+    const float* d;        // [NT][k/32]
+    const int* bs2;        // [NT][k/32] pairs of int16 bsums as one word (Q4_K only)
+    int kq, kd;            // strides in words: k/4, k/32
+};
+
+// One row against NT activations: the lanes of an aligned group of LPR lanes share the row's units; acc[t] holds this
+// lane's part.  `sub` = lane index inside the group.
+template <int TYPE, int NT, int LPR>
+__device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, int sub, const ActLds& a,
+                                        const uint2* __restrict__ grid, float (&acc)[NT]) {
+    if constexpr (TYPE == kQ4_K) {
+        const int np = k >> 6;
+        for (int p = sub; p < np; p += LPR) {
+            const uint8_t* blk = row + (size_t) (p >> 2) * 144;
+            UnitQ4K u;
+            Fmt<kQ4_K>::decode(blk, p & 3, u);
+            const float D = Fmt<kQ4_K>::scale(blk), Dm = Fmt<kQ4_K>::scale_min(blk);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int* y = a.q + t * a.kq + p * 16;
+                int lo = 0, hi = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    lo = dot4(u.lo[i], y[i], lo);
+                    hi = dot4(u.hi[i], y[8 + i], hi);
+                }
+                const int b0 = a.bs2[t * a.kd + 2 * p], b1 = a.bs2[t * a.kd + 2 * p + 1];
+                const int ms = u.m0 * ((int) (short) (b0 & 0xffff) + (b0 >> 16)) +
+                               u.m1 * ((int) (short) (b1 & 0xffff) + (b1 >> 16));
+                const float dy = a.d[t * a.kd + 2 * p];
+                acc[t] = fmaf(__fmul_rn(dy, D), (float) (u.sc0 * lo + u.sc1 * hi), acc[t]);
+                acc[t] = fmaf(-__fmul_rn(dy, Dm), (float) ms, acc[t]);
+            }
+        }
+    } else {
+        const int nu = k >> 5;
+        for (int un = sub; un < nu; un += LPR) {
+            const uint8_t* blk;
+            int ib;
+            if constexpr (TYPE == kQ8_0) {
+                blk = row + (size_t) un * 34;
+                ib = 0;
+            } else {
+                blk = row + (size_t) (un >> 3) * Fmt<TYPE>::kBytes;
+                ib = un & 7;
+            }
+            Unit32 u;
+            Fmt<TYPE>::decode(blk, ib, grid, u);
+            const float D = Fmt<TYPE>::scale(blk);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int* y = a.q + t * a.kq + un * 8;
+                int lo = 0, hi = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    lo = dot4(u.q[i], y[i], lo);
+                    hi = dot4(u.q[4 + i], y[4 + i], hi);
+                }
+                acc[t] = fmaf(__fmul_rn(D, a.d[t * a.kd + un]), (float) (u.s0 * lo + u.s1 * hi), acc[t]);
+            }
+        }
+    }
+}
+
+template <int TYPE> __device__ __forceinline__ const uint64_t* codebook_of(const Codebooks& cb) {
+    if constexpr (TYPE == kIQ2_S) return cb.iq2s;
+    else if constexpr (TYPE == kIQ1_S || TYPE == kIQ1_M) return cb.iq1s;
+    else return nullptr;
+}
+
+// stage the codebook (once) and NT activation rows into LDS; rows[t] = the activation row of staged slot t (-1: none)
+template <int TYPE, int NT>
+__device__ __forceinline__ void stage_act(int* lds_act, int k, const maya_act& src, const int (&rows)[NT], bool want_bs) {
+    const int kq = k >> 2, kd = k >> 5;
+    int* q = lds_act;
+    float* d = (float*) (lds_act + NT * kq);
+    int* bs = lds_act + NT * kq + NT * kd;
+    for (int t = 0; t < NT; ++t) {
+        if (rows[t] < 0) continue;
+        const int* sq = (const int*) (src.q + (size_t) rows[t] * k);
+        const float* sd = src.d + (size_t) rows[t] * kd;
+        for (int i = threadIdx.x; i < kq; i += blockDim.x) q[t * kq + i] = sq[i];
+        for (int i = threadIdx.x; i < kd; i += blockDim.x) d[t * kd + i] = sd[i];
+        if (want_bs) {
+            const int* sb = (const int*) (src.bsums + (size_t) rows[t] * (k >> 4));
+            for (int i = threadIdx.x; i < kd; i += blockDim.x) bs[t * kd + i] = sb[i];
+        }
+    }
+}
+
+struct GroupRef {
+    uint64_t blob;
+    int e0, ne;          // entries [e0, e0 + ne) of grp_ent (or the single entry e0 when grp_ent is null)
+};
+__device__ __forceinline__ bool group_of(const maya_moe_args& a, int g, GroupRef& r) {
+    if (a.skip && *a.skip) return false;
+    const int total = a.n_tokens * a.k;
+    if (a.grp_ptr) {
+        if (g >= *a.n_groups) return false;
+        r.blob = a.grp_ptr[g];
+        r.e0 = a.grp_start[g];
+        r.ne = a.grp_start[g + 1] - r.e0;
+    } else {
+        if (g >= total) return false;
+        r.blob = a.plan_ptr[g];
+        r.e0 = g;
+        r.ne = 1;
+    }
+    return r.blob != 0ull && r.ne > 0;
+}
+__device__ __forceinline__ int entry_of(const maya_moe_args& a, const GroupRef& r, int i) {
+    return a.grp_ptr ? a.grp_ent[r.e0 + i] : r.e0;
+}
+
+__device__ __forceinline__ float swiglu(float g, float u, float limit) {
+    if (limit > 0.0f && limit < INFINITY) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
+}
+
+constexpr int kGuThreads = 512, kGuRows = 32;   // a workgroup: 8 waves, 32 gate + 32 up rows
+constexpr int kDnThreads = 512, kDnRows = 64;   // 8 waves x 4 rows a pass, 2 passes
+
+// grid (n_ff / kGuRows, groups): wave w takes row pairs w, w + 8, ...: lanes 0..31 the gate row, 32..63 the up row
+template <int TG, int TU, int NT>
+__global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Codebooks cb) {
+    extern __shared__ int lds[];
+    GroupRef gr;
+    if (!group_of(a, blockIdx.y, gr)) return;
+    const int k = a.layout.n_embd, n_ff = a.layout.n_ff;
+    // the codebooks of the gate and of the up type (one copy when they share it)
+    constexpr int cbg = Fmt<TG>::kLdsWords, cbu = Fmt<TG>::kLdsWords == Fmt<TU>::kLdsWords ? 0 : Fmt<TU>::kLdsWords;
+    constexpr int cbw = cbg + cbu;
+    if constexpr (cbg > 0) {
+        const int* src = (const int*) codebook_of<TG>(cb);
+        for (int i = threadIdx.x; i < cbg; i += kGuThreads) lds[i] = src[i];
+    }
+    if constexpr (cbu > 0) {
+        const int* src = (const int*) codebook_of<TU>(cb);
+        for (int i = threadIdx.x; i < cbu; i += kGuThreads) lds[cbg + i] = src[i];
+    }
+    const uint2* grid_g = (const uint2*) lds;
+    const uint2* grid_u = (const uint2*) (lds + (cbu > 0 ? cbg : 0));
+    int* lds_act = lds + cbw;
+    const int kq = k >> 2, kd = k >> 5;
+    ActLds al{lds_act, (const float*) (lds_act + NT * kq), lds_act + NT * kq + NT * kd, kq, kd};
+    const uint8_t* blob = (const uint8_t*) gr.blob;
+    const size_t grow = (size_t) (k / Fmt<TG>::kValues) * Fmt<TG>::kBytes, urow = (size_t) (k / Fmt<TU>::kValues) * Fmt<TU>::kBytes;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31;
+    const bool is_up = lane >= 32;
+    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
+        int ents[NT], rows[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            ents[t] = c0 + t < gr.ne ? entry_of(a, gr, c0 + t) : -1;
+            rows[t] = ents[t] >= 0 ? ents[t] / a.k : -1;
+        }
+        __syncthreads();
+        stage_act<TG, NT>(lds_act, k, a.x, rows, Fmt<TG>::kMin || Fmt<TU>::kMin);
+        __syncthreads();
+        for (int r = blockIdx.x * kGuRows + wave; r < min(n_ff, (int) (blockIdx.x + 1) * kGuRows); r += kGuThreads / 64) {
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+            if constexpr (TG == TU) {
+                const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) r * grow;
+                row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc);
+            } else {
+                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) r * grow, k, sub, al, grid_g, acc);
+                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) r * urow, k, sub, al, grid_u, acc);
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float s = group_sum<32>(acc[t]);
+                const float up = __shfl(s, 32, kWave);
+                if (lane == 0 && ents[t] >= 0) a.h[(size_t) ents[t] * n_ff + r] = swiglu(s, up, a.limit);
+            }
+        }
+    }
+}
+
+// grid (n_embd / kDnRows, groups): a wave takes 4 rows a pass, 16 lanes a row
+template <int TD, int NT>
+__global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codebooks cb) {
+    extern __shared__ int lds[];
+    GroupRef gr;
+    if (!group_of(a, blockIdx.y, gr)) return;
+    const int k = a.layout.n_ff, n_embd = a.layout.n_embd;
+    constexpr int cbw = Fmt<TD>::kLdsWords;
+    if constexpr (cbw > 0) {
+        const int* src = (const int*) codebook_of<TD>(cb);
+        for (int i = threadIdx.x; i < cbw; i += kDnThreads) lds[i] = src[i];
+    }
+    const uint2* grid = (const uint2*) lds;
+    int* lds_act = lds + cbw;
+    const int kq = k >> 2, kd = k >> 5;
+    ActLds al{lds_act, (const float*) (lds_act + NT * kq), lds_act + NT * kq + NT * kd, kq, kd};
+    const uint8_t* base = (const uint8_t*) gr.blob + a.layout.down_off;
+    const size_t drow = (size_t) (k / Fmt<TD>::kValues) * Fmt<TD>::kBytes;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, rsub = lane >> 4;
+    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
+        int ents[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? entry_of(a, gr, c0 + t) : -1;
+        __syncthreads();
+        stage_act<TD, NT>(lds_act, k, a.hq, ents, Fmt<TD>::kMin);
+        __syncthreads();
+        const int r_end = min(n_embd, (int) (blockIdx.x + 1) * kDnRows);
+        for (int r = blockIdx.x * kDnRows + wave * 4 + rsub; r < r_end; r += (kDnThreads / 64) * 4) {
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+            row_dot<TD, NT, 16>(base + (size_t) r * drow, k, sub, al, grid, acc);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float s = group_sum<16>(acc[t]);
+                if (sub == 0 && ents[t] >= 0) a.part[(size_t) ents[t] * n_embd + r] = s;
+            }
+        }
+    }
+}
+
+// out[t][c] = sum_i w[t*k+i] * part[t*k+i][c] in slot order, each product and sum rounded (native_moe.cu:36-52);
+// skipped slots (null blob) are left out; + add[t][c] when given and flagged
+__global__ __launch_bounds__(256) void combine_kernel(maya_moe_args a) {
+    if (a.skip && *a.skip) return;
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x, n = a.layout.n_embd;
+    if (c >= n) return;
+    float sum = 0.0f;
+    bool first = true;
+    for (int i = 0; i < a.k; ++i) {
+        const int e = t * a.k + i;
+        if (a.plan_ptr[e] == 0ull) continue;
+        const float p = __fmul_rn(a.part[(size_t) e * n + c], a.plan_w[e]);
+        sum = first ? p : __fadd_rn(sum, p);
+        first = false;
+    }
+    if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[(size_t) t * n + c]);
+    a.out[(size_t) t * n + c] = sum;
+}
+
+// ------------------------------------------------------------------------------------------------ host launchers
+
+bool type_ok(int t) { return t == kQ8_0 || t == kQ4_K || t == kIQ1_S || t == kIQ2_S || t == kIQ1_M; }
+bool q8k_act(int t) { return t != kQ8_0; }
+int block_bytes(int t) {
+    switch (t) {
+        case kQ8_0: return 34;
+        case kQ4_K: return 144;
+        case kIQ1_S: return 50;
+        case kIQ2_S: return 82;
+        case kIQ1_M: return 56;
+        default: return 0;
+    }
+}
+int block_values(int t) { return t == kQ8_0 ? 32 : (type_ok(t) ? 256 : 0); }
+int codebook_words(int t) { return t == kIQ2_S ? 2048 : (t == kIQ1_S || t == kIQ1_M) ? 4096 : 0; }
+size_t act_lds_bytes(int k, int nt) { return (size_t) nt * ((size_t) k + (size_t) (k / 32) * 8); }
+
+int check_layout(const maya_moe_layout& l) {
+    if (!type_ok(l.gate_type) || !type_ok(l.up_type) || !type_ok(l.down_type))
+        return fail(MAYA_E_UNSUPPORTED, "expert types %d/%d/%d: no kernel", l.gate_type, l.up_type, l.down_type);
+    if (q8k_act(l.gate_type) != q8k_act(l.up_type))
+        return fail(MAYA_E_UNSUPPORTED, "gate type %d and up type %d quantize their activation differently", l.gate_type,
+                    l.up_type);
+    if (l.n_embd <= 0 || l.n_ff <= 0 || l.n_embd % 256 || l.n_ff % 256)
+        return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d: multiples of 256 wanted", l.n_embd, l.n_ff);
+    if (l.n_embd > 16384 || l.n_ff > 16384) return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d past 16384", l.n_embd, l.n_ff);
+    return MAYA_OK;
+}
+int check_args(const maya_moe_args* a) {
+    if (!a) return fail(MAYA_E_ARG, "null args");
+    if (const int rc = check_layout(a->layout)) return rc;
+    if (a->n_tokens < 1 || a->n_tokens > MAYA_MAX_TOKENS || a->k < 1 || a->k > MAYA_MAX_K)
+        return fail(MAYA_E_SHAPE, "n_tokens %d / k %d outside 1..%d / 1..%d", a->n_tokens, a->k, MAYA_MAX_TOKENS, MAYA_MAX_K);
+    if (!a->plan_ptr || !a->plan_w) return fail(MAYA_E_ARG, "null plan");
+    if (a->grp_ptr && (!a->grp_start || !a->grp_ent || !a->n_groups)) return fail(MAYA_E_ARG, "incomplete groups");
+    return MAYA_OK;
+}
+
+template <int TG, int TU>
+int launch_gate_up_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    const int nt = a.grp_ptr ? (a.n_tokens >= 4 ? 4 : a.n_tokens >= 2 ? 2 : 1) : 1;
+    const int cbw = codebook_words(TG) + (codebook_words(TG) == codebook_words(TU) ? 0 : codebook_words(TU));
+    const size_t lds = (size_t) cbw * 4 + act_lds_bytes(a.layout.n_embd, nt);
+    if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    const dim3 grid((unsigned) ((a.layout.n_ff + kGuRows - 1) / kGuRows), (unsigned) (a.n_tokens * a.k));
+    if (nt == 4) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 4>), grid, dim3(kGuThreads), lds, s, a, st.cb);
+    else if (nt == 2) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 2>), grid, dim3(kGuThreads), lds, s, a, st.cb);
+    else hipLaunchKernelGGL((gate_up_kernel<TG, TU, 1>), grid, dim3(kGuThreads), lds, s, a, st.cb);
+    MAYA_LAUNCHED("gate_up_kernel");
+    return MAYA_OK;
+}
+template <int TD>
+int launch_down_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    const int nt = a.grp_ptr ? (a.n_tokens >= 4 ? 4 : a.n_tokens >= 2 ? 2 : 1) : 1;
+    const size_t lds = (size_t) codebook_words(TD) * 4 + act_lds_bytes(a.layout.n_ff, nt);
+    if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    const dim3 grid((unsigned) ((a.layout.n_embd + kDnRows - 1) / kDnRows), (unsigned) (a.n_tokens * a.k));
+    if (nt == 4) hipLaunchKernelGGL((down_kernel<TD, 4>), grid, dim3(kDnThreads), lds, s, a, st.cb);
+    else if (nt == 2) hipLaunchKernelGGL((down_kernel<TD, 2>), grid, dim3(kDnThreads), lds, s, a, st.cb);
+    else hipLaunchKernelGGL((down_kernel<TD, 1>), grid, dim3(kDnThreads), lds, s, a, st.cb);
+    MAYA_LAUNCHED("down_kernel");
+    return MAYA_OK;
+}
+
+}  // namespace maya
+
+using namespace maya;
+
+// ================================================================================================= C ABI
+
+extern "C" {
+
+const char* maya_last_error(void) { return g_err; }
+
+int maya_init(void) {
+    DeviceState* st;
+    return current_state(&st);
+}
+
+const char* maya_device_info(void) {
+    static thread_local char buf[256];
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) {
+        snprintf(buf, sizeof buf, "no device");
+        return buf;
+    }
+    snprintf(buf, sizeof buf, "%s %s cus=%d lds=%zu clock_khz=%d mem_clock_khz=%d bus_bits=%d", p.gcnArchName, p.name,
+             p.multiProcessorCount, p.sharedMemPerBlock, p.clockRate, p.memoryClockRate, p.memoryBusWidth);
+    return buf;
+}
+
+int maya_moe_supported(int t) { return type_ok(t) ? 1 : 0; }
+int maya_moe_block_bytes(int t) { return block_bytes(t); }
+int maya_moe_block_values(int t) { return block_values(t); }
+size_t maya_moe_row_bytes(int t, int64_t k) {
+    return type_ok(t) && k % block_values(t) == 0 ? (size_t) (k / block_values(t)) * (size_t) block_bytes(t) : 0;
+}
+size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int down_type, int n_embd, int n_ff) {
+    if (!l) return 0;
+    l->gate_type = gate_type;
+    l->up_type = up_type;
+    l->down_type = down_type;
+    l->n_embd = n_embd;
+    l->n_ff = n_ff;
+    l->gate_off = l->up_off = l->down_off = 0;
+    if (check_layout(*l) != MAYA_OK) return 0;
+    l->up_off = maya_moe_row_bytes(gate_type, n_embd) * (size_t) n_ff;
+    l->down_off = l->up_off + maya_moe_row_bytes(up_type, n_embd) * (size_t) n_ff;
+    return l->down_off + maya_moe_row_bytes(down_type, n_ff) * (size_t) n_embd;
+}
+
+int maya_dequant_rows(int t, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!type_ok(t)) return fail(MAYA_E_UNSUPPORTED, "dequant: type %d", t);
+    if (!w || !out) return fail(MAYA_E_ARG, "dequant: null pointer");
+    if (k <= 0 || k % block_values(t) || n_rows <= 0 || n_rows > 65535)
+        return fail(MAYA_E_SHAPE, "dequant: k %lld rows %lld", (long long) k, (long long) n_rows);
+    if (row_stride == 0) row_stride = maya_moe_row_bytes(t, k);
+    const dim3 grid((unsigned) ((k + 255) / 256), (unsigned) n_rows);
+    const uint8_t* wb = (const uint8_t*) w;
+    hipStream_t s = as_stream(stream);
+    switch (t) {
+        case kQ8_0: hipLaunchKernelGGL(dequant_kernel<kQ8_0>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+        case kQ4_K: hipLaunchKernelGGL(dequant_kernel<kQ4_K>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+        case kIQ2_S: hipLaunchKernelGGL(dequant_kernel<kIQ2_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+        case kIQ1_S: hipLaunchKernelGGL(dequant_kernel<kIQ1_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+        default: hipLaunchKernelGGL(dequant_kernel<kIQ1_M>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+    }
+    MAYA_LAUNCHED("dequant_kernel");
+    return MAYA_OK;
+}
+
+int maya_quant_act(int act_type, const void* x, int x_dtype, int64_t x_stride, int rows, int64_t k, maya_act out,
+                   void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!type_ok(act_type)) return fail(MAYA_E_UNSUPPORTED, "quant_act: weight type %d", act_type);
+    if (x_dtype < 0 || x_dtype > 2) return fail(MAYA_E_UNSUPPORTED, "quant_act: dtype %d", x_dtype);
+    if (!x || !out.q || !out.d || !out.bsums) return fail(MAYA_E_ARG, "quant_act: null pointer");
+    if (rows <= 0 || rows > 65535 || k <= 0 || k % 256) return fail(MAYA_E_SHAPE, "quant_act: rows %d k %lld", rows, (long long) k);
+    if (x_stride == 0) x_stride = k;
+    const dim3 grid((unsigned) (k / 256), (unsigned) rows);
+    hipStream_t s = as_stream(stream);
+#define MAYA_Q(KERNEL)                                                                                              \
+    switch (x_dtype) {                                                                                              \
+        case MAYA_DT_F32: hipLaunchKernelGGL(KERNEL<MAYA_DT_F32>, grid, dim3(256), 0, s, x, x_stride, k, out); break;   \
+        case MAYA_DT_BF16: hipLaunchKernelGGL(KERNEL<MAYA_DT_BF16>, grid, dim3(256), 0, s, x, x_stride, k, out); break; \
+        default: hipLaunchKernelGGL(KERNEL<MAYA_DT_F16>, grid, dim3(256), 0, s, x, x_stride, k, out); break;            \
+    }
+    if (q8k_act(act_type)) {
+        MAYA_Q(quant_q8k_kernel)
+    } else {
+        MAYA_Q(quant_q80_kernel)
+    }
+#undef MAYA_Q
+    MAYA_LAUNCHED("quant_act kernel");
+    return MAYA_OK;
+}
+
+int maya_quant_i8x32(const void* x, int x_dtype, int64_t x_stride, const int32_t* row_idx, int rows, int64_t k, int8_t* q,
+                     float* d, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (x_dtype < 0 || x_dtype > 2) return fail(MAYA_E_UNSUPPORTED, "quant_i8x32: dtype %d", x_dtype);
+    if (!x || !q || !d) return fail(MAYA_E_ARG, "quant_i8x32: null pointer");
+    if (rows <= 0 || rows > 65535 || k <= 0 || k % 256) return fail(MAYA_E_SHAPE, "quant_i8x32: rows %d k %lld", rows, (long long) k);
+    if (x_stride == 0) x_stride = k;
+    const dim3 grid((unsigned) (k / 256), (unsigned) rows);
+    hipStream_t s = as_stream(stream);
+    switch (x_dtype) {
+        case MAYA_DT_F32: hipLaunchKernelGGL(quant_i8x32_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, x, x_stride, row_idx, k, q, d); break;
+        case MAYA_DT_BF16: hipLaunchKernelGGL(quant_i8x32_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, x, x_stride, row_idx, k, q, d); break;
+        default: hipLaunchKernelGGL(quant_i8x32_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, x, x_stride, row_idx, k, q, d); break;
+    }
+    MAYA_LAUNCHED("quant_i8x32_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights,
+                        void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!logits || !ids || !weights) return fail(MAYA_E_ARG, "route_topk: null pointer");
+    if (n_tokens <= 0 || n_tokens > 65535 || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k <= 0 || k > MAYA_MAX_K || k > n_expert)
+        return fail(MAYA_E_SHAPE, "route_topk: tokens %d experts %d k %d (limits %d experts, k %d)", n_tokens, n_expert, k,
+                    MAYA_MAX_EXPERTS, MAYA_MAX_K);
+    hipLaunchKernelGGL(router_kernel, dim3((unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, ids, weights);
+    MAYA_LAUNCHED("router_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,
+                  void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!ids || !expert_table || !plan_ptr) return fail(MAYA_E_ARG, "plan: null pointer");
+    if (n_entries <= 0 || n_expert <= 0) return fail(MAYA_E_SHAPE, "plan: entries %d experts %d", n_entries, n_expert);
+    hipLaunchKernelGGL(plan_kernel, dim3((unsigned) ((n_entries + 255) / 256)), dim3(256), 0, as_stream(stream), ids, n_entries,
+                       expert_table, n_expert, plan_ptr);
+    MAYA_LAUNCHED("plan_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, int32_t* grp_start, int32_t* grp_ent,
+                   int32_t* n_groups, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!plan_ptr || !grp_ptr || !grp_start || !grp_ent || !n_groups) return fail(MAYA_E_ARG, "group: null pointer");
+    if (n_entries <= 0 || n_entries > 256) return fail(MAYA_E_SHAPE, "group: %d entries outside 1..256", n_entries);
+    hipLaunchKernelGGL(group_kernel, dim3(1), dim3(256), 0, as_stream(stream), plan_ptr, n_entries, grp_ptr, grp_start, grp_ent, n_groups);
+    MAYA_LAUNCHED("group_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (const int rc = check_args(a)) return rc;
+    if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
+    hipStream_t s = as_stream(stream);
+    const int tg = a->layout.gate_type, tu = a->layout.up_type;
+#define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
+    MAYA_GU(kIQ2_S, kIQ2_S)
+    MAYA_GU(kQ4_K, kQ4_K)
+    MAYA_GU(kQ8_0, kQ8_0)
+    MAYA_GU(kIQ1_S, kIQ1_S)
+    MAYA_GU(kIQ1_M, kIQ1_M)
+    MAYA_GU(kIQ2_S, kIQ1_M)
+    MAYA_GU(kIQ1_M, kIQ2_S)
+    MAYA_GU(kIQ2_S, kQ4_K)
+    MAYA_GU(kIQ1_S, kIQ1_M)
+    MAYA_GU(kIQ1_M, kIQ1_S)
+#undef MAYA_GU
+    return fail(MAYA_E_UNSUPPORTED, "gate_up: no kernel for gate type %d with up type %d", tg, tu);
+}
+
+int maya_moe_down(const maya_moe_args* a, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (const int rc = check_args(a)) return rc;
+    if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
+    hipStream_t s = as_stream(stream);
+    int rc;
+    switch (a->layout.down_type) {
+        case kIQ2_S: rc = launch_down_t<kIQ2_S>(*a, *st, s); break;
+        case kQ4_K: rc = launch_down_t<kQ4_K>(*a, *st, s); break;
+        case kQ8_0: rc = launch_down_t<kQ8_0>(*a, *st, s); break;
+        case kIQ1_S: rc = launch_down_t<kIQ1_S>(*a, *st, s); break;
+        default: rc = launch_down_t<kIQ1_M>(*a, *st, s); break;
+    }
+    if (rc) return rc;
+    const dim3 grid((unsigned) ((a->layout.n_embd + 255) / 256), (unsigned) a->n_tokens);
+    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, s, *a);
+    MAYA_LAUNCHED("combine_kernel");
+    return MAYA_OK;
+}
+
+// workspace carve-up of maya_moe_layer_decode (every region 256-byte aligned)
+struct LayerWs {
+    uint64_t *plan_ptr, *grp_ptr;
+    int32_t *grp_start, *grp_ent, *n_groups;
+    maya_act x, hq;
+    float *h, *part;
+    size_t bytes;
+};
+static LayerWs carve(const maya_moe_layout& l, int n_tokens, int k, uint8_t* base) {
+    LayerWs w{};
+    size_t off = 0;
+    const int ne = n_tokens * k;
+    auto take = [&](size_t n) {
+        uint8_t* p = base ? base + off : nullptr;
+        off += (n + 255) & ~(size_t) 255;
+        return p;
+    };
+    w.plan_ptr = (uint64_t*) take(sizeof(uint64_t) * ne);
+    w.grp_ptr = (uint64_t*) take(sizeof(uint64_t) * ne);
+    w.grp_start = (int32_t*) take(sizeof(int32_t) * (ne + 1));
+    w.grp_ent = (int32_t*) take(sizeof(int32_t) * ne);
+    w.n_groups = (int32_t*) take(sizeof(int32_t));
+    w.x.q = (int8_t*) take((size_t) n_tokens * l.n_embd);
+    w.x.d = (float*) take(sizeof(float) * (size_t) n_tokens * (l.n_embd / 32));
+    w.x.bsums = (int16_t*) take(sizeof(int16_t) * (size_t) n_tokens * (l.n_embd / 16));
+    w.hq.q = (int8_t*) take((size_t) ne * l.n_ff);
+    w.hq.d = (float*) take(sizeof(float) * (size_t) ne * (l.n_ff / 32));
+    w.hq.bsums = (int16_t*) take(sizeof(int16_t) * (size_t) ne * (l.n_ff / 16));
+    w.h = (float*) take(sizeof(float) * (size_t) ne * l.n_ff);
+    w.part = (float*) take(sizeof(float) * (size_t) ne * l.n_embd);
+    w.bytes = off;
+    return w;
+}
+
+size_t maya_moe_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k) {
+    if (!l || check_layout(*l) != MAYA_OK || n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K) return 0;
+    return carve(*l, n_tokens, k, nullptr).bytes;
+}
+
+int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
+                          const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
+                          float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l) return fail(MAYA_E_ARG, "layer_decode: null layout");
+    if (const int rc = check_layout(*l)) return rc;
+    if (!expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "layer_decode: null pointer");
+    if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K)
+        return fail(MAYA_E_SHAPE, "layer_decode: n_tokens %d / k %d", n_tokens, k);
+    if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "layer_decode: workspace not 256-byte aligned");
+    const LayerWs w = carve(*l, n_tokens, k, (uint8_t*) workspace);
+    if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "layer_decode: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
+    int rc;
+    if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+    if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+    maya_moe_args a{};
+    a.layout = *l;
+    a.n_tokens = n_tokens;
+    a.k = k;
+    a.plan_ptr = w.plan_ptr;
+    a.plan_w = weights;
+    if (n_tokens > 1) {
+        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
+        a.grp_ptr = w.grp_ptr;
+        a.grp_start = w.grp_start;
+        a.grp_ent = w.grp_ent;
+        a.n_groups = w.n_groups;
+    }
+    a.limit = limit;
+    a.x = w.x;
+    a.h = w.h;
+    a.hq = w.hq;
+    a.part = w.part;
+    a.add = add;
+    a.out = out;
+    if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
+    if ((rc = maya_moe_gate_up(&a, stream))) return rc;
+    if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
+    return maya_moe_down(&a, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,218 @@
+"""ctypes bindings of libmaya_moe.so: one Python function per C entry point of include/maya_moe.h, taking torch tensors
+for device memory.  A non-zero status raises MayaError with the library's message."""
+import ctypes as C
+import os
+
+import torch
+
+PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(PKG, "libmaya_moe.so")
+
+Q8_0, Q4_K, IQ1_S, IQ2_S, IQ1_M = 8, 12, 19, 22, 29
+DT_F32, DT_BF16, DT_F16 = 0, 1, 2
+MAX_TOKENS, MAX_K = 16, 16
+
+EXPORTS = [
+    "maya_last_error", "maya_device_info", "maya_init", "maya_moe_supported", "maya_moe_block_bytes",
+    "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
+    "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
+    "maya_moe_workspace_bytes", "maya_moe_layer_decode",
+]
+
+
+class MayaError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("maya_moe status %d: %s" % (code, msg))
+        self.code = code
+
+
+class Layout(C.Structure):
+    _fields_ = [("gate_type", C.c_int32), ("up_type", C.c_int32), ("down_type", C.c_int32), ("n_embd", C.c_int32),
+                ("n_ff", C.c_int32), ("gate_off", C.c_uint64), ("up_off", C.c_uint64), ("down_off", C.c_uint64)]
+
+
+class Act(C.Structure):
+    _fields_ = [("q", C.c_void_p), ("d", C.c_void_p), ("bsums", C.c_void_p)]
+
+
+class Args(C.Structure):
+    _fields_ = [("layout", Layout), ("n_tokens", C.c_int32), ("k", C.c_int32), ("plan_ptr", C.c_void_p),
+                ("plan_w", C.c_void_p), ("grp_ptr", C.c_void_p), ("grp_start", C.c_void_p), ("grp_ent", C.c_void_p),
+                ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", Act), ("h", C.c_void_p),
+                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p)]
+
+
+_lib = None
+
+
+def load():
+    """The loaded library; raises when it was not built (python -m maya_amd.build, or __graft_entry__.build())."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError("%s is missing: the HIP library was not built; there is no CPU fallback" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, sz, f32 = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+    L.maya_last_error.restype = C.c_char_p
+    L.maya_device_info.restype = C.c_char_p
+    L.maya_moe_row_bytes.restype = sz
+    L.maya_moe_row_bytes.argtypes = [i32, i64]
+    L.maya_moe_layout_init.restype = sz
+    L.maya_moe_layout_init.argtypes = [C.POINTER(Layout), i32, i32, i32, i32, i32]
+    L.maya_dequant_rows.argtypes = [i32, vp, sz, i64, i64, vp, vp]
+    L.maya_quant_act.argtypes = [i32, vp, i32, i64, i32, i64, Act, vp]
+    L.maya_quant_i8x32.argtypes = [vp, i32, i64, vp, i32, i64, vp, vp, vp]
+    L.maya_moe_route_topk.argtypes = [vp, i32, i32, i32, vp, vp, vp]
+    L.maya_moe_plan.argtypes = [vp, i32, vp, i32, vp, vp]
+    L.maya_moe_group.argtypes = [vp, i32, vp, vp, vp, vp, vp]
+    L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
+    L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
+    L.maya_moe_workspace_bytes.restype = sz
+    L.maya_moe_workspace_bytes.argtypes = [C.POINTER(Layout), i32, i32]
+    L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != 0:
+        raise MayaError(rc, load().maya_last_error().decode("utf-8", "replace"))
+
+
+def _p(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(stream=None):
+    s = torch.cuda.current_stream() if stream is None else stream
+    return C.c_void_p(s.cuda_stream)
+
+
+def dtype_id(t):
+    return {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}[t.dtype]
+
+
+def layout(gate_type, down_type, n_embd, n_ff, up_type=None):
+    """(Layout, blob bytes) of a contiguous [gate | up | down] expert blob."""
+    l = Layout()
+    n = load().maya_moe_layout_init(C.byref(l), gate_type, gate_type if up_type is None else up_type, down_type, n_embd, n_ff)
+    if n == 0:
+        raise MayaError(1, load().maya_last_error().decode())
+    return l, int(n)
+
+
+def row_bytes(t, k):
+    return int(load().maya_moe_row_bytes(t, k))
+
+
+class ActBuf:
+    """A quantized activation batch on the device (maya_act): codes, per-32 scales, per-16 sums."""
+
+    def __init__(self, rows, k, device="cuda"):
+        self.rows, self.k = rows, k
+        self.q = torch.empty((rows, k), dtype=torch.int8, device=device)
+        self.d = torch.empty((rows, k // 32), dtype=torch.float32, device=device)
+        self.bsums = torch.empty((rows, k // 16), dtype=torch.int16, device=device)
+
+    def c(self):
+        return Act(self.q.data_ptr(), self.d.data_ptr(), self.bsums.data_ptr())
+
+
+def dequant_rows(t, w, k, n_rows, stream=None):
+    out = torch.empty((n_rows, k), dtype=torch.float32, device=w.device)
+    check(load().maya_dequant_rows(t, _p(w), 0, k, n_rows, _p(out), _stream(stream)))
+    return out
+
+
+def quant_act(act_type, x, stream=None):
+    """x [rows, k] (f32 / bf16 / f16, contiguous) -> ActBuf in the activation format of weight type act_type."""
+    assert x.is_contiguous() and x.dim() == 2
+    out = ActBuf(x.shape[0], x.shape[1], x.device)
+    check(load().maya_quant_act(act_type, _p(x), dtype_id(x), 0, x.shape[0], x.shape[1], out.c(), _stream(stream)))
+    return out
+
+
+def quant_i8x32(x, row_idx=None, rows=None, stream=None):
+    assert x.is_contiguous() and x.dim() == 2
+    rows = x.shape[0] if rows is None else rows
+    q = torch.empty((rows, x.shape[1]), dtype=torch.int8, device=x.device)
+    d = torch.empty((rows, x.shape[1] // 32), dtype=torch.float32, device=x.device)
+    check(load().maya_quant_i8x32(_p(x), dtype_id(x), 0, _p(row_idx), rows, x.shape[1], _p(q), _p(d), _stream(stream)))
+    return q, d
+
+
+def route_topk(logits, k, stream=None):
+    assert logits.is_contiguous() and logits.dtype == torch.float32 and logits.dim() == 2
+    nt, ne = logits.shape
+    ids = torch.empty((nt, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((nt, k), dtype=torch.float32, device=logits.device)
+    check(load().maya_moe_route_topk(_p(logits), nt, ne, k, _p(ids), _p(w), _stream(stream)))
+    return ids, w
+
+
+def plan(ids, expert_table, stream=None):
+    out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
+    check(load().maya_moe_plan(_p(ids), ids.numel(), _p(expert_table), expert_table.numel(), _p(out), _stream(stream)))
+    return out
+
+
+def group(plan_ptr, stream=None):
+    n = plan_ptr.numel()
+    dev = plan_ptr.device
+    grp_ptr = torch.zeros(n, dtype=torch.int64, device=dev)
+    grp_start = torch.zeros(n + 1, dtype=torch.int32, device=dev)
+    grp_ent = torch.zeros(n, dtype=torch.int32, device=dev)
+    n_groups = torch.zeros(1, dtype=torch.int32, device=dev)
+    check(load().maya_moe_group(_p(plan_ptr), n, _p(grp_ptr), _p(grp_start), _p(grp_ent), _p(n_groups), _stream(stream)))
+    return grp_ptr, grp_start, grp_ent, n_groups
+
+
+class ExpertStore:
+    """Expert blobs resident in HBM: one contiguous allocation, expert e's [gate | up | down] blob at `offset[e]` (the
+    reference keeps VRAM-resident experts in slots of one pool the same way).  `table` is the device array of blob
+    addresses the plan kernel reads (0: not resident)."""
+
+    def __init__(self, blobs, device="cuda", misalign=0):
+        import numpy as np
+        self.n = len(blobs)
+        sizes = [int(b.size) for b in blobs]
+        stride = (max(sizes) + misalign + 255) & ~255
+        self.pool = torch.empty(stride * self.n + 256, dtype=torch.uint8, device=device)
+        base = self.pool.data_ptr()
+        pad = (-base) % 256
+        addrs = []
+        for e, b in enumerate(blobs):
+            off = pad + e * stride + misalign
+            self.pool[off:off + sizes[e]].copy_(torch.from_numpy(np.ascontiguousarray(b)), non_blocking=False)
+            addrs.append(base + off)
+        self.addrs = addrs
+        self.table = torch.tensor(addrs, dtype=torch.int64, device=device)
+        self.bytes = sum(sizes)
+
+
+class MoeLayer:
+    """One routed layer on the device: route -> plan -> group -> quantize -> gate/up -> quantize -> down -> combine
+    (maya_moe_layer_decode).  Buffers are allocated once here; a call allocates nothing."""
+
+    def __init__(self, gate_type, down_type, n_embd, n_ff, n_expert, k, max_tokens=1, up_type=None, device="cuda"):
+        self.layout, self.blob_bytes = layout(gate_type, down_type, n_embd, n_ff, up_type)
+        self.n_embd, self.n_ff, self.n_expert, self.k, self.max_tokens = n_embd, n_ff, n_expert, k, max_tokens
+        n = int(load().maya_moe_workspace_bytes(C.byref(self.layout), max_tokens, k))
+        if n == 0:
+            raise MayaError(2, load().maya_last_error().decode())
+        self.ws_bytes = n
+        self._ws = torch.empty(n + 256, dtype=torch.uint8, device=device)
+        pad = (-self._ws.data_ptr()) % 256
+        self.ws = self._ws[pad:pad + n]
+        self.ids = torch.empty((max_tokens, k), dtype=torch.int32, device=device)
+        self.weights = torch.empty((max_tokens, k), dtype=torch.float32, device=device)
+        self.out = torch.empty((max_tokens, n_embd), dtype=torch.float32, device=device)
+
+    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None):
+        nt = x.shape[0]
+        assert nt <= self.max_tokens and x.is_contiguous() and logits.is_contiguous()
+        check(load().maya_moe_layer_decode(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, _p(logits), _p(x),
+                                           dtype_id(x), nt, limit, _p(add), _p(self.ids), _p(self.weights), _p(self.out),
+                                           _p(self.ws), self.ws_bytes, _stream(stream)))
+        return self.out[:nt]

@@ -1,0 +1,141 @@
+"""GPU parity, expert rows: the HIP layer against the CPU checker (the reference's CPU expert path in the ggml
+contract) on the same seeded inputs.  Bar: top-k ids bit-exact, expert outputs within 1e-3 relative L2."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, make_experts, oracle_layer, rel_l2
+from maya_amd import synth
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from maya_amd import lib as L
+    L.load()
+    return L
+
+
+def run_layer(lib, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x, limit=float("inf"), up_type=None,
+              misalign=0, add=None, resident=None):
+    store = lib.ExpertStore(blobs, misalign=misalign)
+    table = store.table
+    if resident is not None:
+        table = table.clone()
+        mask = torch.ones(len(blobs), dtype=torch.bool)
+        mask[list(resident)] = False
+        table[mask.cuda()] = 0
+    layer = lib.MoeLayer(gate_type, down_type, n_embd, n_ff, len(blobs), k, max_tokens=x.shape[0], up_type=up_type)
+    out = layer.forward(table, dev(logits), x if torch.is_tensor(x) else dev(x), limit=limit,
+                        add=None if add is None else dev(add))
+    torch.cuda.synchronize()
+    return layer.ids.cpu().numpy(), layer.weights.cpu().numpy(), out.cpu().numpy(), store
+
+
+CASES = [
+    # gate/up type, down type, n_embd, n_ff, experts, k, tokens
+    (22, 22, 1024, 512, 16, 4, 1),
+    (12, 12, 1024, 512, 16, 4, 1),
+    (8, 8, 512, 256, 8, 2, 1),
+    (19, 19, 1024, 512, 8, 4, 1),
+    (29, 29, 1024, 512, 8, 4, 1),
+    (22, 12, 1024, 512, 16, 8, 1),
+    (22, 22, 1024, 512, 16, 8, 4),
+    (22, 12, 1024, 768, 12, 8, 8),
+    (12, 12, 768, 512, 6, 4, 3),
+    (29, 22, 512, 512, 6, 4, 5),
+]
+
+
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", CASES)
+def test_layer_matches_cpu_path(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt):
+    seed = gt * 1000 + dt * 10 + nt
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, seed)
+    rng = np.random.default_rng(seed + 1)
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    print("case", gt, dt, n_embd, n_ff, ne, k, nt, flush=True)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x)
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x)
+    assert np.array_equal(ids, wi)
+    for t in range(nt):
+        assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
+
+
+def test_mixed_gate_up_types(lib, oracle):
+    gt, ut, dt, n_embd, n_ff, ne, k = 22, 29, 22, 512, 256, 6, 3
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 77, up_type=ut)
+    rng = np.random.default_rng(78)
+    logits = rng.standard_normal((2, ne)).astype(np.float32)
+    x = rng.standard_normal((2, n_embd)).astype(np.float32)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, up_type=ut)
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x, up_type=ut)
+    assert np.array_equal(ids, wi)
+    assert rel_l2(out, wout) <= TOL
+
+
+def test_two_byte_aligned_blobs_clamp_and_add(lib, oracle):
+    """Blobs at a +2 byte offset (GGUF slices are only 2-byte aligned), GLM's clamped SwiGLU, a shared-expert part added."""
+    gt, dt, n_embd, n_ff, ne, k, nt = 22, 12, 1024, 512, 8, 4, 2
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 91)
+    rng = np.random.default_rng(92)
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    x = (rng.standard_normal((nt, n_embd)) * 3).astype(np.float32)
+    add = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, limit=0.75, misalign=2, add=add)
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x, limit=0.75)
+    assert np.array_equal(ids, wi)
+    assert rel_l2(out, wout + add) <= TOL
+
+
+def test_null_plan_slots_are_left_out(lib, oracle):
+    gt, dt, n_embd, n_ff, ne, k, nt = 22, 22, 512, 256, 8, 4, 3
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 55)
+    rng = np.random.default_rng(56)
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    resident = {0, 2, 3, 5, 6}
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, resident=resident)
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x, skip=set(range(ne)) - resident)
+    assert np.array_equal(ids, wi)
+    assert rel_l2(out, wout) <= TOL
+
+
+def test_zero_input_and_bf16_input(lib, oracle):
+    gt, dt, n_embd, n_ff, ne, k = 22, 22, 512, 256, 4, 2
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 60)
+    rng = np.random.default_rng(61)
+    logits = rng.standard_normal((1, ne)).astype(np.float32)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, np.zeros((1, n_embd), dtype=np.float32))
+    assert not out.any()
+    xb = torch.from_numpy(rng.standard_normal((1, n_embd)).astype(np.float32)).to(torch.bfloat16)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, xb.cuda())
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, xb.to(torch.float32).numpy())
+    assert np.array_equal(ids, wi) and rel_l2(out, wout) <= TOL
+
+
+def test_window_rows_equal_token_rows(lib):
+    """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract)."""
+    gt, dt, n_embd, n_ff, ne, k, nt = 22, 12, 1024, 512, 10, 4, 6
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 33)
+    rng = np.random.default_rng(34)
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    _, _, win, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x)
+    for t in range(nt):
+        _, _, one, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits[t:t + 1], x[t:t + 1])
+        assert np.array_equal(win[t].view(np.uint32), one[0].view(np.uint32)), t
+
+
+def test_unsupported_and_bad_shapes_fail_cleanly(lib):
+    import ctypes as C
+    L = lib.load()
+    l = lib.Layout()
+    assert L.maya_moe_layout_init(C.byref(l), 22, 22, 22, 1000, 512) == 0      # not whole blocks
+    assert L.maya_moe_layout_init(C.byref(l), 22, 8, 22, 1024, 512) == 0        # gate/up activation formats differ
+    assert L.maya_moe_layout_init(C.byref(l), 99, 99, 99, 1024, 512) == 0
+    assert L.maya_moe_supported(22) == 1 and L.maya_moe_supported(10) == 0
+    with pytest.raises(lib.MayaError):
+        lib.route_topk(torch.zeros((1, 4), device="cuda"), 8)

@@ -1,0 +1,103 @@
+"""GPU parity, format layer: dequantized weights and quantized activations are bit-exact with the CPU checker."""
+import numpy as np
+import pytest
+import torch
+
+from maya_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+TYPES = (8, 12, 19, 22, 29)
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from maya_amd import lib as L
+    L.load()
+    L.check(L.load().maya_init())
+    print("device:", L.load().maya_device_info().decode(), flush=True)
+    return L
+
+
+@pytest.mark.parametrize("t", TYPES)
+@pytest.mark.parametrize("misalign", (0, 2))
+def test_dequant_bit_exact(lib, oracle, t, misalign):
+    rng = np.random.default_rng(40 + t)
+    n, k = 12, 1024
+    w = synth.constructed_rows(t, n, k, rng)
+    want = oracle.dequant_rows(t, w, k, n)
+    buf = torch.zeros(w.size + 16, dtype=torch.uint8, device="cuda")
+    buf[misalign:misalign + w.size] = torch.from_numpy(w).cuda()
+    got = lib.dequant_rows(t, buf[misalign:], k, n).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_subnormal_scales(lib, oracle):
+    """FP16 block scales in the subnormal range and at the extremes decode to the same bits."""
+    rng = np.random.default_rng(3)
+    for t in (12, 22, 8, 19):
+        w = synth.constructed_rows(t, 2, 512, rng).reshape(-1, synth.BLOCK_BYTES[t])
+        specials = np.array([0x0001, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0x0000, 0x83FF, 0x3C00], dtype=np.uint16)
+        for b in range(w.shape[0]):
+            w[b, 0:2] = specials[b % 8: b % 8 + 1].view(np.uint8)
+        w = w.reshape(-1)
+        want = oracle.dequant_rows(t, w, 512, 2)
+        got = lib.dequant_rows(t, torch.from_numpy(w).cuda(), 512, 2).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), t
+
+
+def _x_cases(k, rng):
+    x = rng.standard_normal((6, k)).astype(np.float32)
+    x[1] *= 1e-3
+    x[2, 256:512] = 0.0
+    x[3, :256] = 0.5
+    x[3, 300] = -7.0
+    x[3, 301] = 7.0                      # equal magnitudes: the first one is the block's maximum
+    x[4] = np.round(x[4] * 4) / 4        # many exact .5 products
+    x[5, 512:768] = (np.arange(256) - 128).astype(np.float32) / 254.0 * 3.0
+    return x
+
+
+@pytest.mark.parametrize("dt", ("f32", "bf16", "f16"))
+def test_q8k_quant_byte_exact(lib, oracle, dt):
+    rng = np.random.default_rng(17)
+    k = 1024
+    x = _x_cases(k, rng)
+    xt = torch.from_numpy(x)
+    if dt == "bf16":
+        xt = xt.to(torch.bfloat16)
+    elif dt == "f16":
+        xt = xt.to(torch.float16)
+    xr = xt.to(torch.float32).numpy()
+    act = lib.quant_act(22, xt.cuda().contiguous())
+    q, d, bs = act.q.cpu().numpy(), act.d.cpu().numpy(), act.bsums.cpu().numpy()
+    for r in range(x.shape[0]):
+        wd, wq, wbs = oracle.q8k_fields(oracle.quant_q8k(xr[r]))
+        assert np.array_equal(q[r], wq), (dt, r)
+        assert np.array_equal(d[r].reshape(-1, 8).view(np.uint32), np.repeat(wd.view(np.uint32)[:, None], 8, 1)), (dt, r)
+        assert np.array_equal(bs[r].reshape(-1, 16), wbs), (dt, r)
+
+
+def test_q80_quant_byte_exact(lib, oracle):
+    rng = np.random.default_rng(18)
+    k = 512
+    x = _x_cases(1024, rng)[:, :k].copy()
+    act = lib.quant_act(8, torch.from_numpy(x).cuda())
+    q, d = act.q.cpu().numpy(), act.d.cpu().numpy()
+    for r in range(x.shape[0]):
+        blocks = oracle.quant_act(8, x[r]).reshape(-1, 34)
+        wq = blocks[:, 2:].copy().view(np.int8).reshape(-1)
+        wd = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+        assert np.array_equal(q[r], wq), r
+        assert np.array_equal(d[r].view(np.uint32), wd.view(np.uint32)), r
+
+
+def test_i8x32_quant_byte_exact(lib, oracle):
+    rng = np.random.default_rng(19)
+    x = _x_cases(1024, rng)
+    idx = np.array([5, 0, 3, 3, 1], dtype=np.int32)
+    q, d = lib.quant_i8x32(torch.from_numpy(x).cuda(), torch.from_numpy(idx).cuda(), rows=len(idx))
+    q, d = q.cpu().numpy(), d.cpu().numpy()
+    for r, src in enumerate(idx):
+        wq, wd = oracle.quant_i8x32(x[src])
+        assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))

@@ -1,0 +1,94 @@
+"""GPU parity, routing: top-k ids bit-exact with the CPU checker on random, tied and degenerate logits; grouping."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from maya_amd import lib as L
+    L.load()
+    return L
+
+
+def _check(lib, oracle, logits, k):
+    ids, w = lib.route_topk(torch.from_numpy(logits).cuda(), k)
+    wi, ww = oracle.router_topk(logits, k)
+    assert np.array_equal(ids.cpu().numpy(), wi)
+    got = w.cpu().numpy()
+    assert np.max(np.abs(got - ww) / np.maximum(ww, 1e-30)) <= 1e-5   # the reference's weight tolerance
+    return got
+
+
+@pytest.mark.parametrize("ne,k", ((256, 8), (160, 8), (512, 10), (8, 8), (1000, 16)))
+def test_random_normal(lib, oracle, ne, k):
+    rng = np.random.default_rng(ne + k)
+    _check(lib, oracle, rng.standard_normal((64, ne)).astype(np.float32), k)
+
+
+def test_all_equal_is_pure_tie_rule(lib, oracle):
+    logits = np.full((3, 256), 0.37, dtype=np.float32)
+    w = _check(lib, oracle, logits, 8)
+    ids, _ = lib.route_topk(torch.from_numpy(logits).cuda(), 8)
+    assert np.array_equal(ids.cpu().numpy(), np.tile(np.arange(8, dtype=np.int32), (3, 1)))
+    assert np.allclose(w, 1.0 / 8, rtol=1e-6)
+
+
+def test_twelve_way_tie_and_dominant(lib, oracle):
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal((4, 256)).astype(np.float32)
+    tie = rng.choice(256, 12, replace=False)
+    logits[0, tie] = 4.0
+    logits[1, 77] = 60.0                 # one dominant expert: the others' p underflow towards 0
+    logits[2] = np.round(logits[2] * 2) / 2   # many equal logits
+    logits[3, :] = -1e30
+    logits[3, 5] = 0.0
+    _check(lib, oracle, logits, 8)
+
+
+def test_zipf_biased(lib, oracle):
+    from maya_amd import synth
+    rng = np.random.default_rng(6)
+    logits = (rng.standard_normal((512, 256)) + synth.zipf_bias(256)[None, :]).astype(np.float32)
+    _check(lib, oracle, logits, 8)
+
+
+def test_float_and_double_selection_agree(oracle):
+    # the kernel selects on float p, the reference's host test on double p: no disagreement on N(0,1) logits
+    rng = np.random.default_rng(8)
+    logits = rng.standard_normal((2000, 256)).astype(np.float32)
+    a, _ = oracle.router_topk(logits, 8)
+    b, _ = oracle.router_topk(logits, 8, f64=True)
+    assert np.array_equal(a, b)
+
+
+def test_plan_and_group(lib):
+    rng = np.random.default_rng(9)
+    for trial in range(20):
+        nt, k, ne = int(rng.integers(1, 17)), 8, 24
+        ids = np.stack([rng.choice(ne, k, replace=False) for _ in range(nt)]).astype(np.int32)
+        table = (np.arange(ne, dtype=np.int64) + 1) * 4096
+        table[rng.choice(ne, 3, replace=False)] = 0          # not resident
+        plan = lib.plan(torch.from_numpy(ids).cuda(), torch.from_numpy(table).cuda())
+        p = plan.cpu().numpy()
+        assert np.array_equal(p, table[ids.reshape(-1)])
+        gp, gs, ge, ng = [t.cpu().numpy() for t in lib.group(plan)]
+        # host restatement: distinct non-null blobs in first-appearance order, entries ascending
+        order, members = [], {}
+        for e, b in enumerate(p):
+            if b == 0:
+                continue
+            if b not in members:
+                members[b] = []
+                order.append(b)
+            members[b].append(e)
+        assert ng[0] == len(order)
+        assert np.array_equal(gp[:len(order)], np.array(order, dtype=np.int64))
+        start = 0
+        for g, b in enumerate(order):
+            assert gs[g] == start
+            assert list(ge[start:start + len(members[b])]) == members[b]
+            start += len(members[b])
+        assert gs[len(order)] == start
