@@ -57,7 +57,16 @@ typedef struct maya_moe_layout {
     int32_t gate_type, up_type, down_type; /* ggml ids; gate and up must share the activation format */
     int32_t n_embd, n_ff;                  /* multiples of 256 */
     uint64_t gate_off, up_off, down_off;   /* byte offsets of the three row arrays inside an expert blob */
+    int32_t packing;                       /* MAYA_PACK_GGUF or MAYA_PACK_STREAM (maya_moe_repack) */
+    int32_t reserved;
 } maya_moe_layout;
+
+/* Row packings.  GGUF: the file's own block sequence.  STREAM: the same bytes of every row regrouped by field so that a
+ * wavefront's loads are aligned and contiguous (IQ2_S rows: all (index word, sign word) pairs, then all (high-bit, scale)
+ * byte pairs, then the block scales; other types are left as they are).  A row keeps its size and its position in the
+ * blob, every field keeps its bits, so dequantized values are unchanged. */
+#define MAYA_PACK_GGUF 0
+#define MAYA_PACK_STREAM 1
 
 /* A quantized activation batch in device memory (rows x k): int8 codes, an F32 scale per 32 values (a 256-value
  * Q8_K block's scale is written 8 times, as ds4's xd / hd hold it: src/ds4/ds4_lane_parity.hpp:40-42) and ggml's
@@ -100,6 +109,13 @@ size_t maya_moe_row_bytes(int ggml_type, int64_t k);
  * (src/kernels/cpu/native_expert.cpp:195-260); returns the blob's bytes (0: unsupported) */
 size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int down_type, int n_embd, int n_ff);
 
+/* One-time regrouping of an expert blob for the streaming kernels, at upload: dst (same size as src, 16-byte aligned)
+ * receives src's rows in MAYA_PACK_STREAM order; maya_moe_unpack is the inverse.  `l` describes the GGUF blob; use a copy
+ * of it with packing = MAYA_PACK_STREAM for calls on dst.  The reference uploads resident experts into VRAM slots of a pool
+ * (include/strata/kernels/glm_fast.hpp:284-300); this is the hook that runs on that copy.  src and dst must not overlap. */
+int maya_moe_repack(const maya_moe_layout* l, const void* src, void* dst, void* stream);
+int maya_moe_unpack(const maya_moe_layout* l, const void* src, void* dst, void* stream);
+
 const char* maya_last_error(void);
 /* Device and library identification: "gfx950 ..." (host string, valid until the next call on this thread). */
 const char* maya_device_info(void);
@@ -112,6 +128,9 @@ int maya_init(void);
  * (src/ds4/ds4_iq.cuh:171-175).  w: n_rows rows of k values, row_stride bytes apart (0: the type's own row size). */
 int maya_dequant_rows(int ggml_type, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out,
                       void* stream);
+/* the same for rows in MAYA_PACK_STREAM order */
+int maya_dequant_rows_packed(int ggml_type, int packing, const void* w, size_t row_stride, int64_t k, int64_t n_rows,
+                             float* out, void* stream);
 
 /* ---- activation quantizers.  act_type = the WEIGHT type whose dot will consume the activation:
  * Q8_K rounding for the 256-value types - quantize_q8_K (src/kernels/cuda/quantize_act.cu:161-207), q8k_quant_kernel

@@ -11,6 +11,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
 #include <stdint.h>
 
 namespace maya {
@@ -74,9 +75,8 @@ template <> struct Fmt<kIQ2_S> {
     static constexpr bool kMin = false;
     __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
     // third_party/ggml/ggml-common.h:396-402; decode: src/kernels/cuda/iq_kernels.cu:686-695
-    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
-        const uint32_t i4 = ld32_a2(blk + 2 + 4 * ib), sg4 = ld32_a2(blk + 34 + 4 * ib);
-        const uint32_t h = blk[66 + ib], sc = blk[74 + ib];
+    __device__ static __forceinline__ void decode_fields(uint32_t i4, uint32_t sg4, uint32_t h, uint32_t sc,
+                                                         const uint2* grid, Unit32& u) {
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
             const uint32_t idx = ((i4 >> (8 * l)) & 255u) | ((h << (8 - 2 * l)) & 0x300u);
@@ -87,6 +87,17 @@ template <> struct Fmt<kIQ2_S> {
         }
         u.s0 = 2 * (int) (sc & 15u) + 1;
         u.s1 = 2 * (int) (sc >> 4) + 1;
+    }
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
+        decode_fields(ld32_a2(blk + 2 + 4 * ib), ld32_a2(blk + 34 + 4 * ib), blk[66 + ib], blk[74 + ib], grid, u);
+    }
+    // the stream packing of a row of nu sub-blocks: [nu x (index word, sign word)] [nu x (high bits, scales)] [nu/8 x d]
+    __device__ static __forceinline__ void decode_stream(const uint8_t* row, int nu, int un, const uint2* grid, Unit32& u,
+                                                         float& d) {
+        const uint2 is = ((const uint2*) row)[un];
+        const uint32_t hs = ((const uint16_t*) (row + 8 * (size_t) nu))[un];
+        d = f16_bits_to_f32(((const uint16_t*) (row + 10 * (size_t) nu))[un >> 3]) * 0.125f;
+        decode_fields(is.x, is.y, hs & 255u, hs >> 8, grid, u);
     }
 };
 

@@ -12,6 +12,7 @@
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -105,7 +106,7 @@ inline hipStream_t as_stream(void* s) { return (hipStream_t) s; }
 
 template <int TYPE>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, size_t row_stride, int64_t k,
-                                                      float* __restrict__ out, Codebooks cb) {
+                                                      float* __restrict__ out, Codebooks cb, int packing) {
     const int64_t row = blockIdx.y;
     const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;  // value index in the row
     if (v >= k) return;
@@ -125,14 +126,29 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         const int q = (j & 1) ? (qb >> 4) : (qb & 15);
         r = __fsub_rn(__fmul_rn(d1, (float) q), m1);
     } else if constexpr (TYPE == kIQ2_S) {
-        const uint8_t* blk = rp + (size_t) (v >> 8) * 82;
         const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
-        const uint32_t idx = blk[2 + 4 * ib + il] | (((uint32_t) blk[66 + ib] << (8 - 2 * il)) & 0x300u);
+        uint32_t qs, sg, h, sc, dbits;
+        if (packing == MAYA_PACK_STREAM) {
+            const int64_t nu = k >> 5, un = v >> 5;
+            qs = rp[8 * un + il];
+            sg = rp[8 * un + 4 + il];
+            h = rp[8 * nu + 2 * un];
+            sc = rp[8 * nu + 2 * un + 1];
+            dbits = ld16(rp + 10 * nu + 2 * (un >> 3));
+        } else {
+            const uint8_t* blk = rp + (size_t) (v >> 8) * 82;
+            qs = blk[2 + 4 * ib + il];
+            sg = blk[34 + 4 * ib + il];
+            h = blk[66 + ib];
+            sc = blk[74 + ib];
+            dbits = ld16(blk);
+        }
+        const uint32_t idx = qs | ((h << (8 - 2 * il)) & 0x300u);
         const uint64_t g = cb.iq2s[idx];
-        const int ls = (blk[74 + ib] >> (4 * (il >> 1))) & 15;
-        const float dl = __fmul_rn(__fmul_rn(f16_bits_to_f32(ld16(blk)), __fadd_rn(0.5f, (float) ls)), 0.25f);
+        const int ls = (sc >> (4 * (il >> 1))) & 15;
+        const float dl = __fmul_rn(__fmul_rn(f16_bits_to_f32(dbits), __fadd_rn(0.5f, (float) ls)), 0.25f);
         const float mag = __fmul_rn(dl, (float) (uint32_t) ((g >> (8 * j)) & 255u));
-        r = (blk[34 + 4 * ib + il] >> j) & 1 ? -mag : mag;
+        r = (sg >> j) & 1 ? -mag : mag;
     } else if constexpr (TYPE == kIQ1_S) {
         const uint8_t* blk = rp + (size_t) (v >> 8) * 50;
         const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
@@ -154,6 +170,47 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
     }
     out[(size_t) row * k + v] = r;
+}
+
+// ------------------------------------------------------------------------------------------------ stream packing
+
+// IQ2_S rows between the GGUF block sequence and the stream order; one thread a sub-block, grid (k/256 blocks / 32, rows).
+// DIR 0: GGUF -> stream, 1: stream -> GGUF.  Every byte of a row is written exactly once.
+template <int DIR>
+__global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                          int64_t k, int64_t n_rows) {
+    const int64_t nu = k >> 5, rb = (k >> 8) * 82;
+    const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (un >= nu) return;
+    const uint8_t* s = src + row * rb;
+    uint8_t* d = dst + row * rb;
+    const int64_t b = un >> 3;
+    const int ib = (int) (un & 7);
+    const uint8_t* g = (DIR == 0 ? s : d) + b * 82;   // the GGUF side's block (only its address matters for DIR 1)
+    if (DIR == 0) {
+        for (int i = 0; i < 4; ++i) d[8 * un + i] = g[2 + 4 * ib + i];
+        for (int i = 0; i < 4; ++i) d[8 * un + 4 + i] = g[34 + 4 * ib + i];
+        d[8 * nu + 2 * un] = g[66 + ib];
+        d[8 * nu + 2 * un + 1] = g[74 + ib];
+        if (ib == 0) {
+            d[10 * nu + 2 * b] = g[0];
+            d[10 * nu + 2 * b + 1] = g[1];
+        }
+    } else {
+        uint8_t* o = d + b * 82;
+        for (int i = 0; i < 4; ++i) o[2 + 4 * ib + i] = s[8 * un + i];
+        for (int i = 0; i < 4; ++i) o[34 + 4 * ib + i] = s[8 * un + 4 + i];
+        o[66 + ib] = s[8 * nu + 2 * un];
+        o[74 + ib] = s[8 * nu + 2 * un + 1];
+        if (ib == 0) {
+            o[0] = s[10 * nu + 2 * b];
+            o[1] = s[10 * nu + 2 * b + 1];
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n) {
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) gridDim.x * 256) dst[i] = src[i];
 }
 
 // ------------------------------------------------------------------------------------------------ activation quantizers
@@ -423,7 +480,7 @@ struct ActLds {
 // lane's part.  `sub` = lane index inside the group.
 template <int TYPE, int NT, int LPR>
 __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, int sub, const ActLds& a,
-                                        const uint2* __restrict__ grid, float (&acc)[NT]) {
+                                        const uint2* __restrict__ grid, float (&acc)[NT], bool stream_packed) {
     if constexpr (TYPE == kQ4_K) {
         const int np = k >> 6;
         for (int p = sub; p < np; p += LPR) {
@@ -461,8 +518,13 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
                 ib = un & 7;
             }
             Unit32 u;
-            Fmt<TYPE>::decode(blk, ib, grid, u);
-            const float D = Fmt<TYPE>::scale(blk);
+            float D;
+            if (TYPE == kIQ2_S && stream_packed) {
+                if constexpr (TYPE == kIQ2_S) Fmt<kIQ2_S>::decode_stream(row, nu, un, grid, u, D);
+            } else {
+                Fmt<TYPE>::decode(blk, ib, grid, u);
+                D = Fmt<TYPE>::scale(blk);
+            }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const int* y = a.q + t * a.kq + un * 8;
@@ -537,7 +599,7 @@ __device__ __forceinline__ float swiglu(float g, float u, float limit) {
 }
 
 constexpr int kGuThreads = 512, kGuRows = 32;   // a workgroup: 8 waves, 32 gate + 32 up rows
-constexpr int kDnThreads = 512, kDnRows = 64;   // 8 waves x 4 rows a pass, 2 passes
+constexpr int kDnThreads = 512, kDnRows = 64;   // 8 waves x 2 rows a pass, 4 passes
 
 // grid (n_ff / kGuRows, groups): wave w takes row pairs w, w + 8, ...: lanes 0..31 the gate row, 32..63 the up row
 template <int TG, int TU, int NT>
@@ -566,6 +628,7 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
     const size_t grow = (size_t) (k / Fmt<TG>::kValues) * Fmt<TG>::kBytes, urow = (size_t) (k / Fmt<TU>::kValues) * Fmt<TU>::kBytes;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31;
     const bool is_up = lane >= 32;
+    const bool packed = a.layout.packing == MAYA_PACK_STREAM;
     for (int c0 = 0; c0 < gr.ne; c0 += NT) {
         int ents[NT], rows[NT];
 #pragma unroll
@@ -582,10 +645,10 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
             if constexpr (TG == TU) {
                 const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) r * grow;
-                row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc);
+                row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc, packed);
             } else {
-                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) r * grow, k, sub, al, grid_g, acc);
-                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) r * urow, k, sub, al, grid_u, acc);
+                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) r * grow, k, sub, al, grid_g, acc, packed);
+                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) r * urow, k, sub, al, grid_u, acc, packed);
             }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -597,7 +660,8 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
     }
 }
 
-// grid (n_embd / kDnRows, groups): a wave takes 4 rows a pass, 16 lanes a row
+// grid (n_embd / kDnRows, groups): a wave takes 2 rows a pass, 32 lanes a row (the single-token kernel's split of a
+// row over lanes, so a window's rows get the token path's bits)
 template <int TD, int NT>
 __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codebooks cb) {
     extern __shared__ int lds[];
@@ -615,7 +679,8 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
     ActLds al{lds_act, (const float*) (lds_act + NT * kq), lds_act + NT * kq + NT * kd, kq, kd};
     const uint8_t* base = (const uint8_t*) gr.blob + a.layout.down_off;
     const size_t drow = (size_t) (k / Fmt<TD>::kValues) * Fmt<TD>::kBytes;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, rsub = lane >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
+    const bool packed = a.layout.packing == MAYA_PACK_STREAM;
     for (int c0 = 0; c0 < gr.ne; c0 += NT) {
         int ents[NT];
 #pragma unroll
@@ -624,14 +689,14 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
         stage_act<TD, NT>(lds_act, k, a.hq, ents, Fmt<TD>::kMin);
         __syncthreads();
         const int r_end = min(n_embd, (int) (blockIdx.x + 1) * kDnRows);
-        for (int r = blockIdx.x * kDnRows + wave * 4 + rsub; r < r_end; r += (kDnThreads / 64) * 4) {
+        for (int r = blockIdx.x * kDnRows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
-            row_dot<TD, NT, 16>(base + (size_t) r * drow, k, sub, al, grid, acc);
+            row_dot<TD, NT, 32>(base + (size_t) r * drow, k, sub, al, grid, acc, packed);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const float s = group_sum<16>(acc[t]);
+                const float s = group_sum<32>(acc[t]);
                 if (sub == 0 && ents[t] >= 0) a.part[(size_t) ents[t] * n_embd + r] = s;
             }
         }
@@ -656,6 +721,12 @@ __global__ __launch_bounds__(256) void combine_kernel(maya_moe_args a) {
     if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[(size_t) t * n + c]);
     a.out[(size_t) t * n + c] = sum;
 }
+
+}  // namespace maya
+
+#include "maya_fast.cuh"
+
+namespace maya {
 
 // ------------------------------------------------------------------------------------------------ host launchers
 
@@ -683,6 +754,7 @@ int check_layout(const maya_moe_layout& l) {
                     l.up_type);
     if (l.n_embd <= 0 || l.n_ff <= 0 || l.n_embd % 256 || l.n_ff % 256)
         return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d: multiples of 256 wanted", l.n_embd, l.n_ff);
+    if (l.packing != MAYA_PACK_GGUF && l.packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "packing %d", l.packing);
     if (l.n_embd > 16384 || l.n_ff > 16384) return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d past 16384", l.n_embd, l.n_ff);
     return MAYA_OK;
 }
@@ -720,6 +792,52 @@ int launch_down_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) 
     else hipLaunchKernelGGL((down_kernel<TD, 1>), grid, dim3(kDnThreads), lds, s, a, st.cb);
     MAYA_LAUNCHED("down_kernel");
     return MAYA_OK;
+}
+
+bool fast_1tok(const maya_moe_args& a) { return a.n_tokens == 1 && a.grp_ptr == nullptr; }
+
+int tuning_variant(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+template <bool STREAM>
+int launch_gate_up_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    constexpr int kRows = 32;
+    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) a.k);
+    static const int variant = tuning_variant("MAYA_GU_VARIANT", 0);
+#define MAYA_KU(N)                                                                                                                        \
+    case N:                                                                                                                               \
+        if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, true, false, 4, STREAM>), grid, dim3(512), 0, s, a, st.cb);  \
+        else if (variant == 3) hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, false, false, 4, STREAM>), grid, dim3(512), 0, s, a, st.cb); \
+        else hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, true, true, 1, STREAM>), grid, dim3(512), 0, s, a, st.cb);             \
+        break;
+    switch (a.layout.n_embd / 1024) {
+        MAYA_KU(1) MAYA_KU(2) MAYA_KU(3) MAYA_KU(4) MAYA_KU(5) MAYA_KU(6) MAYA_KU(7) MAYA_KU(8)
+    }
+#undef MAYA_KU
+    MAYA_LAUNCHED("gate_up_iq2s_1tok_kernel");
+    return MAYA_OK;
+}
+int launch_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    return a.layout.packing == MAYA_PACK_STREAM ? launch_gate_up_iq2s_1tok_t<true>(a, st, s)
+                                                : launch_gate_up_iq2s_1tok_t<false>(a, st, s);
+}
+template <bool STREAM>
+int launch_down_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    constexpr int kRows = 14;
+    const dim3 grid((unsigned) (a.layout.n_embd / kRows));
+#define MAYA_KU(N) case N: hipLaunchKernelGGL((down_iq2s_1tok_kernel<N, kRows, STREAM>), grid, dim3(512), 0, s, a, st.cb); break;
+    switch (a.layout.n_ff / 1024) {
+        MAYA_KU(1) MAYA_KU(2) MAYA_KU(3) MAYA_KU(4)
+    }
+#undef MAYA_KU
+    MAYA_LAUNCHED("down_iq2s_1tok_kernel");
+    return MAYA_OK;
+}
+int launch_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    return a.layout.packing == MAYA_PACK_STREAM ? launch_down_iq2s_1tok_t<true>(a, st, s)
+                                                : launch_down_iq2s_1tok_t<false>(a, st, s);
 }
 
 }  // namespace maya
@@ -764,16 +882,53 @@ size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int 
     l->n_embd = n_embd;
     l->n_ff = n_ff;
     l->gate_off = l->up_off = l->down_off = 0;
+    l->packing = MAYA_PACK_GGUF;
+    l->reserved = 0;
     if (check_layout(*l) != MAYA_OK) return 0;
     l->up_off = maya_moe_row_bytes(gate_type, n_embd) * (size_t) n_ff;
     l->down_off = l->up_off + maya_moe_row_bytes(up_type, n_embd) * (size_t) n_ff;
     return l->down_off + maya_moe_row_bytes(down_type, n_ff) * (size_t) n_embd;
 }
 
+static int repack_impl(const maya_moe_layout* l, const void* src, void* dst, void* stream, int dir) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l || !src || !dst) return fail(MAYA_E_ARG, "repack: null pointer");
+    if (const int rc = check_layout(*l)) return rc;
+    if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_ARG, "repack: the layout must describe the GGUF blob");
+    hipStream_t s = as_stream(stream);
+    const struct { int type; uint64_t off; int64_t k, rows; } roles[3] = {
+        {l->gate_type, l->gate_off, l->n_embd, l->n_ff},
+        {l->up_type, l->up_off, l->n_embd, l->n_ff},
+        {l->down_type, l->down_off, l->n_ff, l->n_embd}};
+    for (const auto& r : roles) {
+        const uint8_t* sp = (const uint8_t*) src + r.off;
+        uint8_t* dp = (uint8_t*) dst + r.off;
+        if (r.type == kIQ2_S) {
+            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
+            if (dir == 0) hipLaunchKernelGGL(repack_iq2s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+            else hipLaunchKernelGGL(repack_iq2s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+        } else {
+            const size_t n = maya_moe_row_bytes(r.type, r.k) * (size_t) r.rows;
+            hipLaunchKernelGGL(copy_bytes_kernel, dim3(1024), dim3(256), 0, s, sp, dp, n);
+        }
+        MAYA_LAUNCHED("repack kernel");
+    }
+    return MAYA_OK;
+}
+int maya_moe_repack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_impl(l, src, dst, stream, 0); }
+int maya_moe_unpack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_impl(l, src, dst, stream, 1); }
+
 int maya_dequant_rows(int t, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out, void* stream) {
+    return maya_dequant_rows_packed(t, MAYA_PACK_GGUF, w, row_stride, k, n_rows, out, stream);
+}
+
+int maya_dequant_rows_packed(int t, int packing, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out,
+                             void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (!type_ok(t)) return fail(MAYA_E_UNSUPPORTED, "dequant: type %d", t);
+    if (packing != MAYA_PACK_GGUF && packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "dequant: packing %d", packing);
     if (!w || !out) return fail(MAYA_E_ARG, "dequant: null pointer");
     if (k <= 0 || k % block_values(t) || n_rows <= 0 || n_rows > 65535)
         return fail(MAYA_E_SHAPE, "dequant: k %lld rows %lld", (long long) k, (long long) n_rows);
@@ -782,11 +937,11 @@ int maya_dequant_rows(int t, const void* w, size_t row_stride, int64_t k, int64_
     const uint8_t* wb = (const uint8_t*) w;
     hipStream_t s = as_stream(stream);
     switch (t) {
-        case kQ8_0: hipLaunchKernelGGL(dequant_kernel<kQ8_0>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
-        case kQ4_K: hipLaunchKernelGGL(dequant_kernel<kQ4_K>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
-        case kIQ2_S: hipLaunchKernelGGL(dequant_kernel<kIQ2_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
-        case kIQ1_S: hipLaunchKernelGGL(dequant_kernel<kIQ1_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
-        default: hipLaunchKernelGGL(dequant_kernel<kIQ1_M>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb); break;
+        case kQ8_0: hipLaunchKernelGGL(dequant_kernel<kQ8_0>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
+        case kQ4_K: hipLaunchKernelGGL(dequant_kernel<kQ4_K>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
+        case kIQ2_S: hipLaunchKernelGGL(dequant_kernel<kIQ2_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
+        case kIQ1_S: hipLaunchKernelGGL(dequant_kernel<kIQ1_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
+        default: hipLaunchKernelGGL(dequant_kernel<kIQ1_M>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
     }
     MAYA_LAUNCHED("dequant_kernel");
     return MAYA_OK;
@@ -881,6 +1036,9 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
     hipStream_t s = as_stream(stream);
     const int tg = a->layout.gate_type, tu = a->layout.up_type;
+    if (tg == kIQ2_S && tu == kIQ2_S && fast_1tok(*a) && a->layout.n_embd % 1024 == 0 && a->layout.n_embd <= 8192 &&
+        a->layout.n_ff % 32 == 0)
+        return launch_gate_up_iq2s_1tok(*a, *st, s);
 #define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
     MAYA_GU(kIQ2_S, kIQ2_S)
     MAYA_GU(kQ4_K, kQ4_K)
@@ -902,6 +1060,9 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     if (const int rc = check_args(a)) return rc;
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
     hipStream_t s = as_stream(stream);
+    if (a->layout.down_type == kIQ2_S && fast_1tok(*a) && a->k <= 8 && a->layout.n_ff % 1024 == 0 && a->layout.n_ff <= 4096 &&
+        a->layout.n_embd % 14 == 0)
+        return launch_down_iq2s_1tok(*a, *st, s);
     int rc;
     switch (a->layout.down_type) {
         case kIQ2_S: rc = launch_down_t<kIQ2_S>(*a, *st, s); break;

@@ -11,12 +11,14 @@ LIB_PATH = os.path.join(PKG, "libmaya_moe.so")
 Q8_0, Q4_K, IQ1_S, IQ2_S, IQ1_M = 8, 12, 19, 22, 29
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 MAX_TOKENS, MAX_K = 16, 16
+PACK_GGUF, PACK_STREAM = 0, 1
 
 EXPORTS = [
     "maya_last_error", "maya_device_info", "maya_init", "maya_moe_supported", "maya_moe_block_bytes",
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
-    "maya_moe_workspace_bytes", "maya_moe_layer_decode",
+    "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack",
+    "maya_dequant_rows_packed",
 ]
 
 
@@ -28,7 +30,8 @@ class MayaError(RuntimeError):
 
 class Layout(C.Structure):
     _fields_ = [("gate_type", C.c_int32), ("up_type", C.c_int32), ("down_type", C.c_int32), ("n_embd", C.c_int32),
-                ("n_ff", C.c_int32), ("gate_off", C.c_uint64), ("up_off", C.c_uint64), ("down_off", C.c_uint64)]
+                ("n_ff", C.c_int32), ("gate_off", C.c_uint64), ("up_off", C.c_uint64), ("down_off", C.c_uint64),
+                ("packing", C.c_int32), ("reserved", C.c_int32)]
 
 
 class Act(C.Structure):
@@ -61,6 +64,9 @@ def load():
     L.maya_moe_layout_init.restype = sz
     L.maya_moe_layout_init.argtypes = [C.POINTER(Layout), i32, i32, i32, i32, i32]
     L.maya_dequant_rows.argtypes = [i32, vp, sz, i64, i64, vp, vp]
+    L.maya_dequant_rows_packed.argtypes = [i32, i32, vp, sz, i64, i64, vp, vp]
+    L.maya_moe_repack.argtypes = [C.POINTER(Layout), vp, vp, vp]
+    L.maya_moe_unpack.argtypes = [C.POINTER(Layout), vp, vp, vp]
     L.maya_quant_act.argtypes = [i32, vp, i32, i64, i32, i64, Act, vp]
     L.maya_quant_i8x32.argtypes = [vp, i32, i64, vp, i32, i64, vp, vp, vp]
     L.maya_moe_route_topk.argtypes = [vp, i32, i32, i32, vp, vp, vp]
@@ -119,10 +125,27 @@ class ActBuf:
         return Act(self.q.data_ptr(), self.d.data_ptr(), self.bsums.data_ptr())
 
 
-def dequant_rows(t, w, k, n_rows, stream=None):
+def dequant_rows(t, w, k, n_rows, stream=None, packing=PACK_GGUF):
     out = torch.empty((n_rows, k), dtype=torch.float32, device=w.device)
-    check(load().maya_dequant_rows(t, _p(w), 0, k, n_rows, _p(out), _stream(stream)))
+    check(load().maya_dequant_rows_packed(t, packing, _p(w), 0, k, n_rows, _p(out), _stream(stream)))
     return out
+
+
+def copy_layout(l, packing=None):
+    c = Layout()
+    C.memmove(C.byref(c), C.byref(l), C.sizeof(Layout))
+    if packing is not None:
+        c.packing = packing
+    return c
+
+
+def repack(l, src, dst, stream=None):
+    """src (GGUF blob on the device, layout l) -> dst in the stream packing."""
+    check(load().maya_moe_repack(C.byref(l), _p(src), _p(dst), _stream(stream)))
+
+
+def unpack(l, src, dst, stream=None):
+    check(load().maya_moe_unpack(C.byref(l), _p(src), _p(dst), _stream(stream)))
 
 
 def quant_act(act_type, x, stream=None):
@@ -171,9 +194,10 @@ def group(plan_ptr, stream=None):
 class ExpertStore:
     """Expert blobs resident in HBM: one contiguous allocation, expert e's [gate | up | down] blob at `offset[e]` (the
     reference keeps VRAM-resident experts in slots of one pool the same way).  `table` is the device array of blob
-    addresses the plan kernel reads (0: not resident)."""
+    addresses the plan kernel reads (0: not resident).  With `pack_layout` (a GGUF Layout) every blob is regrouped into
+    the stream packing on its way in (maya_moe_repack), as an engine would do when it uploads an expert."""
 
-    def __init__(self, blobs, device="cuda", misalign=0):
+    def __init__(self, blobs, device="cuda", misalign=0, pack_layout=None):
         import numpy as np
         self.n = len(blobs)
         sizes = [int(b.size) for b in blobs]
@@ -182,9 +206,16 @@ class ExpertStore:
         base = self.pool.data_ptr()
         pad = (-base) % 256
         addrs = []
+        staging = torch.empty(max(sizes), dtype=torch.uint8, device=device) if pack_layout is not None else None
         for e, b in enumerate(blobs):
             off = pad + e * stride + misalign
-            self.pool[off:off + sizes[e]].copy_(torch.from_numpy(np.ascontiguousarray(b)), non_blocking=False)
+            src = torch.from_numpy(np.ascontiguousarray(b))
+            if pack_layout is None:
+                self.pool[off:off + sizes[e]].copy_(src, non_blocking=False)
+            else:
+                staging[:sizes[e]].copy_(src, non_blocking=False)
+                repack(pack_layout, staging, self.pool[off:off + sizes[e]])
+                torch.cuda.synchronize()
             addrs.append(base + off)
         self.addrs = addrs
         self.table = torch.tensor(addrs, dtype=torch.int64, device=device)
@@ -195,8 +226,10 @@ class MoeLayer:
     """One routed layer on the device: route -> plan -> group -> quantize -> gate/up -> quantize -> down -> combine
     (maya_moe_layer_decode).  Buffers are allocated once here; a call allocates nothing."""
 
-    def __init__(self, gate_type, down_type, n_embd, n_ff, n_expert, k, max_tokens=1, up_type=None, device="cuda"):
-        self.layout, self.blob_bytes = layout(gate_type, down_type, n_embd, n_ff, up_type)
+    def __init__(self, gate_type, down_type, n_embd, n_ff, n_expert, k, max_tokens=1, up_type=None, device="cuda",
+                 packing=PACK_GGUF):
+        self.gguf_layout, self.blob_bytes = layout(gate_type, down_type, n_embd, n_ff, up_type)
+        self.layout = copy_layout(self.gguf_layout, packing)
         self.n_embd, self.n_ff, self.n_expert, self.k, self.max_tokens = n_embd, n_ff, n_expert, k, max_tokens
         n = int(load().maya_moe_workspace_bytes(C.byref(self.layout), max_tokens, k))
         if n == 0:

@@ -19,15 +19,17 @@ def lib():
 
 
 def run_layer(lib, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x, limit=float("inf"), up_type=None,
-              misalign=0, add=None, resident=None):
-    store = lib.ExpertStore(blobs, misalign=misalign)
+              misalign=0, add=None, resident=None, packing=0):
+    gguf_layout, _ = lib.layout(gate_type, down_type, n_embd, n_ff, up_type)
+    store = lib.ExpertStore(blobs, misalign=misalign, pack_layout=gguf_layout if packing else None)
     table = store.table
     if resident is not None:
         table = table.clone()
         mask = torch.ones(len(blobs), dtype=torch.bool)
         mask[list(resident)] = False
         table[mask.cuda()] = 0
-    layer = lib.MoeLayer(gate_type, down_type, n_embd, n_ff, len(blobs), k, max_tokens=x.shape[0], up_type=up_type)
+    layer = lib.MoeLayer(gate_type, down_type, n_embd, n_ff, len(blobs), k, max_tokens=x.shape[0], up_type=up_type,
+                         packing=packing)
     out = layer.forward(table, dev(logits), x if torch.is_tensor(x) else dev(x), limit=limit,
                         add=None if add is None else dev(add))
     torch.cuda.synchronize()
@@ -46,18 +48,23 @@ CASES = [
     (22, 12, 1024, 768, 12, 8, 8),
     (12, 12, 768, 512, 6, 4, 3),
     (29, 22, 512, 512, 6, 4, 5),
+    # the single-token streaming kernels (n_embd and n_ff multiples of 1024, n_embd a multiple of 14)
+    (22, 22, 7168, 1024, 10, 8, 1),
+    (22, 22, 7168, 2048, 9, 8, 1),
+    (22, 22, 14336, 1024, 4, 3, 1),
 ]
 
 
+@pytest.mark.parametrize("packing", (0, 1))
 @pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", CASES)
-def test_layer_matches_cpu_path(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt):
+def test_layer_matches_cpu_path(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt, packing):
     seed = gt * 1000 + dt * 10 + nt
     blobs = make_experts(gt, dt, n_embd, n_ff, ne, seed)
     rng = np.random.default_rng(seed + 1)
     logits = rng.standard_normal((nt, ne)).astype(np.float32)
     x = rng.standard_normal((nt, n_embd)).astype(np.float32)
-    print("case", gt, dt, n_embd, n_ff, ne, k, nt, flush=True)
-    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x)
+    print("case", gt, dt, n_embd, n_ff, ne, k, nt, packing, flush=True)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=packing)
     wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x)
     assert np.array_equal(ids, wi)
     for t in range(nt):
@@ -116,17 +123,21 @@ def test_zero_input_and_bf16_input(lib, oracle):
     assert np.array_equal(ids, wi) and rel_l2(out, wout) <= TOL
 
 
-def test_window_rows_equal_token_rows(lib):
-    """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract)."""
-    gt, dt, n_embd, n_ff, ne, k, nt = 22, 12, 1024, 512, 10, 4, 6
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3)))
+def test_window_rows_equal_token_rows(lib, gt, dt, n_embd, n_ff, ne, k, nt):
+    """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract), in either
+    row packing."""
     blobs = make_experts(gt, dt, n_embd, n_ff, ne, 33)
     rng = np.random.default_rng(34)
     logits = rng.standard_normal((nt, ne)).astype(np.float32)
     x = rng.standard_normal((nt, n_embd)).astype(np.float32)
     _, _, win, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x)
+    _, _, winp, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=1)
+    assert np.array_equal(win.view(np.uint32), winp.view(np.uint32))
     for t in range(nt):
-        _, _, one, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits[t:t + 1], x[t:t + 1])
-        assert np.array_equal(win[t].view(np.uint32), one[0].view(np.uint32)), t
+        for packing in (0, 1):
+            _, _, one, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits[t:t + 1], x[t:t + 1], packing=packing)
+            assert np.array_equal(win[t].view(np.uint32), one[0].view(np.uint32)), (t, packing)
 
 
 def test_unsupported_and_bad_shapes_fail_cleanly(lib):

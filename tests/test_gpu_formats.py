@@ -101,3 +101,31 @@ def test_i8x32_quant_byte_exact(lib, oracle):
     for r, src in enumerate(idx):
         wq, wd = oracle.quant_i8x32(x[src])
         assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
+
+
+@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8)))
+def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
+    """maya_moe_repack regroups bytes only: unpack(repack(blob)) == blob, and the packed rows dequantize to the same bits."""
+    n_embd, n_ff = 1024, 512
+    rng = np.random.default_rng(gt * 100 + dt)
+    blob = synth.expert_blob(gt, dt, n_embd, n_ff, rng)
+    l, nbytes = lib.layout(gt, dt, n_embd, n_ff)
+    assert nbytes == blob.size
+    src = torch.from_numpy(blob).cuda()
+    packed = torch.zeros_like(src)
+    back = torch.zeros_like(src)
+    lib.repack(l, src, packed)
+    lib.unpack(l, packed, back)
+    torch.cuda.synchronize()
+    assert torch.equal(back, src)
+    # a permutation of bytes inside each row: same multiset of bytes per row
+    for t, off, k, rows in ((gt, 0, n_embd, n_ff), (gt, l.up_off, n_embd, n_ff), (dt, l.down_off, n_ff, n_embd)):
+        rb = lib.row_bytes(t, k)
+        a = src[off:off + rb * rows].view(rows, rb).cpu().numpy()
+        b = packed[off:off + rb * rows].view(rows, rb).cpu().numpy()
+        assert np.array_equal(np.sort(a, axis=1), np.sort(b, axis=1))
+        if t != 22:
+            assert np.array_equal(a, b)
+        want = oracle.dequant_rows(t, blob[off:off + rb * 16], k, 16)
+        got = lib.dequant_rows(t, packed[off:], k, 16, packing=1).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
