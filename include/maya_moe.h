@@ -98,6 +98,9 @@ typedef struct maya_moe_args {
     const float* add;          /* NULL or [n_tokens][n_embd] added to the combined output (shared expert, CPU lane part) */
     const int32_t* add_flag;   /* NULL or a device flag: `add` is added only when it is non-zero */
     float* out;                /* [n_tokens][n_embd] */
+    int32_t* hq_sync;          /* NULL, or [n_tokens*k][n_ff/256] arrival counters, all zero at the call: a gate/up
+                                * kernel that can (maya_moe_gate_up_fuses_hq) then also writes hq, the Q8_K rounding of
+                                * h, from the last workgroup to finish each 256-value block */
 } maya_moe_args;
 
 /* ---- probes: glmf::moe_supported, iq::supported / block_bytes / row_bytes (src/ds4/ds4_iq.cuh:40-52) */
@@ -167,6 +170,9 @@ int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, i
  *   glmf::moe_down (glm_fast.hpp:499-501), iq::down (ds4_iq.cuh:90-91), native_down_rows_split
  *   (native_expert.cpp:395-417), native_moe_combine (src/kernels/cuda/native_moe.cu:36-52). */
 int maya_moe_gate_up(const maya_moe_args* a, void* stream);
+/* 1 when maya_moe_gate_up, given hq_sync, writes hq itself for these arguments (the caller then skips maya_quant_act
+ * of h), 0 when it leaves hq alone. */
+int maya_moe_gate_up_fuses_hq(const maya_moe_args* a);
 int maya_moe_down(const maya_moe_args* a, void* stream);
 
 /* ---- the whole routed layer for a decode step / verify window of n_tokens <= MAYA_MAX_TOKENS tokens:

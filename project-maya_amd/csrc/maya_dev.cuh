@@ -91,12 +91,14 @@ template <> struct Fmt<kIQ2_S> {
     __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
         decode_fields(ld32_a2(blk + 2 + 4 * ib), ld32_a2(blk + 34 + 4 * ib), blk[66 + ib], blk[74 + ib], grid, u);
     }
-    // the stream packing of a row of nu sub-blocks: [nu x (index word, sign word)] [nu x (high bits, scales)] [nu/8 x d]
-    __device__ static __forceinline__ void decode_stream(const uint8_t* row, int nu, int un, const uint2* grid, Unit32& u,
-                                                         float& d) {
-        const uint2 is = ((const uint2*) row)[un];
-        const uint32_t hs = ((const uint16_t*) (row + 8 * (size_t) nu))[un];
-        d = f16_bits_to_f32(((const uint16_t*) (row + 10 * (size_t) nu))[un >> 3]) * 0.125f;
+    // the stream packing: rows in quads (rows 4q .. 4q+3); a quad of rows of nu sub-blocks is
+    //   [nu][4] (index word, sign word) | [nu][4] (high bits, scales) | [nu/8][4] d      (4 x the row's bytes)
+    // quad = the quad's first byte, rq = the row inside it
+    __device__ static __forceinline__ void decode_stream(const uint8_t* quad, int nu, int rq, int un, const uint2* grid,
+                                                         Unit32& u, float& d) {
+        const uint2 is = ((const uint2*) quad)[un * 4 + rq];
+        const uint32_t hs = ((const uint16_t*) (quad + 32 * (size_t) nu))[un * 4 + rq];
+        d = f16_bits_to_f32(((const uint16_t*) (quad + 40 * (size_t) nu))[(un >> 3) * 4 + rq]) * 0.125f;
         decode_fields(is.x, is.y, hs & 255u, hs >> 8, grid, u);
     }
 };

@@ -29,23 +29,11 @@ struct RawIQ2S {
 };
 
 // the lane's KU sub-blocks of one IQ2_S row: sub-block u = sub + LPR j.
-// GGUF rows: u sits in block u / 8 at position u % 8 (2-byte aligned fields).  Stream rows: field arrays, aligned.
+// GGUF rows: u sits in block u / 8 at position u % 8 (2-byte aligned fields).
 template <int KU, int LPR, bool STREAM>
 __device__ __forceinline__ void load_iq2s(gptr8 row, int sub, RawIQ2S (&raw)[KU]) {
-    if constexpr (STREAM) {
-        constexpr int NU = KU * LPR;
-        gptr64 is = (gptr64) row + sub;
-        gptr16 hs = (gptr16) (row + 8 * NU) + sub;
-        gptr16 d = (gptr16) (row + 10 * NU) + (sub >> 3);
-#pragma unroll
-        for (int j = 0; j < KU; ++j) {
-            const u32x2 v = is[j * LPR];
-            raw[j].i4 = v.x;
-            raw[j].sg4 = v.y;
-            raw[j].hs = hs[j * LPR];
-            raw[j].d = d[j * (LPR / 8)];
-        }
-    } else {
+    static_assert(!STREAM, "the stream packing is read by the position-mapped kernels");
+    {
         gptr8 p = row + (sub >> 3) * 82 + (sub & 7);
         const int ib3 = 3 * (sub & 7);  // the 4-byte fields advance 4 bytes a sub-block: 1 from p, 3 here
 #pragma unroll
@@ -236,6 +224,285 @@ __global__ __launch_bounds__(512) void down_iq2s_1tok_kernel(maya_moe_args a, Co
 #pragma unroll
                 for (int j = 0; j < KU; ++j) cur[j] = nxt[j];
             }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < ROWS) {
+        const int c = threadIdx.x;
+        float sum = 0.0f;
+        bool first = true;
+        for (int i = 0; i < a.k; ++i) {
+            if (a.plan_ptr[i] == 0ull) continue;
+            const float p = __fmul_rn(part[i][c], a.plan_w[i]);
+            sum = first ? p : __fadd_rn(sum, p);
+            first = false;
+        }
+        if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[r0 + c]);
+        a.out[r0 + c] = sum;
+        if (a.part)
+            for (int i = 0; i < a.k; ++i)
+                if (a.plan_ptr[i] != 0ull) a.part[(size_t) i * n_embd + r0 + c] = part[i][c];
+    }
+}
+
+// ================================================================================================================
+// Position-mapped kernels (stream packing): a lane owns ONE sub-block position of the row (its 32 activation codes
+// stay in 8 registers), walks down the rows with a ring of prefetched rows, and every 8 rows a butterfly over the
+// lanes turns 8 per-lane values into per-row sums.  Loads of a wave are contiguous 512-byte / 128-byte runs.
+
+// acc[i] = this lane's value for row i of the batch.  On return every lane holds, in acc[0], the sum over its
+// 32-lane half of the values of row (lane >> 2) & 7.
+__device__ __forceinline__ float reduce8_half(float (&acc)[8], int lane) {
+    const bool b4 = lane & 16, b3 = lane & 8, b2 = lane & 4;
+    float v4[4], v2[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float send = b4 ? acc[i] : acc[i + 4], keep = b4 ? acc[i + 4] : acc[i];
+        v4[i] = keep + __shfl_xor(send, 16, kWave);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float send = b3 ? v4[i] : v4[i + 2], keep = b3 ? v4[i + 2] : v4[i];
+        v2[i] = keep + __shfl_xor(send, 8, kWave);
+    }
+    const float send = b2 ? v2[0] : v2[1], keep = b2 ? v2[1] : v2[0];
+    float v = keep + __shfl_xor(send, 4, kWave);
+    v += __shfl_xor(v, 2, kWave);
+    v += __shfl_xor(v, 1, kWave);
+    return v;
+}
+
+typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
+
+// A lane's share of one quad of rows (4 rows x its sub-block): 12 registers
+struct QuadIQ2S {
+    u32x4 is01, is23;  // (index word, sign word) of rows 0,1 and 2,3
+    u32x2 hs, d;       // four (high bits | scales << 8) halfwords, four FP16 block scales
+};
+struct QuadOffs {  // byte offsets of the lane's fields inside a quad; quads advance through the scalar offset
+    uint32_t is, hs, d;
+};
+template <int NU>
+__device__ __forceinline__ QuadOffs quad_offs(uint32_t mat_off, int u) {
+    return QuadOffs{mat_off + 32u * u, mat_off + 32u * NU + 8u * u, mat_off + 40u * NU + 8u * (u >> 3)};
+}
+// A raw buffer resource over `bytes` of weights at `base`: loads take a per-lane 32-bit offset plus a scalar offset
+// (no vector address arithmetic in the row loop), and a load past `bytes` returns zero instead of faulting.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t weight_rsrc(uint64_t base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*) base, 0, (int) bytes, 0x00020000);
+}
+__device__ __forceinline__ QuadIQ2S load_quad(__amdgpu_buffer_rsrc_t rs, const QuadOffs& o, uint32_t quad_off) {
+    QuadIQ2S q;
+    q.is01 = __builtin_amdgcn_raw_buffer_load_b128(rs, o.is, quad_off, 0);
+    q.is23 = __builtin_amdgcn_raw_buffer_load_b128(rs, o.is + 16u, quad_off, 0);
+    q.hs = __builtin_amdgcn_raw_buffer_load_b64(rs, o.hs, quad_off, 0);
+    q.d = __builtin_amdgcn_raw_buffer_load_b64(rs, o.d, quad_off, 0);
+    return q;
+}
+template <int R>
+__device__ __forceinline__ RawIQ2S quad_row(const QuadIQ2S& q) {
+    RawIQ2S r;
+    const u32x4 v = R < 2 ? q.is01 : q.is23;
+    r.i4 = (R & 1) ? v.z : v.x;
+    r.sg4 = (R & 1) ? v.w : v.y;
+    const uint32_t h = R < 2 ? q.hs.x : q.hs.y, d = R < 2 ? q.d.x : q.d.y;
+    r.hs = (R & 1) ? (h >> 16) : (h & 0xffffu);
+    r.d = (R & 1) ? (d >> 16) : (d & 0xffffu);
+    return r;
+}
+// One sub-block against the lane's activation codes y and their negation yn: with m the negative values' mask,
+//   sum s_i g_i y_i = dot4(g ^ m, y) + dot4(m, -y)      (g ^ 0xff = -g - 1, m = -1 there)
+// so each 16-value half needs one accumulator and no subtraction.  dy8 = the activation scale / 8.
+__device__ __forceinline__ float unit_value(const RawIQ2S& r, const uint2* grid, const uint2* stab, const int (&y)[8],
+                                            const int (&yn)[8], float dy8) {
+    int t0 = 0, t1 = 0;
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        const uint32_t idx = ((r.i4 >> (8 * l)) & 255u) | ((r.hs << (8 - 2 * l)) & 0x300u);
+        const uint2 g = grid[idx];
+        const uint2 m = stab[(r.sg4 >> (8 * l)) & 255u];
+        if (l < 2) {
+            t0 = dot4((int) (g.x ^ m.x), y[2 * l], t0);
+            t0 = dot4((int) m.x, yn[2 * l], t0);
+            t0 = dot4((int) (g.y ^ m.y), y[2 * l + 1], t0);
+            t0 = dot4((int) m.y, yn[2 * l + 1], t0);
+        } else {
+            t1 = dot4((int) (g.x ^ m.x), y[2 * l], t1);
+            t1 = dot4((int) m.x, yn[2 * l], t1);
+            t1 = dot4((int) (g.y ^ m.y), y[2 * l + 1], t1);
+            t1 = dot4((int) m.y, yn[2 * l + 1], t1);
+        }
+    }
+    const int s0 = 2 * (int) ((r.hs >> 8) & 15u) + 1, s1 = 2 * (int) ((r.hs >> 12) & 15u) + 1;
+    const int isum = __mul24(s0, t0) + __mul24(s1, t1);
+    return __fmul_rn(__fmul_rn(f16_bits_to_f32(r.d), dy8), (float) isum);
+}
+// the byte-wise negation of four int8 codes (none is -128)
+__device__ __forceinline__ int neg4(int v) {
+    const uint32_t x = ~(uint32_t) v;
+    return (int) (((x & 0x7f7f7f7fu) + 0x01010101u) ^ (x & 0x80808080u));
+}
+// the four rows of a quad: acc[B + r] = this lane's value for row r.  Each value is pinned where it is made: without
+// that the optimizer sinks all the batch's decodes down to the reduction and keeps every prefetched quad live.
+template <int B>
+__device__ __forceinline__ void quad_values(const QuadIQ2S& q, const uint2* grid, const uint2* stab, const int (&y)[8],
+                                            const int (&yn)[8], float dy8, float (&acc)[8]) {
+#define MAYA_ROW(R)                                                              \
+    acc[B + R] = unit_value(quad_row<R>(q), grid, stab, y, yn, dy8);             \
+    asm volatile("" : "+v"(acc[B + R]));                                         \
+    __builtin_amdgcn_sched_barrier(0);
+    MAYA_ROW(0) MAYA_ROW(1) MAYA_ROW(2) MAYA_ROW(3)
+#undef MAYA_ROW
+}
+
+// ---- gate/up, one token, n_embd = 1024 NW: a workgroup of NW waves = the 2 * 32 NW sub-block positions of a
+// (gate row, up row) pair; grid (n_ff / ROWS, k).  DEPTH rows are in flight per lane.
+template <int NW, int ROWS, int DEPTH, int MINW>
+__global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
+    static_assert(ROWS % 8 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads; the ring holds one or two");
+    constexpr int NU = 32 * NW;  // sub-blocks a row
+    __shared__ int lds[kFastLdsWords];
+    __shared__ float part[2][2 * NW][8];
+    if (a.skip && *a.skip) return;
+    const int e = blockIdx.y;
+    const uint64_t blob = a.plan_ptr[e];
+    if (blob == 0ull) return;
+    stage_iq2s_tables(lds, cb, 64 * NW);
+    const uint2* grid = (const uint2*) lds;
+    const uint2* stab = (const uint2*) (lds + 2048);
+    const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
+    const bool is_up = t >= NU;
+    const int u = is_up ? t - NU : t;
+    int y[8];
+    {
+        const int4* q = (const int4*) a.x.q;
+        const int4 ya = q[2 * u], yb = q[2 * u + 1];
+        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+    }
+    int yn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
+    const float dy8 = a.x.d[u] * 0.125f;
+    constexpr uint32_t qb = NU / 8 * 82 * 4;  // bytes of a quad of rows
+    const int n_ff = a.layout.n_ff, r0 = blockIdx.x * ROWS;
+    // one resource over the expert's gate and up rows; the up rows ride in the lane offset
+    const __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob + a.layout.gate_off, (uint32_t) (a.layout.down_off - a.layout.gate_off));
+    const QuadOffs qo = quad_offs<NU>(is_up ? (uint32_t) (a.layout.up_off - a.layout.gate_off) : 0u, u);
+    const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+    constexpr int NQ = ROWS / 4;
+    QuadIQ2S ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
+    __syncthreads();
+    float acc[8];
+#pragma unroll 1
+    for (int r = 0; r < ROWS; r += 8) {
+        const int q = r >> 2;
+        {
+            const QuadIQ2S cur = ring[0];
+            if (q + DEPTH < NQ) ring[0] = load_quad(rs, qo, quad0 + (uint32_t) (q + DEPTH) * qb);
+            quad_values<0>(cur, grid, stab, y, yn, dy8, acc);
+        }
+        {
+            const QuadIQ2S cur = ring[1 % DEPTH];
+            if (q + 1 + DEPTH < NQ) ring[1 % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + 1 + DEPTH) * qb);
+            quad_values<4>(cur, grid, stab, y, yn, dy8, acc);
+        }
+        const float v = reduce8_half(acc, lane);
+        const int buf = (r >> 3) & 1;
+        if ((lane & 3) == 0) part[buf][hw][(lane >> 2) & 7] = v;
+        __syncthreads();
+        if (t < 8) {
+            float g = part[buf][0][t], up = part[buf][NW][t];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                g += part[buf][w][t];
+                up += part[buf][NW + w][t];
+            }
+            // (a device-coherent store: another workgroup may read the row back to round h, with no cache flush between)
+            if (r0 + r + t < n_ff)
+                __hip_atomic_store(a.h + (size_t) e * n_ff + r0 + r + t, swiglu(g, up, a.limit), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (a.hq_sync == nullptr) return;
+    // The Q8_K rounding of h for the down rows: the last of the 256 / ROWS workgroups that share a 256-value block
+    // of h rounds it.  The rows of h are written and read back with device-coherent accesses, so no cache-wide
+    // fence is needed (on this multi-die part a device-scope fence writes back and invalidates whole L2 caches): a
+    // writer waits for its stores to be acknowledged, the workgroup meets, and only then is its arrival counted.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    __shared__ int s_last;
+    const int blk = r0 >> 8, nblk = n_ff >> 8;
+    if (t == 0) {
+        const int seen = __hip_atomic_fetch_add(a.hq_sync + e * nblk + blk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = seen == 256 / ROWS - 1;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    static_assert(NW >= 4, "the block rounding wants 256 threads");
+    const bool active = t < 256;
+    const float hv = active ? __hip_atomic_load(a.h + (size_t) e * n_ff + (size_t) blk * 256 + t, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT)
+                            : 0.0f;
+    quant_q8k_block(hv, t, active, lds, a.hq, (size_t) e * n_ff + (size_t) blk * 256);
+}
+
+// ---- down + combine, one token, n_ff = 2048 (64 sub-blocks a row = one wave): wave w = plan slot w, rows in batches
+// of 8; grid (n_embd / ROWS).  The slots' rows meet in LDS and are summed in slot order.
+template <int ROWS, int DEPTH, int MINW>
+__global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
+    static_assert(ROWS % 8 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads; the ring holds one or two");
+    constexpr int NU = 64;
+    __shared__ int lds[kFastLdsWords];
+    __shared__ float part[8][ROWS];
+    if (a.skip && *a.skip) return;
+    stage_iq2s_tables(lds, cb, 512);
+    const uint2* grid = (const uint2*) lds;
+    const uint2* stab = (const uint2*) (lds + 2048);
+    const int n_embd = a.layout.n_embd;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r0 = blockIdx.x * ROWS;
+    const uint64_t blob = wave < a.k ? a.plan_ptr[wave] : 0ull;
+    __syncthreads();
+    if (blob != 0ull) {
+        int y[8];
+        const int4* q = (const int4*) (a.hq.q + (size_t) wave * 2048);
+        const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+        int yn[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
+        const float dy8 = a.hq.d[(size_t) wave * 64 + lane] * 0.125f;
+        constexpr uint32_t qb = NU / 8 * 82 * 4;
+        // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
+        // scalar registers for the buffer resource
+        const uint64_t mat = blob + a.layout.down_off;
+        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
+        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
+        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
+        const QuadOffs qo = quad_offs<NU>(0u, lane);
+        const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+        constexpr int NQ = ROWS / 4;
+        QuadIQ2S ring[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
+        float acc[8];
+#pragma unroll 1
+        for (int r = 0; r < ROWS; r += 8) {
+            const int q = r >> 2;
+            {
+                const QuadIQ2S cur = ring[0];
+                if (q + DEPTH < NQ) ring[0] = load_quad(rs, qo, quad0 + (uint32_t) (q + DEPTH) * qb);
+                quad_values<0>(cur, grid, stab, y, yn, dy8, acc);
+            }
+            {
+                const QuadIQ2S cur = ring[1 % DEPTH];
+                if (q + 1 + DEPTH < NQ) ring[1 % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + 1 + DEPTH) * qb);
+                quad_values<4>(cur, grid, stab, y, yn, dy8, acc);
+            }
+            float v = reduce8_half(acc, lane);
+            v += __shfl_xor(v, 32, kWave);
+            if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
         }
     }
     __syncthreads();

@@ -129,12 +129,13 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
         uint32_t qs, sg, h, sc, dbits;
         if (packing == MAYA_PACK_STREAM) {
-            const int64_t nu = k >> 5, un = v >> 5;
-            qs = rp[8 * un + il];
-            sg = rp[8 * un + 4 + il];
-            h = rp[8 * nu + 2 * un];
-            sc = rp[8 * nu + 2 * un + 1];
-            dbits = ld16(rp + 10 * nu + 2 * (un >> 3));
+            const int64_t nu = k >> 5, un = v >> 5, rq = row & 3;
+            const uint8_t* quad = w + (size_t) (row >> 2) * 4 * row_stride;
+            qs = quad[8 * (un * 4 + rq) + il];
+            sg = quad[8 * (un * 4 + rq) + 4 + il];
+            h = quad[32 * nu + 2 * (un * 4 + rq)];
+            sc = quad[32 * nu + 2 * (un * 4 + rq) + 1];
+            dbits = ld16(quad + 40 * nu + 2 * ((un >> 3) * 4 + rq));
         } else {
             const uint8_t* blk = rp + (size_t) (v >> 8) * 82;
             qs = blk[2 + 4 * ib + il];
@@ -174,37 +175,38 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 
 // ------------------------------------------------------------------------------------------------ stream packing
 
-// IQ2_S rows between the GGUF block sequence and the stream order; one thread a sub-block, grid (k/256 blocks / 32, rows).
-// DIR 0: GGUF -> stream, 1: stream -> GGUF.  Every byte of a row is written exactly once.
+// IQ2_S rows between the GGUF block sequence and the stream order (rows in quads, fields regrouped); one thread a
+// sub-block, grid (k/32 sub-blocks / 256, rows).  DIR 0: GGUF -> stream, 1: stream -> GGUF.  Every byte is written once.
 template <int DIR>
 __global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
                                                           int64_t k, int64_t n_rows) {
     const int64_t nu = k >> 5, rb = (k >> 8) * 82;
     const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
     if (un >= nu) return;
-    const uint8_t* s = src + row * rb;
-    uint8_t* d = dst + row * rb;
-    const int64_t b = un >> 3;
+    const int64_t b = un >> 3, rq = row & 3;
     const int ib = (int) (un & 7);
-    const uint8_t* g = (DIR == 0 ? s : d) + b * 82;   // the GGUF side's block (only its address matters for DIR 1)
+    const uint8_t* gs = src + row * rb + b * 82;              // GGUF side when DIR == 0
+    uint8_t* gd = dst + row * rb + b * 82;                    // GGUF side when DIR == 1
+    const uint8_t* qs = src + (row >> 2) * 4 * rb;            // stream side (the quad) when DIR == 1
+    uint8_t* qd = dst + (row >> 2) * 4 * rb;                  // stream side when DIR == 0
+    const int64_t o_is = 8 * (un * 4 + rq), o_hs = 32 * nu + 2 * (un * 4 + rq), o_d = 40 * nu + 2 * (b * 4 + rq);
     if (DIR == 0) {
-        for (int i = 0; i < 4; ++i) d[8 * un + i] = g[2 + 4 * ib + i];
-        for (int i = 0; i < 4; ++i) d[8 * un + 4 + i] = g[34 + 4 * ib + i];
-        d[8 * nu + 2 * un] = g[66 + ib];
-        d[8 * nu + 2 * un + 1] = g[74 + ib];
+        for (int i = 0; i < 4; ++i) qd[o_is + i] = gs[2 + 4 * ib + i];
+        for (int i = 0; i < 4; ++i) qd[o_is + 4 + i] = gs[34 + 4 * ib + i];
+        qd[o_hs] = gs[66 + ib];
+        qd[o_hs + 1] = gs[74 + ib];
         if (ib == 0) {
-            d[10 * nu + 2 * b] = g[0];
-            d[10 * nu + 2 * b + 1] = g[1];
+            qd[o_d] = gs[0];
+            qd[o_d + 1] = gs[1];
         }
     } else {
-        uint8_t* o = d + b * 82;
-        for (int i = 0; i < 4; ++i) o[2 + 4 * ib + i] = s[8 * un + i];
-        for (int i = 0; i < 4; ++i) o[34 + 4 * ib + i] = s[8 * un + 4 + i];
-        o[66 + ib] = s[8 * nu + 2 * un];
-        o[74 + ib] = s[8 * nu + 2 * un + 1];
+        for (int i = 0; i < 4; ++i) gd[2 + 4 * ib + i] = qs[o_is + i];
+        for (int i = 0; i < 4; ++i) gd[34 + 4 * ib + i] = qs[o_is + 4 + i];
+        gd[66 + ib] = qs[o_hs];
+        gd[74 + ib] = qs[o_hs + 1];
         if (ib == 0) {
-            o[0] = s[10 * nu + 2 * b];
-            o[1] = s[10 * nu + 2 * b + 1];
+            gd[0] = qs[o_d];
+            gd[1] = qs[o_d + 1];
         }
     }
 }
@@ -229,11 +231,10 @@ __device__ __forceinline__ int nearest_int(float f) {
 
 // Q8_K: one workgroup of 256 threads a 256-value block (src/kernels/cuda/quantize_act.cu:161-207).  The block's signed
 // maximum is the value at the FIRST largest magnitude: the reduction keeps (|x|, index) and prefers the lower index.
-template <int DT>
-__global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__ x, int64_t x_stride, int64_t k,
-                                                        maya_act out) {
-    const int row = blockIdx.y, b = blockIdx.x, j = threadIdx.x;
-    const float xv = load_x<DT>(x, (int64_t) row * x_stride + (int64_t) b * 256 + j);
+// One 256-value block by the first 256 threads of a workgroup (j = the thread's value, active = j < 256); `sm` is
+// 256 + 8 words of LDS.  EVERY thread of the workgroup calls it (it holds a workgroup barrier); whole waves are active
+// or idle.
+__device__ __forceinline__ void quant_q8k_block(float xv, int j, bool active, int* sm, const maya_act& out, size_t base) {
     float am = fabsf(xv);
     int ix = j;
 #pragma unroll
@@ -245,15 +246,18 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__
             ix = oi;
         }
     }
-    __shared__ float s_am[4];
-    __shared__ int s_ix[4];
-    __shared__ float s_x[256];
-    s_x[j] = xv;
-    if ((j & 63) == 0) {
-        s_am[j >> 6] = am;
-        s_ix[j >> 6] = ix;
+    float* s_x = (float*) sm;
+    float* s_am = (float*) (sm + 256);
+    int* s_ix = sm + 260;
+    if (active) {
+        s_x[j] = xv;
+        if ((j & 63) == 0) {
+            s_am[j >> 6] = am;
+            s_ix[j >> 6] = ix;
+        }
     }
     __syncthreads();
+    if (!active) return;
     am = s_am[0];
     ix = s_ix[0];
 #pragma unroll
@@ -269,13 +273,21 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__
         q = min(127, nearest_int(__fmul_rn(iscale, xv)));
         d = __fdiv_rn(1.0f, iscale);
     }
-    const size_t base = (size_t) row * k + (size_t) b * 256;
     out.q[base + j] = (int8_t) q;
     int s = q;
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
     if ((j & 15) == 0) out.bsums[(base >> 4) + (j >> 4)] = (int16_t) s;
     if (j < 8) out.d[(base >> 5) + j] = d;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__ x, int64_t x_stride, int64_t k,
+                                                        maya_act out) {
+    __shared__ int sm[264];
+    const int row = blockIdx.y, b = blockIdx.x, j = threadIdx.x;
+    const float xv = load_x<DT>(x, (int64_t) row * x_stride + (int64_t) b * 256 + j);
+    quant_q8k_block(xv, j, true, sm, out, (size_t) row * k + (size_t) b * 256);
 }
 
 // Q8_0: 32-value blocks, d = amax / 127 kept as FP16, q = roundf(x / d) with the unrounded F32 d
@@ -323,40 +335,51 @@ __global__ __launch_bounds__(256) void quant_i8x32_kernel(const void* __restrict
 // One workgroup a token (src/kernels/cuda/router_top10.cu:68-187): the maximum (exact in any order), the exponentials in
 // double in parallel, their sum ascending on one thread, p = (float)(ex * inv) with inv a float, k rounds of a
 // workgroup-wide arg-max with a strict > and the lower index on ties, renormalisation by max(sum, 2^-14) in double.
-__global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k,
-                                                     int32_t* __restrict__ ids, float* __restrict__ weights) {
-    __shared__ double s_ex[MAYA_MAX_EXPERTS];
-    __shared__ float s_p[MAYA_MAX_EXPERTS];
-    __shared__ float s_rv[4];
-    __shared__ int s_ri[4];
-    __shared__ double s_sum;
-    __shared__ float s_w[MAYA_MAX_K];
-    const int t = blockIdx.x, tid = threadIdx.x;
-    const float* l = logits + (size_t) t * n_expert;
+struct RouterLds {
+    double ex[MAYA_MAX_EXPERTS];
+    float p[MAYA_MAX_EXPERTS];
+    float rv[4];
+    int ri[4];
+    double sum;
+    float w[MAYA_MAX_K];
+    int id[MAYA_MAX_K];
+};
+// 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights (thread 0 wrote them)
+__device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
+    const int tid = threadIdx.x;
     float mx = -INFINITY;
     for (int e = tid; e < n_expert; e += 256) mx = fmaxf(mx, l[e]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
-    if ((tid & 63) == 0) s_rv[tid >> 6] = mx;
+    if ((tid & 63) == 0) sm.rv[tid >> 6] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(s_rv[0], s_rv[1]), fmaxf(s_rv[2], s_rv[3]));
+    mx = fmaxf(fmaxf(sm.rv[0], sm.rv[1]), fmaxf(sm.rv[2], sm.rv[3]));
     __syncthreads();
-    for (int e = tid; e < n_expert; e += 256) s_ex[e] = exp((double) l[e] - (double) mx);
+    for (int e = tid; e < n_expert; e += 256) sm.ex[e] = exp((double) l[e] - (double) mx);
     __syncthreads();
     if (tid == 0) {
+        // ascending, one add after the other (the reference's order); the reads run eight ahead of the adds
         double sum = 0.0;
-        for (int e = 0; e < n_expert; ++e) sum += s_ex[e];
-        s_sum = sum;
+        int e = 0;
+        for (; e + 8 <= n_expert; e += 8) {
+            double v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = sm.ex[e + j];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum += v[j];
+        }
+        for (; e < n_expert; ++e) sum += sm.ex[e];
+        sm.sum = sum;
     }
     __syncthreads();
-    const float inv = (float) (1.0 / s_sum);
-    for (int e = tid; e < n_expert; e += 256) s_p[e] = (float) (s_ex[e] * (double) inv);
+    const float inv = (float) (1.0 / sm.sum);
+    for (int e = tid; e < n_expert; e += 256) sm.p[e] = (float) (sm.ex[e] * (double) inv);
     __syncthreads();
     for (int i = 0; i < k; ++i) {
         float bv = -INFINITY;
         int bi = n_expert;
         for (int e = tid; e < n_expert; e += 256) {
-            const float pe = s_p[e];
+            const float pe = sm.p[e];
             if (pe > bv) {
                 bv = pe;
                 bi = e;
@@ -372,30 +395,71 @@ __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ l
             }
         }
         if ((tid & 63) == 0) {
-            s_rv[tid >> 6] = bv;
-            s_ri[tid >> 6] = bi;
+            sm.rv[tid >> 6] = bv;
+            sm.ri[tid >> 6] = bi;
         }
         __syncthreads();
         if (tid == 0) {
-            float v = s_rv[0];
-            int ix = s_ri[0];
+            float v = sm.rv[0];
+            int ix = sm.ri[0];
             for (int w = 1; w < 4; ++w)
-                if (s_rv[w] > v || (s_rv[w] == v && s_ri[w] < ix)) {
-                    v = s_rv[w];
-                    ix = s_ri[w];
+                if (sm.rv[w] > v || (sm.rv[w] == v && sm.ri[w] < ix)) {
+                    v = sm.rv[w];
+                    ix = sm.ri[w];
                 }
             if (ix >= n_expert) ix = 0;  // only when every remaining probability is NaN
-            ids[(size_t) t * k + i] = ix;
-            s_w[i] = s_p[ix];
-            s_p[ix] = -INFINITY;  // taken: never selected again (a probability is >= 0)
+            sm.id[i] = ix;
+            sm.w[i] = sm.p[ix];
+            sm.p[ix] = -INFINITY;  // taken: never selected again (a probability is >= 0)
         }
         __syncthreads();
     }
     if (tid == 0) {
         double s = 0.0;
-        for (int i = 0; i < k; ++i) s += (double) s_w[i];
+        for (int i = 0; i < k; ++i) s += (double) sm.w[i];
         const double sc = fmax(s, 6.103515625e-05);
-        for (int i = 0; i < k; ++i) weights[(size_t) t * k + i] = (float) ((double) s_w[i] / sc);
+        for (int i = 0; i < k; ++i) sm.w[i] = (float) ((double) sm.w[i] / sc);
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k,
+                                                     int32_t* __restrict__ ids, float* __restrict__ weights) {
+    __shared__ RouterLds sm;
+    const int t = blockIdx.x;
+    route_token(logits + (size_t) t * n_expert, n_expert, k, sm);
+    if (threadIdx.x < k) {
+        ids[(size_t) t * k + threadIdx.x] = sm.id[threadIdx.x];
+        weights[(size_t) t * k + threadIdx.x] = sm.w[threadIdx.x];
+    }
+}
+
+// The layer's head in one launch, grid (1 + n_embd / 256, n_tokens): workgroup 0 of a token routes it, writes its
+// plan slots (blob addresses from the residency table) and - for token 0 - clears the gate/up kernels' arrival
+// counters; the other workgroups round one 256-value block of the hidden state each to Q8_K.
+template <int DT>
+__global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict__ logits, int n_expert, int k,
+                                                         const uint64_t* __restrict__ table, int32_t* __restrict__ ids,
+                                                         float* __restrict__ weights, uint64_t* __restrict__ plan,
+                                                         const void* __restrict__ x, int64_t n_embd, maya_act xq,
+                                                         int32_t* __restrict__ counters, int n_counters) {
+    __shared__ RouterLds sm;
+    __shared__ int qs[264];
+    const int t = blockIdx.y;
+    if (blockIdx.x == 0) {
+        if (t == 0)
+            for (int i = threadIdx.x; i < n_counters; i += 256) counters[i] = 0;
+        route_token(logits + (size_t) t * n_expert, n_expert, k, sm);
+        if (threadIdx.x < k) {
+            const int id = sm.id[threadIdx.x];
+            ids[(size_t) t * k + threadIdx.x] = id;
+            weights[(size_t) t * k + threadIdx.x] = sm.w[threadIdx.x];
+            plan[(size_t) t * k + threadIdx.x] = (id >= 0 && id < n_expert) ? table[id] : 0ull;
+        }
+    } else {
+        const int b = blockIdx.x - 1, j = threadIdx.x;
+        const float xv = load_x<DT>(x, (int64_t) t * n_embd + (int64_t) b * 256 + j);
+        quant_q8k_block(xv, j, true, qs, xq, (size_t) t * n_embd + (size_t) b * 256);
     }
 }
 
@@ -480,7 +544,7 @@ struct ActLds {
 // lane's part.  `sub` = lane index inside the group.
 template <int TYPE, int NT, int LPR>
 __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, int sub, const ActLds& a,
-                                        const uint2* __restrict__ grid, float (&acc)[NT], bool stream_packed) {
+                                        const uint2* __restrict__ grid, float (&acc)[NT], bool stream_packed, int rq) {
     if constexpr (TYPE == kQ4_K) {
         const int np = k >> 6;
         for (int p = sub; p < np; p += LPR) {
@@ -520,7 +584,7 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
             Unit32 u;
             float D;
             if (TYPE == kIQ2_S && stream_packed) {
-                if constexpr (TYPE == kIQ2_S) Fmt<kIQ2_S>::decode_stream(row, nu, un, grid, u, D);
+                if constexpr (TYPE == kIQ2_S) Fmt<kIQ2_S>::decode_stream(row, nu, rq, un, grid, u, D);
             } else {
                 Fmt<TYPE>::decode(blk, ib, grid, u);
                 D = Fmt<TYPE>::scale(blk);
@@ -643,12 +707,16 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+            // (stream packing: the row's quad and its place in it; the GGUF packing: the row itself)
+            // (only IQ2_S rows have a stream order; the other types' rows stay where GGUF puts them)
+            const bool pg = packed && TG == kIQ2_S, pu = packed && TU == kIQ2_S;
+            const int rq = r & 3;
             if constexpr (TG == TU) {
-                const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) r * grow;
-                row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc, packed);
+                const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) (pg ? (r & ~3) : r) * grow;
+                row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc, pg, rq);
             } else {
-                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) r * grow, k, sub, al, grid_g, acc, packed);
-                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) r * urow, k, sub, al, grid_u, acc, packed);
+                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) (pg ? (r & ~3) : r) * grow, k, sub, al, grid_g, acc, pg, rq);
+                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) (pu ? (r & ~3) : r) * urow, k, sub, al, grid_u, acc, pu, rq);
             }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -680,7 +748,7 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
     const uint8_t* base = (const uint8_t*) gr.blob + a.layout.down_off;
     const size_t drow = (size_t) (k / Fmt<TD>::kValues) * Fmt<TD>::kBytes;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
-    const bool packed = a.layout.packing == MAYA_PACK_STREAM;
+    const bool packed = a.layout.packing == MAYA_PACK_STREAM && TD == kIQ2_S;
     for (int c0 = 0; c0 < gr.ne; c0 += NT) {
         int ents[NT];
 #pragma unroll
@@ -693,7 +761,7 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
-            row_dot<TD, NT, 32>(base + (size_t) r * drow, k, sub, al, grid, acc, packed);
+            row_dot<TD, NT, 32>(base + (size_t) (packed ? (r & ~3) : r) * drow, k, sub, al, grid, acc, packed, r & 3);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const float s = group_sum<32>(acc[t]);
@@ -755,6 +823,8 @@ int check_layout(const maya_moe_layout& l) {
     if (l.n_embd <= 0 || l.n_ff <= 0 || l.n_embd % 256 || l.n_ff % 256)
         return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d: multiples of 256 wanted", l.n_embd, l.n_ff);
     if (l.packing != MAYA_PACK_GGUF && l.packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "packing %d", l.packing);
+    if (l.packing == MAYA_PACK_STREAM && (l.gate_off % 16 || l.up_off % 16 || l.down_off % 16))
+        return fail(MAYA_E_ARG, "stream packing wants 16-byte aligned row arrays");
     if (l.n_embd > 16384 || l.n_ff > 16384) return fail(MAYA_E_SHAPE, "n_embd %d / n_ff %d past 16384", l.n_embd, l.n_ff);
     return MAYA_OK;
 }
@@ -801,17 +871,10 @@ int tuning_variant(const char* name, int dflt) {
     return v && *v ? atoi(v) : dflt;
 }
 
-template <bool STREAM>
-int launch_gate_up_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+int launch_gate_up_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 32;
     const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) a.k);
-    static const int variant = tuning_variant("MAYA_GU_VARIANT", 0);
-#define MAYA_KU(N)                                                                                                                        \
-    case N:                                                                                                                               \
-        if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, true, false, 4, STREAM>), grid, dim3(512), 0, s, a, st.cb);  \
-        else if (variant == 3) hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, false, false, 4, STREAM>), grid, dim3(512), 0, s, a, st.cb); \
-        else hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, true, true, 1, STREAM>), grid, dim3(512), 0, s, a, st.cb);             \
-        break;
+#define MAYA_KU(N) case N: hipLaunchKernelGGL((gate_up_iq2s_1tok_kernel<N, kRows, true, false, 4, false>), grid, dim3(512), 0, s, a, st.cb); break;
     switch (a.layout.n_embd / 1024) {
         MAYA_KU(1) MAYA_KU(2) MAYA_KU(3) MAYA_KU(4) MAYA_KU(5) MAYA_KU(6) MAYA_KU(7) MAYA_KU(8)
     }
@@ -819,15 +882,33 @@ int launch_gate_up_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hi
     MAYA_LAUNCHED("gate_up_iq2s_1tok_kernel");
     return MAYA_OK;
 }
-int launch_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
-    return a.layout.packing == MAYA_PACK_STREAM ? launch_gate_up_iq2s_1tok_t<true>(a, st, s)
-                                                : launch_gate_up_iq2s_1tok_t<false>(a, st, s);
+// (MAYA_GU_VARIANT / MAYA_DN_VARIANT: tuning knobs for the row tile and the prefetch depth; unset = the measured best)
+template <int NW>
+int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    constexpr int kRows = 16;
+    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) a.k);
+    static const int variant = tuning_variant("MAYA_GU_VARIANT", 0);
+    if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 2, 5>), grid, dim3(64 * NW), 0, s, a, st.cb);
+    else if (variant == 2) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 32, 1, 8>), dim3(grid.x / 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
+    else if (variant == 3) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 8, 1, 8>), dim3(grid.x * 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
+    else hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 8>), grid, dim3(64 * NW), 0, s, a, st.cb);
+    MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
+    return MAYA_OK;
 }
-template <bool STREAM>
-int launch_down_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    constexpr int kRows = 16;
+    const dim3 grid((unsigned) (a.layout.n_embd / kRows));
+    static const int variant = tuning_variant("MAYA_DN_VARIANT", 0);
+    if (variant == 1) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 2, 5>), grid, dim3(512), 0, s, a, st.cb);
+    else if (variant == 2) hipLaunchKernelGGL((down_iq2s_pos_kernel<8, 1, 8>), dim3(grid.x * 2), dim3(512), 0, s, a, st.cb);
+    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 8>), grid, dim3(512), 0, s, a, st.cb);
+    MAYA_LAUNCHED("down_iq2s_pos_kernel");
+    return MAYA_OK;
+}
+int launch_down_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 14;
     const dim3 grid((unsigned) (a.layout.n_embd / kRows));
-#define MAYA_KU(N) case N: hipLaunchKernelGGL((down_iq2s_1tok_kernel<N, kRows, STREAM>), grid, dim3(512), 0, s, a, st.cb); break;
+#define MAYA_KU(N) case N: hipLaunchKernelGGL((down_iq2s_1tok_kernel<N, kRows, false>), grid, dim3(512), 0, s, a, st.cb); break;
     switch (a.layout.n_ff / 1024) {
         MAYA_KU(1) MAYA_KU(2) MAYA_KU(3) MAYA_KU(4)
     }
@@ -835,9 +916,43 @@ int launch_down_iq2s_1tok_t(const maya_moe_args& a, const DeviceState& st, hipSt
     MAYA_LAUNCHED("down_iq2s_1tok_kernel");
     return MAYA_OK;
 }
-int launch_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
-    return a.layout.packing == MAYA_PACK_STREAM ? launch_down_iq2s_1tok_t<true>(a, st, s)
-                                                : launch_down_iq2s_1tok_t<false>(a, st, s);
+
+// single-token IQ2_S gate/up: 1 launched, 0 no specialised kernel for this shape (the caller takes the general one)
+int try_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
+    const maya_moe_layout& l = a.layout;
+    if (l.packing == MAYA_PACK_STREAM) {
+        if (l.n_ff % 16 != 0) return 0;
+        switch (l.n_embd / 1024 * (l.n_embd % 1024 == 0)) {
+            case 4: *rc = launch_gate_up_iq2s_pos<4>(a, st, s); return 1;
+            case 6: *rc = launch_gate_up_iq2s_pos<6>(a, st, s); return 1;
+            case 7: *rc = launch_gate_up_iq2s_pos<7>(a, st, s); return 1;
+            case 8: *rc = launch_gate_up_iq2s_pos<8>(a, st, s); return 1;
+            default: return 0;
+        }
+    }
+    if (l.n_embd % 1024 != 0 || l.n_embd > 8192 || l.n_ff % 32 != 0) return 0;
+    *rc = launch_gate_up_iq2s_gguf(a, st, s);
+    return 1;
+}
+// whether try_gate_up_iq2s_1tok would take the position-mapped kernel, which can round h itself (hq_sync)
+bool gate_up_fuses_hq(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && fast_1tok(a) && l.packing == MAYA_PACK_STREAM)) return false;
+    if (l.n_ff % 256 != 0 || l.n_embd % 1024 != 0 || !q8k_act(l.down_type)) return false;
+    const int nw = l.n_embd / 1024;
+    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+}
+int try_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
+    const maya_moe_layout& l = a.layout;
+    if (a.k > 8) return 0;
+    if (l.packing == MAYA_PACK_STREAM) {
+        if (l.n_ff != 2048 || l.n_embd % 16 != 0) return 0;
+        *rc = launch_down_iq2s_pos(a, st, s);
+        return 1;
+    }
+    if (l.n_ff % 1024 != 0 || l.n_ff > 4096 || l.n_embd % 14 != 0) return 0;
+    *rc = launch_down_iq2s_gguf(a, st, s);
+    return 1;
 }
 
 }  // namespace maya
@@ -930,7 +1045,7 @@ int maya_dequant_rows_packed(int t, int packing, const void* w, size_t row_strid
     if (!type_ok(t)) return fail(MAYA_E_UNSUPPORTED, "dequant: type %d", t);
     if (packing != MAYA_PACK_GGUF && packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "dequant: packing %d", packing);
     if (!w || !out) return fail(MAYA_E_ARG, "dequant: null pointer");
-    if (k <= 0 || k % block_values(t) || n_rows <= 0 || n_rows > 65535)
+    if (k <= 0 || k % block_values(t) || n_rows <= 0 || n_rows > 65535 || (packing == MAYA_PACK_STREAM && n_rows % 4))
         return fail(MAYA_E_SHAPE, "dequant: k %lld rows %lld", (long long) k, (long long) n_rows);
     if (row_stride == 0) row_stride = maya_moe_row_bytes(t, k);
     const dim3 grid((unsigned) ((k + 255) / 256), (unsigned) n_rows);
@@ -1036,9 +1151,10 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
     hipStream_t s = as_stream(stream);
     const int tg = a->layout.gate_type, tu = a->layout.up_type;
-    if (tg == kIQ2_S && tu == kIQ2_S && fast_1tok(*a) && a->layout.n_embd % 1024 == 0 && a->layout.n_embd <= 8192 &&
-        a->layout.n_ff % 32 == 0)
-        return launch_gate_up_iq2s_1tok(*a, *st, s);
+    if (tg == kIQ2_S && tu == kIQ2_S && fast_1tok(*a)) {
+        int rc = 0;
+        if (try_gate_up_iq2s_1tok(*a, *st, s, &rc)) return rc;
+    }
 #define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
     MAYA_GU(kIQ2_S, kIQ2_S)
     MAYA_GU(kQ4_K, kQ4_K)
@@ -1054,15 +1170,18 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     return fail(MAYA_E_UNSUPPORTED, "gate_up: no kernel for gate type %d with up type %d", tg, tu);
 }
 
+int maya_moe_gate_up_fuses_hq(const maya_moe_args* a) { return a && a->hq_sync && gate_up_fuses_hq(*a) ? 1 : 0; }
+
 int maya_moe_down(const maya_moe_args* a, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (const int rc = check_args(a)) return rc;
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
     hipStream_t s = as_stream(stream);
-    if (a->layout.down_type == kIQ2_S && fast_1tok(*a) && a->k <= 8 && a->layout.n_ff % 1024 == 0 && a->layout.n_ff <= 4096 &&
-        a->layout.n_embd % 14 == 0)
-        return launch_down_iq2s_1tok(*a, *st, s);
+    if (a->layout.down_type == kIQ2_S && fast_1tok(*a)) {
+        int rc = 0;
+        if (try_down_iq2s_1tok(*a, *st, s, &rc)) return rc;
+    }
     int rc;
     switch (a->layout.down_type) {
         case kIQ2_S: rc = launch_down_t<kIQ2_S>(*a, *st, s); break;
@@ -1081,7 +1200,7 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
 // workspace carve-up of maya_moe_layer_decode (every region 256-byte aligned)
 struct LayerWs {
     uint64_t *plan_ptr, *grp_ptr;
-    int32_t *grp_start, *grp_ent, *n_groups;
+    int32_t *grp_start, *grp_ent, *n_groups, *hq_sync;
     maya_act x, hq;
     float *h, *part;
     size_t bytes;
@@ -1100,6 +1219,7 @@ static LayerWs carve(const maya_moe_layout& l, int n_tokens, int k, uint8_t* bas
     w.grp_start = (int32_t*) take(sizeof(int32_t) * (ne + 1));
     w.grp_ent = (int32_t*) take(sizeof(int32_t) * ne);
     w.n_groups = (int32_t*) take(sizeof(int32_t));
+    w.hq_sync = (int32_t*) take(sizeof(int32_t) * (size_t) ne * (l.n_ff / 256));
     w.x.q = (int8_t*) take((size_t) n_tokens * l.n_embd);
     w.x.d = (float*) take(sizeof(float) * (size_t) n_tokens * (l.n_embd / 32));
     w.x.bsums = (int16_t*) take(sizeof(int16_t) * (size_t) n_tokens * (l.n_embd / 16));
@@ -1131,21 +1251,12 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
     const LayerWs w = carve(*l, n_tokens, k, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "layer_decode: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     int rc;
-    if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
-    if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
     maya_moe_args a{};
     a.layout = *l;
     a.n_tokens = n_tokens;
     a.k = k;
     a.plan_ptr = w.plan_ptr;
     a.plan_w = weights;
-    if (n_tokens > 1) {
-        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
-        a.grp_ptr = w.grp_ptr;
-        a.grp_start = w.grp_start;
-        a.grp_ent = w.grp_ent;
-        a.n_groups = w.n_groups;
-    }
     a.limit = limit;
     a.x = w.x;
     a.h = w.h;
@@ -1153,9 +1264,34 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
     a.part = w.part;
     a.add = add;
     a.out = out;
-    if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
+    if (q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
+        // one launch: route, plan, Q8_K of x, cleared counters
+        const int n_counters = n_tokens * k * (l->n_ff / 256);
+        const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
+        hipStream_t s = as_stream(stream);
+        if (k > n_expert) return fail(MAYA_E_SHAPE, "layer_decode: k %d > n_expert %d", k, n_expert);
+        switch (x_dtype) {
+            case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+        }
+        MAYA_LAUNCHED("layer_head_kernel");
+        a.hq_sync = w.hq_sync;
+    } else {
+        if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+        if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+        if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
+    }
+    if (n_tokens > 1) {
+        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
+        a.grp_ptr = w.grp_ptr;
+        a.grp_start = w.grp_start;
+        a.grp_ent = w.grp_ent;
+        a.n_groups = w.n_groups;
+    }
     if ((rc = maya_moe_gate_up(&a, stream))) return rc;
-    if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
+    if (!maya_moe_gate_up_fuses_hq(&a))
+        if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
     return maya_moe_down(&a, stream);
 }
 

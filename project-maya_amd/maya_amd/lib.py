@@ -18,7 +18,7 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack",
-    "maya_dequant_rows_packed",
+    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq",
 ]
 
 
@@ -42,7 +42,8 @@ class Args(C.Structure):
     _fields_ = [("layout", Layout), ("n_tokens", C.c_int32), ("k", C.c_int32), ("plan_ptr", C.c_void_p),
                 ("plan_w", C.c_void_p), ("grp_ptr", C.c_void_p), ("grp_start", C.c_void_p), ("grp_ent", C.c_void_p),
                 ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", Act), ("h", C.c_void_p),
-                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p)]
+                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p),
+                ("hq_sync", C.c_void_p)]
 
 
 _lib = None
@@ -74,6 +75,7 @@ def load():
     L.maya_moe_group.argtypes = [vp, i32, vp, vp, vp, vp, vp]
     L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
+    L.maya_moe_gate_up_fuses_hq.argtypes = [C.POINTER(Args)]
     L.maya_moe_workspace_bytes.restype = sz
     L.maya_moe_workspace_bytes.argtypes = [C.POINTER(Layout), i32, i32]
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
