@@ -187,6 +187,61 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
                           int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/* ================================================================================================ EXL3
+ * EXL3 (exllamav3) trellis weights: a matrix with k inputs and n outputs is `trellis` uint32 [k/16][n/16][4*k2]
+ * (16x16 tiles, 16*k2 bytes each, k2 = twice the bits per weight), FP16 `suh` [k] and `svh` [n];
+ *   y = H(H(x * suh) W') * svh,   H = the 128-point Sylvester-Hadamard transform over sqrt(128), per 128 values,
+ * W' decoded from each tile's 256 16-bit trellis states (include/strata/kernels/exl3.hpp:4-22). */
+#define MAYA_TYPE_EXL3 200 /* exl3::kTypeEXL3 (include/strata/kernels/exl3.hpp:32) */
+
+/* One routed expert's blob: exl3::ExpertLayout (include/strata/kernels/exl3.hpp:96-103): for each of gate, up, down the
+ * byte offsets of its suh, svh and trellis from the blob base (trellis 4-byte aligned, suh / svh 2-byte), its k2, and
+ * the codebook (0 3inst, 1 mcg, 2 mul1). */
+typedef struct maya_exl3_layout {
+    uint64_t suh[3], svh[3], trellis[3];
+    int32_t k2[3];
+    int32_t cb;
+    int32_t n_embd, n_ff; /* multiples of 128 */
+} maya_exl3_layout;
+
+/* exl3::MoeArgs / exl3::WinArgs (include/strata/kernels/exl3.hpp:118-168): the routed experts of n_tokens tokens,
+ * entry e = token e / k, slot e % k; groups as in maya_moe_args (NULL grp_ptr: group g = entry g). */
+typedef struct maya_exl3_args {
+    maya_exl3_layout layout;
+    int32_t n_tokens, k;
+    const uint64_t* plan_ptr;
+    const float* plan_w;
+    const uint64_t* grp_ptr;
+    const int32_t* grp_start;
+    const int32_t* grp_ent;
+    const int32_t* n_groups;
+    const int32_t* skip;
+    float limit;        /* SwiGLU clamp; 0 or +inf: none */
+    const float* x;     /* [n_tokens][x_stride] F32 */
+    int64_t x_stride;   /* floats between tokens (0: n_embd) */
+    float* h;           /* [n_tokens*k][n_ff] */
+    float* part;        /* [n_tokens*k][n_embd] */
+    const float* add;   /* NULL or [n_tokens][n_embd] (shared expert / CPU lane part) */
+    const int32_t* add_flag;
+    float* out;         /* [n_tokens][n_embd] */
+} maya_exl3_args;
+
+/* exl3::k2_supported (include/strata/kernels/exl3.hpp:56-58) */
+int maya_exl3_supported(int k2, int cb);
+/* bytes of a k x n trellis at k2: exl3::trellis_bytes_k2 (exl3.hpp:50-52) */
+size_t maya_exl3_trellis_bytes(int64_t k, int64_t n, int k2);
+/* the decoded W' [k][n] as FP16 bits, exactly the codebook's values: exl3::reconstruct_inner (exl3.hpp:213-214) */
+int maya_exl3_reconstruct_inner(const uint32_t* trellis, int64_t k, int64_t n, int k2, int cb, uint16_t* dst, void* stream);
+/* exl3::moe_gate_up / moe_down / win_experts (exl3.hpp:133-169): h = clamped swiglu of the gate and up products;
+ * part[e] = the down product of h[e]; out[t] = sum_i plan_w * part in slot order (+ add). */
+int maya_exl3_gate_up(const maya_exl3_args* a, void* stream);
+int maya_exl3_down(const maya_exl3_args* a, void* stream);
+/* route -> plan -> group -> gate/up -> down -> combine for n_tokens <= MAYA_MAX_TOKENS tokens, all on `stream` */
+size_t maya_exl3_workspace_bytes(const maya_exl3_layout* l, int n_tokens, int k);
+int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
+                           const float* x, int n_tokens, float limit, const float* add, int32_t* ids, float* weights,
+                           float* out, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

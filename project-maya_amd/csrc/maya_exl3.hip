@@ -1,0 +1,453 @@
+// maya_exl3.hip - EXL3 (exllamav3 trellis) routed experts on gfx950: decode mat-vec kernels and their C ABI.
+//
+// A workgroup owns 128 output columns (one block of the output Hadamard transform): its 8 waves take one 16-column
+// tile each and walk down the k / 16 row tiles.  For a tile a lane decodes 4 consecutive trellis steps - by the tile's
+// element order (include/strata/kernels/exl3.hpp:15-16) those are 4 rows of ONE column - and multiplies them with the
+// rotated, FP16-rounded activation held in LDS; the rotation H(x * suh) is done by the workgroup itself before the walk
+// and the output rotation, the svh scaling, the SwiGLU and the FP32 stores after it.  Several activations (a verify
+// window's tokens routed to one expert) share one decode of the weights.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <math.h>
+#include <stdint.h>
+
+#include "maya_host.h"
+
+namespace maya {
+
+constexpr int kExThreads = 512;
+
+// ---- codebooks: the value of a 16-bit state, as the FP16 bits the format defines (src/kernels/cpu/exl3_ref.cpp:11-27)
+template <int CB>
+__device__ __forceinline__ __half exl3_value(uint32_t state) {
+    if constexpr (CB == 2) {
+        // fp16(1024 + bytesum(state * 0x83DCD12D)) * fp16(0x1eee) + fp16(0xc931) in one FP16 FMA
+        const uint32_t x = state * 0x83DCD12Du;
+        const uint32_t bs = __builtin_amdgcn_sad_u8(x, 0u, 1024u);   // 1024 + the sum of the four bytes
+        const __half h = __ushort2half_rn((unsigned short) bs);      // exact: an integer below 2048
+        return __hfma(h, __ushort_as_half(0x1eee), __ushort_as_half(0xc931));
+    } else {
+        uint32_t x = CB == 1 ? state * 0xCBAC1FEDu : state * 89226354u + 64248484u;
+        x = (x & 0x8fff8fffu) ^ 0x3b603b60u;
+        return __hadd(__ushort_as_half((unsigned short) (x & 0xffffu)), __ushort_as_half((unsigned short) (x >> 16)));
+    }
+}
+
+// step p's state of a tile whose 4 * k2 words are in t[] (LDS or registers): the 16-bit window that ends at bit
+// floor((p + 1) k2 / 2) of the words read MSB-first, around the ring (src/kernels/cpu/exl3_ref.cpp:33-43)
+__device__ __forceinline__ uint32_t exl3_state(const uint32_t* t, int k2, int p) {
+    const int W = 4 * k2;
+    const int e = ((p + 1) * k2) >> 1;            // the window's end bit, 1 .. 128 k2
+    const int i1 = (e - 1) >> 5;                  // the word of its last bit
+    const int i0 = e < 16 ? W - 1 : (e - 16) >> 5;  // ... of its first bit (before bit 0: the ring's last word)
+    const int sh = ((i1 + 1) << 5) - e;
+    const uint64_t m = ((uint64_t) t[i0] << 32) | (uint64_t) t[i1];
+    return (uint32_t) (m >> sh) & 0xffffu;
+}
+
+// tile step p -> (row, column) inside the 16 x 16 tile (src/kernels/cpu/exl3_ref.cpp:52-55)
+__device__ __forceinline__ void exl3_rc(int p, int& r, int& c) {
+    const int lane = p >> 3, j = p & 7;
+    r = (lane & 3) * 2 + (j & 1) + 8 * ((j >> 1) & 1);
+    c = (lane >> 2) + 8 * (j >> 2);
+}
+
+template <int CB>
+__global__ __launch_bounds__(256) void exl3_inner_kernel(const uint32_t* __restrict__ trellis, int64_t k, int64_t n, int k2,
+                                                         uint16_t* __restrict__ dst) {
+    __shared__ uint32_t t[64];
+    const int64_t tiles_n = n >> 4;
+    const int64_t tile = blockIdx.x;
+    const int W = 4 * k2;
+    if ((int) threadIdx.x < W) t[threadIdx.x] = trellis[tile * W + threadIdx.x];
+    __syncthreads();
+    const int p = threadIdx.x;
+    int r, c;
+    exl3_rc(p, r, c);
+    const __half v = exl3_value<CB>(exl3_state(t, k2, p));
+    const int64_t ks = tile / tiles_n, tc = tile % tiles_n;
+    dst[(ks * 16 + r) * n + tc * 16 + c] = __half_as_ushort(v);
+}
+
+// ---- the blockwise Hadamard transform of LDS data: v holds nb blocks of 128 floats; every thread of the workgroup calls
+// it.  The butterflies and their order are the reference's (src/kernels/cpu/exl3_ref.cpp:61-75): the same bits.
+__device__ __forceinline__ void had128_lds(float* v, int nb) {
+    for (int h = 1; h < 128; h <<= 1) {
+        for (int idx = threadIdx.x; idx < nb * 64; idx += kExThreads) {
+            const int blk = idx >> 6, j = idx & 63;
+            const int lo = blk * 128 + (j / h) * 2 * h + (j % h);
+            const float a = v[lo], c = v[lo + h];
+            v[lo] = __fadd_rn(a, c);
+            v[lo + h] = __fsub_rn(a, c);
+        }
+        __syncthreads();
+    }
+    const float s = 1.0f / sqrtf(128.0f);
+    for (int i = threadIdx.x; i < nb * 128; i += kExThreads) v[i] = __fmul_rn(v[i], s);
+    __syncthreads();
+}
+
+struct ExGroup {
+    uint64_t blob;
+    int e0, ne;
+};
+__device__ __forceinline__ bool ex_group_of(const maya_exl3_args& a, int g, ExGroup& r) {
+    if (a.skip && *a.skip) return false;
+    if (a.grp_ptr) {
+        if (g >= *a.n_groups) return false;
+        r.blob = a.grp_ptr[g];
+        r.e0 = a.grp_start[g];
+        r.ne = a.grp_start[g + 1] - r.e0;
+    } else {
+        if (g >= a.n_tokens * a.k) return false;
+        r.blob = a.plan_ptr[g];
+        r.e0 = g;
+        r.ne = 1;
+    }
+    return r.blob != 0ull && r.ne > 0;
+}
+__device__ __forceinline__ int ex_entry_of(const maya_exl3_args& a, const ExGroup& r, int i) {
+    return a.grp_ptr ? a.grp_ent[r.e0 + i] : r.e0;
+}
+
+// xr = FP16(H(x * suh)) of one activation into LDS (as FP16 pairs); `tmp` is k floats of LDS scratch
+__device__ __forceinline__ void rotate_in(const float* __restrict__ x, const uint16_t* __restrict__ suh, int k, float* tmp,
+                                          __half* xr) {
+    for (int i = threadIdx.x; i < k; i += kExThreads) tmp[i] = __fmul_rn(x[i], f16_bits_to_f32(suh[i]));
+    __syncthreads();
+    had128_lds(tmp, k >> 7);
+    for (int i = threadIdx.x; i < k; i += kExThreads) xr[i] = __float2half_rn(tmp[i]);
+    __syncthreads();
+}
+
+// One matrix's 16-column tile over all its row tiles for NT activations: returns this lane's partial sums for its column
+// (the lane's 4 steps are rows 2q, 2q+1, 2q+8, 2q+9 of column (L >> 3) + 8 (L & 1), q = (L >> 1) & 3)
+template <int CB, int NT>
+__device__ __forceinline__ void walk_tiles(const uint32_t* __restrict__ trellis, int k, int ld, int tc, int k2, int lane,
+                                           uint32_t* wt, const __half* xr, int xr_stride, float (&acc)[NT]) {
+    const int W = 4 * k2, q = (lane >> 1) & 3;
+    for (int ks = 0; ks < (k >> 4); ++ks) {
+        const uint32_t* tile = trellis + ((size_t) ks * ld + tc) * W;
+        if (lane < W) wt[lane] = tile[lane];
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0);  // the wave's own LDS writes have landed before any lane reads them
+        float w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = __half2float(exl3_value<CB>(exl3_state(wt, k2, 4 * lane + i)));
+        __builtin_amdgcn_wave_barrier();
+        const int rb = ks * 16 + 2 * q;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const __half* xv = xr + t * xr_stride + rb;
+            float s = acc[t];
+            s = fmaf(w[0], __half2float(xv[0]), s);
+            s = fmaf(w[1], __half2float(xv[1]), s);
+            s = fmaf(w[2], __half2float(xv[8]), s);
+            s = fmaf(w[3], __half2float(xv[9]), s);
+            acc[t] = s;
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {  // the 4 lanes of a column: q = bits 1, 2 of the lane
+        acc[t] += __shfl_xor(acc[t], 2, 64);
+        acc[t] += __shfl_xor(acc[t], 4, 64);
+    }
+}
+
+__device__ __forceinline__ float ex_swiglu(float g, float u, float limit) {
+    if (limit > 0.0f && limit < INFINITY) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
+}
+
+// dynamic LDS: [8 waves x 64 words of tile][NT x 2 x k halves of rotated inputs][max(k, NT*2*128) floats of scratch]
+// grid (n_ff / 128, groups)
+template <int CB, int NT>
+__global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args a) {
+    extern __shared__ uint32_t lds[];
+    ExGroup gr;
+    if (!ex_group_of(a, blockIdx.y, gr)) return;
+    const int k = a.layout.n_embd, n = a.layout.n_ff;
+    uint32_t* wt = lds + (threadIdx.x >> 6) * 64;
+    __half* xr = (__half*) (lds + 8 * 64);                       // [NT][2][k]
+    float* tmp = (float*) (xr + (size_t) NT * 2 * k);            // k floats; later the raw outputs [NT][2][128]
+    const uint8_t* blob = (const uint8_t*) gr.blob;
+    const int64_t xs = a.x_stride ? a.x_stride : k;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tc = blockIdx.x * 8 + wave;
+    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
+        int ents[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? ex_entry_of(a, gr, c0 + t) : -1;
+        __syncthreads();
+        for (int t = 0; t < NT; ++t) {
+            if (ents[t] < 0) continue;
+            const float* x = a.x + (size_t) (ents[t] / a.k) * xs;
+            for (int role = 0; role < 2; ++role)
+                rotate_in(x, (const uint16_t*) (blob + a.layout.suh[role]), k, tmp, xr + ((size_t) t * 2 + role) * k);
+        }
+        float raw[2][NT];
+#pragma unroll
+        for (int role = 0; role < 2; ++role) {
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+            walk_tiles<CB, NT>((const uint32_t*) (blob + a.layout.trellis[role]), k, n >> 4, tc, a.layout.k2[role], lane, wt,
+                               xr + (size_t) role * k, 2 * k, acc);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) raw[role][t] = acc[t];
+        }
+        __syncthreads();
+        // the lane with q = 0 of each column holds the sums: column (L >> 3) + 8 (L & 1) of the wave's tile
+        if (((lane >> 1) & 3) == 0) {
+            const int col = wave * 16 + (lane >> 3) + 8 * (lane & 1);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                tmp[(t * 2 + 0) * 128 + col] = raw[0][t];
+                tmp[(t * 2 + 1) * 128 + col] = raw[1][t];
+            }
+        }
+        __syncthreads();
+        had128_lds(tmp, NT * 2);
+        const uint16_t* svg = (const uint16_t*) (blob + a.layout.svh[0]) + blockIdx.x * 128;
+        const uint16_t* svu = (const uint16_t*) (blob + a.layout.svh[1]) + blockIdx.x * 128;
+        for (int i = threadIdx.x; i < NT * 128; i += kExThreads) {
+            const int t = i >> 7, c = i & 127;
+            if (ents[t] < 0) continue;
+            const float g = __fmul_rn(tmp[(t * 2 + 0) * 128 + c], f16_bits_to_f32(svg[c]));
+            const float u = __fmul_rn(tmp[(t * 2 + 1) * 128 + c], f16_bits_to_f32(svu[c]));
+            a.h[(size_t) ents[t] * n + blockIdx.x * 128 + c] = ex_swiglu(g, u, a.limit);
+        }
+    }
+}
+
+// grid (n_embd / 128, groups): part[e][columns] = the down product of h[e]
+template <int CB, int NT>
+__global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a) {
+    extern __shared__ uint32_t lds[];
+    ExGroup gr;
+    if (!ex_group_of(a, blockIdx.y, gr)) return;
+    const int k = a.layout.n_ff, n = a.layout.n_embd;
+    uint32_t* wt = lds + (threadIdx.x >> 6) * 64;
+    __half* xr = (__half*) (lds + 8 * 64);             // [NT][k]
+    float* tmp = (float*) (xr + (size_t) NT * k);      // k floats; later [NT][128]
+    const uint8_t* blob = (const uint8_t*) gr.blob;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tc = blockIdx.x * 8 + wave;
+    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
+        int ents[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? ex_entry_of(a, gr, c0 + t) : -1;
+        __syncthreads();
+        for (int t = 0; t < NT; ++t)
+            if (ents[t] >= 0)
+                rotate_in(a.h + (size_t) ents[t] * k, (const uint16_t*) (blob + a.layout.suh[2]), k, tmp, xr + (size_t) t * k);
+        float acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+        walk_tiles<CB, NT>((const uint32_t*) (blob + a.layout.trellis[2]), k, n >> 4, tc, a.layout.k2[2], lane, wt, xr, k, acc);
+        __syncthreads();
+        if (((lane >> 1) & 3) == 0) {
+            const int col = wave * 16 + (lane >> 3) + 8 * (lane & 1);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) tmp[t * 128 + col] = acc[t];
+        }
+        __syncthreads();
+        had128_lds(tmp, NT);
+        const uint16_t* sv = (const uint16_t*) (blob + a.layout.svh[2]) + blockIdx.x * 128;
+        for (int i = threadIdx.x; i < NT * 128; i += kExThreads) {
+            const int t = i >> 7, c = i & 127;
+            if (ents[t] < 0) continue;
+            a.part[(size_t) ents[t] * n + blockIdx.x * 128 + c] = __fmul_rn(tmp[t * 128 + c], f16_bits_to_f32(sv[c]));
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void exl3_combine_kernel(maya_exl3_args a) {
+    if (a.skip && *a.skip) return;
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x, n = a.layout.n_embd;
+    if (c >= n) return;
+    float sum = 0.0f;
+    bool first = true;
+    for (int i = 0; i < a.k; ++i) {
+        const int e = t * a.k + i;
+        if (a.plan_ptr[e] == 0ull) continue;
+        const float p = __fmul_rn(a.part[(size_t) e * n + c], a.plan_w[e]);
+        sum = first ? p : __fadd_rn(sum, p);
+        first = false;
+    }
+    if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[(size_t) t * n + c]);
+    a.out[(size_t) t * n + c] = sum;
+}
+
+bool exl3_k2_ok(int k2, int cb) {
+    return (k2 >= 2 && k2 <= 16 && (k2 & 1) == 0 && cb >= 0 && cb <= 2) || ((k2 == 3 || k2 == 5 || k2 == 7) && cb == 2);
+}
+int exl3_check(const maya_exl3_args* a) {
+    if (!a) return fail(MAYA_E_ARG, "exl3: null args");
+    const maya_exl3_layout& l = a->layout;
+    for (int r = 0; r < 3; ++r)
+        if (!exl3_k2_ok(l.k2[r], l.cb)) return fail(MAYA_E_UNSUPPORTED, "exl3: k2 %d with codebook %d", l.k2[r], l.cb);
+    if (l.n_embd <= 0 || l.n_ff <= 0 || l.n_embd % 128 || l.n_ff % 128 || l.n_embd > 16384 || l.n_ff > 16384)
+        return fail(MAYA_E_SHAPE, "exl3: n_embd %d / n_ff %d: multiples of 128 up to 16384 wanted", l.n_embd, l.n_ff);
+    for (int r = 0; r < 3; ++r)
+        if (l.trellis[r] % 4 || l.suh[r] % 2 || l.svh[r] % 2) return fail(MAYA_E_ARG, "exl3: misaligned part offsets");
+    if (a->n_tokens < 1 || a->n_tokens > MAYA_MAX_TOKENS || a->k < 1 || a->k > MAYA_MAX_K)
+        return fail(MAYA_E_SHAPE, "exl3: n_tokens %d / k %d", a->n_tokens, a->k);
+    if (!a->plan_ptr || !a->plan_w) return fail(MAYA_E_ARG, "exl3: null plan");
+    if (a->grp_ptr && (!a->grp_start || !a->grp_ent || !a->n_groups)) return fail(MAYA_E_ARG, "exl3: incomplete groups");
+    return MAYA_OK;
+}
+
+template <int NT>
+int launch_exl3_gate_up(const maya_exl3_args& a, const DeviceState& st, hipStream_t s) {
+    const int k = a.layout.n_embd;
+    const size_t scratch = (size_t) (k > NT * 256 ? k : NT * 256) * 4;
+    const size_t lds = 8 * 64 * 4 + (size_t) NT * 2 * k * 2 + scratch;
+    if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    const dim3 grid((unsigned) (a.layout.n_ff / 128), (unsigned) (a.n_tokens * a.k));
+#define MAYA_EX(CBV)                                                                                              \
+    {                                                                                                             \
+        auto kern = exl3_gate_up_kernel<CBV, NT>;                                                                 \
+        if (lds > 65536) MAYA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+        hipLaunchKernelGGL(kern, grid, dim3(kExThreads), lds, s, a);                                              \
+    }
+    if (a.layout.cb == 2) MAYA_EX(2) else if (a.layout.cb == 1) MAYA_EX(1) else MAYA_EX(0)
+#undef MAYA_EX
+    MAYA_LAUNCHED("exl3_gate_up_kernel");
+    return MAYA_OK;
+}
+template <int NT>
+int launch_exl3_down(const maya_exl3_args& a, const DeviceState& st, hipStream_t s) {
+    const int k = a.layout.n_ff;
+    const size_t scratch = (size_t) (k > NT * 128 ? k : NT * 128) * 4;
+    const size_t lds = 8 * 64 * 4 + (size_t) NT * k * 2 + scratch;
+    if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    const dim3 grid((unsigned) (a.layout.n_embd / 128), (unsigned) (a.n_tokens * a.k));
+#define MAYA_EX(CBV)                                                                                              \
+    {                                                                                                             \
+        auto kern = exl3_down_kernel<CBV, NT>;                                                                    \
+        if (lds > 65536) MAYA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+        hipLaunchKernelGGL(kern, grid, dim3(kExThreads), lds, s, a);                                              \
+    }
+    if (a.layout.cb == 2) MAYA_EX(2) else if (a.layout.cb == 1) MAYA_EX(1) else MAYA_EX(0)
+#undef MAYA_EX
+    MAYA_LAUNCHED("exl3_down_kernel");
+    return MAYA_OK;
+}
+
+}  // namespace maya
+
+using namespace maya;
+
+extern "C" {
+
+int maya_exl3_supported(int k2, int cb) { return exl3_k2_ok(k2, cb) ? 1 : 0; }
+size_t maya_exl3_trellis_bytes(int64_t k, int64_t n, int k2) { return (size_t) (k / 16) * (size_t) (n / 16) * 16u * (size_t) k2; }
+
+int maya_exl3_reconstruct_inner(const uint32_t* trellis, int64_t k, int64_t n, int k2, int cb, uint16_t* dst, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!exl3_k2_ok(k2, cb)) return fail(MAYA_E_UNSUPPORTED, "exl3: k2 %d with codebook %d", k2, cb);
+    if (!trellis || !dst) return fail(MAYA_E_ARG, "exl3 reconstruct: null pointer");
+    if (k <= 0 || n <= 0 || k % 16 || n % 16) return fail(MAYA_E_SHAPE, "exl3 reconstruct: k %lld n %lld", (long long) k, (long long) n);
+    const dim3 grid((unsigned) ((k / 16) * (n / 16)));
+    hipStream_t s = as_stream(stream);
+    if (cb == 2) hipLaunchKernelGGL(exl3_inner_kernel<2>, grid, dim3(256), 0, s, trellis, k, n, k2, dst);
+    else if (cb == 1) hipLaunchKernelGGL(exl3_inner_kernel<1>, grid, dim3(256), 0, s, trellis, k, n, k2, dst);
+    else hipLaunchKernelGGL(exl3_inner_kernel<0>, grid, dim3(256), 0, s, trellis, k, n, k2, dst);
+    MAYA_LAUNCHED("exl3_inner_kernel");
+    return MAYA_OK;
+}
+
+int maya_exl3_gate_up(const maya_exl3_args* a, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (const int rc = exl3_check(a)) return rc;
+    if (!a->x || !a->h) return fail(MAYA_E_ARG, "exl3 gate_up: null x or h");
+    const int nt = a->grp_ptr && a->n_tokens >= 2 ? 2 : 1;
+    return nt == 2 ? launch_exl3_gate_up<2>(*a, *st, as_stream(stream)) : launch_exl3_gate_up<1>(*a, *st, as_stream(stream));
+}
+
+int maya_exl3_down(const maya_exl3_args* a, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (const int rc = exl3_check(a)) return rc;
+    if (!a->h || !a->part || !a->out) return fail(MAYA_E_ARG, "exl3 down: null h, part or out");
+    const int nt = a->grp_ptr && a->n_tokens >= 2 ? 2 : 1;
+    const int rc = nt == 2 ? launch_exl3_down<2>(*a, *st, as_stream(stream)) : launch_exl3_down<1>(*a, *st, as_stream(stream));
+    if (rc) return rc;
+    const dim3 grid((unsigned) ((a->layout.n_embd + 255) / 256), (unsigned) a->n_tokens);
+    hipLaunchKernelGGL(exl3_combine_kernel, grid, dim3(256), 0, as_stream(stream), *a);
+    MAYA_LAUNCHED("exl3_combine_kernel");
+    return MAYA_OK;
+}
+
+struct Exl3Ws {
+    uint64_t *plan_ptr, *grp_ptr;
+    int32_t *grp_start, *grp_ent, *n_groups;
+    float *h, *part;
+    size_t bytes;
+};
+static Exl3Ws exl3_carve(const maya_exl3_layout& l, int n_tokens, int k, uint8_t* base) {
+    Exl3Ws w{};
+    size_t off = 0;
+    const int ne = n_tokens * k;
+    auto take = [&](size_t n) {
+        uint8_t* p = base ? base + off : nullptr;
+        off += (n + 255) & ~(size_t) 255;
+        return p;
+    };
+    w.plan_ptr = (uint64_t*) take(sizeof(uint64_t) * ne);
+    w.grp_ptr = (uint64_t*) take(sizeof(uint64_t) * ne);
+    w.grp_start = (int32_t*) take(sizeof(int32_t) * (ne + 1));
+    w.grp_ent = (int32_t*) take(sizeof(int32_t) * ne);
+    w.n_groups = (int32_t*) take(sizeof(int32_t));
+    w.h = (float*) take(sizeof(float) * (size_t) ne * l.n_ff);
+    w.part = (float*) take(sizeof(float) * (size_t) ne * l.n_embd);
+    w.bytes = off;
+    return w;
+}
+size_t maya_exl3_workspace_bytes(const maya_exl3_layout* l, int n_tokens, int k) {
+    if (!l || n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K || l->n_embd <= 0 || l->n_ff <= 0) return 0;
+    return exl3_carve(*l, n_tokens, k, nullptr).bytes;
+}
+
+int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
+                           const float* x, int n_tokens, float limit, const float* add, int32_t* ids, float* weights,
+                           float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!l || !expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "exl3 layer: null pointer");
+    if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K) return fail(MAYA_E_SHAPE, "exl3 layer: n_tokens %d / k %d", n_tokens, k);
+    if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "exl3 layer: workspace not 256-byte aligned");
+    const Exl3Ws w = exl3_carve(*l, n_tokens, k, (uint8_t*) workspace);
+    if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "exl3 layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
+    int rc;
+    if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+    if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+    maya_exl3_args a{};
+    a.layout = *l;
+    a.n_tokens = n_tokens;
+    a.k = k;
+    a.plan_ptr = w.plan_ptr;
+    a.plan_w = weights;
+    if (n_tokens > 1) {
+        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
+        a.grp_ptr = w.grp_ptr;
+        a.grp_start = w.grp_start;
+        a.grp_ent = w.grp_ent;
+        a.n_groups = w.n_groups;
+    }
+    a.limit = limit;
+    a.x = x;
+    a.h = w.h;
+    a.part = w.part;
+    a.add = add;
+    a.out = out;
+    if ((rc = maya_exl3_gate_up(&a, stream))) return rc;
+    return maya_exl3_down(&a, stream);
+}
+
+}  // extern "C"

@@ -17,8 +17,7 @@
 
 #include <mutex>
 
-#include "../../include/maya_moe.h"
-#include "maya_dev.cuh"
+#include "maya_host.h"
 #include "maya_iq_grids.h"
 
 namespace maya {
@@ -26,7 +25,6 @@ namespace maya {
 // ------------------------------------------------------------------------------------------------ host state
 
 thread_local char g_err[512] = "";
-int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail(int code, const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -38,23 +36,8 @@ int hip_fail(hipError_t e, const char* what) {
     snprintf(g_err, sizeof g_err, "%s: %s", what, hipGetErrorString(e));
     return -(int) e;
 }
-#define MAYA_HIP(call)                                         \
-    do {                                                       \
-        const hipError_t e_ = (call);                          \
-        if (e_ != hipSuccess) return hip_fail(e_, #call);      \
-    } while (0)
-#define MAYA_LAUNCHED(name)                                    \
-    do {                                                       \
-        const hipError_t e_ = hipGetLastError();               \
-        if (e_ != hipSuccess) return hip_fail(e_, name);       \
-    } while (0)
 
 constexpr int kMaxDevices = 16;
-struct DeviceState {
-    bool ready = false;
-    Codebooks cb{};
-    int lds_limit = 65536;
-};
 DeviceState g_dev[kMaxDevices];
 std::mutex g_init_mu;
 
@@ -90,6 +73,7 @@ int current_state(DeviceState** out) {
             s.cb.iq2s = d;
             s.cb.iq1s = d + 1024;
             s.lds_limit = (int) p.sharedMemPerBlock;
+            s.n_cu = p.multiProcessorCount;
             s.ready = true;
         }
     }
@@ -97,7 +81,6 @@ int current_state(DeviceState** out) {
     return MAYA_OK;
 }
 
-inline hipStream_t as_stream(void* s) { return (hipStream_t) s; }
 
 // ------------------------------------------------------------------------------------------------ dequantize
 //
