@@ -187,6 +187,56 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
                           int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/* ============================================================================================= prefill
+ * A prompt chunk's routed experts as a grouped GEMM (the reference's expert_count_kernel / expert_scatter_kernel,
+ * src/kernels/cuda/glm_batch.cu:2102-2133, with the host's prefix sum of src/prefill/glm_prefill.cu:3339-3361 done on
+ * the device; mmq::quantize / Context::run / run_glu, src/kernels/cuda/moe_mmq.cu:120-228; the per-32 int8 activation
+ * format of src/prefill/moe_fused_rdna4.cu:87-109 and its requantized H, :620-660).
+ * Entry e = t * k + j is token t's j-th expert.  The plan sorts the entries by expert, stably: expert x's rows are
+ * bounds[x] .. bounds[x + 1], row r serves entry row_entry[r], entry e sits at row entry_row[e] (-1: its expert is not
+ * resident or its id is out of range).  Tiles of at most maya_moe_prefill_tile_rows() rows of one expert are what a
+ * workgroup of the GEMM kernels takes; all counts stay on the device, so nothing here synchronises. */
+typedef struct maya_prefill_plan {
+    int32_t* bounds;      /* [n_expert + 1] */
+    int32_t* row_entry;   /* [n_entries] */
+    int32_t* entry_row;   /* [n_entries] */
+    int32_t* tile_expert; /* [maya_moe_prefill_max_tiles()] */
+    int32_t* tile_row0;   /* [maya_moe_prefill_max_tiles()] */
+    int32_t* n_tiles;     /* [1] */
+} maya_prefill_plan;
+/* Rows of activations as int8 codes with one F32 scale per 32 values, c = rint(x * (127 / amax)), d = amax / 127, and
+ * s = d * (the 32 codes' sum) for the formats with a minimum. */
+typedef struct maya_prefill_act {
+    int8_t* q; /* [rows][k], 16-byte aligned */
+    float* d;  /* [rows][k / 32] */
+    float* s;  /* [rows][k / 32] */
+} maya_prefill_act;
+
+int maya_moe_prefill_tile_rows(void);
+int maya_moe_prefill_max_tiles(int n_entries, int n_expert);
+/* 1 when the prefill GEMMs take this weight type (Q4_K) */
+int maya_moe_prefill_supported(int type);
+int maya_moe_prefill_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert,
+                          const maya_prefill_plan* plan, void* stream);
+/* row r = the quantized x[row_entry[r] / k] for the plan's rows (rows past bounds[n_expert] are left alone) */
+int maya_moe_prefill_quant(const void* x, int x_dtype, int64_t x_stride, const maya_prefill_plan* plan, int n_entries,
+                           int n_expert, int k, int64_t n_embd, maya_prefill_act xq, void* stream);
+/* hq row r = the per-32 int8 of swiglu(gate_e . x_r, up_e . x_r) (clamped by limit), e the row's expert; int8 MFMA over
+ * the 4-bit codes and the activation codes, F32 scales per 32.  Expert blobs 8-byte aligned (GGUF packing). */
+int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, const maya_prefill_plan* plan,
+                             int n_entries, maya_prefill_act xq, float limit, maya_prefill_act hq, void* stream);
+/* part row r [n_embd] F32 = down_e . h_r */
+int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, const maya_prefill_plan* plan,
+                          int n_entries, maya_prefill_act hq, float* part, void* stream);
+/* out[t] = sum_j weights[t][j] * part[entry_row[t k + j]] in slot order (+ add[t]), stored as out_dtype */
+int maya_moe_prefill_combine(const maya_prefill_plan* plan, const float* weights, const float* part, int n_tokens, int k,
+                             int64_t n_embd, const float* add, void* out, int out_dtype, void* stream);
+/* route -> plan -> quantize -> gate/up -> down -> combine of one chunk, all on `stream` */
+size_t maya_moe_prefill_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k, int n_expert);
+int maya_moe_prefill_layer(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
+                           const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
+                           float* weights, void* out, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ================================================================================================ EXL3
  * EXL3 (exllamav3) trellis weights: a matrix with k inputs and n outputs is `trellis` uint32 [k/16][n/16][4*k2]
  * (16x16 tiles, 16*k2 bytes each, k2 = twice the bits per weight), FP16 `suh` [k] and `svh` [n];

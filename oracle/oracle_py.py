@@ -263,3 +263,78 @@ def exl3_mv(w, suh, svh, x):
     y = np.zeros(n, dtype=np.float32)
     lib().mo_exl3_mv(_ptr(w), _ptr(suh), _ptr(svh), k, n, _ptr(x), _ptr(y))
     return y
+
+
+def grouped_ref(t, mats, bounds, k, n, xq, xd, nthreads=8):
+    """mats: one uint8 array an expert (n rows of k values of type t, or None where the expert has no rows); rows
+    bounds[e] .. bounds[e + 1] of xq / xd are expert e's.  Returns float32 [rows, n]: the double products of the
+    dequantized weights with the dequantized int8 rows."""
+    ne = len(mats)
+    bounds = np.ascontiguousarray(bounds, dtype=np.int32)
+    xq = np.ascontiguousarray(xq, dtype=np.int8)
+    xd = np.ascontiguousarray(xd, dtype=np.float32)
+    keep = [None if m is None else np.ascontiguousarray(m, dtype=np.uint8) for m in mats]
+    ptrs = (C.c_void_p * ne)(*[None if m is None else m.ctypes.data for m in keep])
+    y = np.zeros((int(bounds[ne]), n), dtype=np.float32)
+    lib().mo_grouped_ref(t, ptrs, _ptr(bounds), ne, k, n, _ptr(xq), _ptr(xd), _ptr(y), nthreads)
+    return y
+
+
+def prefill_plan(ids, n_expert, resident=None):
+    """The stable sort of the entries e = t * k + j by expert: bounds [n_expert + 1], row_entry [rows], entry_row
+    [entries] (-1 where the expert is not resident or the id is out of range) (src/kernels/cuda/glm_batch.cu:2102-2133)."""
+    flat = np.asarray(ids, dtype=np.int64).reshape(-1)
+    ok = (flat >= 0) & (flat < n_expert)
+    if resident is not None:
+        ok &= np.asarray(resident, dtype=bool)[np.clip(flat, 0, n_expert - 1)]
+    ent = np.nonzero(ok)[0]
+    order = ent[np.argsort(flat[ent], kind="stable")]
+    counts = np.bincount(flat[ent], minlength=n_expert)
+    bounds = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    entry_row = np.full(flat.size, -1, dtype=np.int32)
+    entry_row[order] = np.arange(order.size, dtype=np.int32)
+    return bounds, order.astype(np.int32), entry_row
+
+
+def swiglu_rows(g, u, limit):
+    g = np.asarray(g, dtype=np.float32)
+    u = np.asarray(u, dtype=np.float32)
+    if limit > 0 and np.isfinite(limit):
+        g = np.minimum(g, np.float32(limit))
+        u = np.clip(u, -np.float32(limit), np.float32(limit))
+    return (g / (np.float32(1) + np.exp(-g)) * u).astype(np.float32)
+
+
+def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=0.0, resident=None, nthreads=8):
+    """A prompt chunk's routed experts the way the reference's fused prefill defines them
+    (src/prefill/moe_fused_rdna4.cu:87-109, 620-660; tests/hip/prefill_fused_parity.cpp:150-175): per-32 int8 rows of
+    x, double products with the dequantized gate / up rows, the clamped SwiGLU in F32, H requantized per 32, double
+    products with the down rows, the weighted sum in slot order.  Returns a dict of every stage."""
+    ids, w = router_topk(logits, k)
+    ne = len(blobs)
+    bounds, row_entry, entry_row = prefill_plan(ids, ne, resident)
+    rows = row_entry.size
+    xq = np.zeros((rows, n_embd), dtype=np.int8)
+    xd = np.zeros((rows, n_embd // 32), dtype=np.float32)
+    cache = {}
+    for r in range(rows):
+        tok = int(row_entry[r]) // k
+        if tok not in cache:
+            cache[tok] = quant_i8x32(x[tok])
+        xq[r], xd[r] = cache[tok]
+    used = [bounds[e + 1] > bounds[e] for e in range(ne)]
+    gate = grouped_ref(t, [blobs[e] if used[e] else None for e in range(ne)], bounds, n_embd, n_ff, xq, xd, nthreads)
+    up = grouped_ref(t, [blobs[e][up_off:] if used[e] else None for e in range(ne)], bounds, n_embd, n_ff, xq, xd, nthreads)
+    h = swiglu_rows(gate, up, limit)
+    hq = np.zeros((rows, n_ff), dtype=np.int8)
+    hd = np.zeros((rows, n_ff // 32), dtype=np.float32)
+    for r in range(rows):
+        hq[r], hd[r] = quant_i8x32(h[r])
+    part = grouped_ref(t, [blobs[e][down_off:] if used[e] else None for e in range(ne)], bounds, n_ff, n_embd, hq, hd, nthreads)
+    out = np.zeros((x.shape[0], n_embd), dtype=np.float32)
+    for tok in range(x.shape[0]):
+        sel = [j for j in range(k) if entry_row[tok * k + j] >= 0]
+        if sel:
+            out[tok] = combine(np.stack([part[entry_row[tok * k + j]] for j in sel]), np.array([w[tok, j] for j in sel]))
+    return dict(ids=ids, w=w, bounds=bounds, row_entry=row_entry, entry_row=entry_row, xq=xq, xd=xd, h=h, hq=hq, hd=hd,
+                part=part, out=out)

@@ -6,7 +6,7 @@ import sys
 PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmaya_moe.so")
-SOURCES = ["maya_kernels.hip", "maya_exl3.hip"]
+SOURCES = ["maya_kernels.hip", "maya_exl3.hip", "maya_prefill.hip"]
 # -packed-fp32-ops off: the compiler then forms no v_pk_*_f32 from scalar float code
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]

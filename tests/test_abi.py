@@ -32,8 +32,8 @@ def test_every_declared_function_is_exported(maya):
     L = C.CDLL(maya.LIB_PATH)
     missing = [n for n in names if not hasattr(L, n)]
     assert not missing, missing
-    from maya_amd import exl3
-    assert set(maya.EXPORTS + exl3.EXPORTS) == set(names)
+    from maya_amd import exl3, prefill
+    assert set(maya.EXPORTS + exl3.EXPORTS + prefill.EXPORTS) == set(names)
 
 
 def test_sizes_and_support_tables(maya, oracle):

@@ -1,0 +1,171 @@
+"""The prompt-chunk path on the GPU through the C ABI: plan (count / scan / stable scatter / tiles), per-32 int8
+activation rows, the grouped int8-MFMA GEMMs over Q4_K experts and the combine, against the CPU checker's restatement
+(double products of dequantized weights and dequantized int8 rows; tests/hip/prefill_fused_parity.cpp:150-175)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+from gpu_util import rel_l2, dev  # noqa: E402
+
+Q4_K = 12
+
+
+@pytest.fixture(scope="module")
+def pf():
+    from maya_amd import prefill
+    prefill.load()
+    return prefill
+
+
+def make_blobs(oracle, n_expert, n_embd, n_ff, seed, encoded=False):
+    from maya_amd import synth
+    rng = np.random.default_rng(seed)
+    if not encoded:
+        return [synth.expert_blob(Q4_K, Q4_K, n_embd, n_ff, rng) for _ in range(n_expert)]
+    blobs = []
+    for _ in range(n_expert):   # N(0, 0.02) weights through the checker's own Q4_K encoder
+        mats = [rng.standard_normal(n_ff * n_embd).astype(np.float32) * 0.02 for _ in range(3)]
+        blobs.append(np.concatenate([oracle.encode_q4k(m) for m in mats]))
+    return blobs
+
+
+PLAN_CASES = [(1, 1, 4, 0), (37, 2, 8, 1), (64, 8, 256, 2), (512, 8, 256, 3), (300, 3, 7, 4), (1000, 4, 1024, 5)]
+
+
+@pytest.mark.parametrize("n_tokens,k,n_expert,seed", PLAN_CASES)
+def test_plan_matches_stable_sort(pf, oracle, n_tokens, k, n_expert, seed):
+    from maya_amd import synth
+    rng = np.random.default_rng(seed)
+    logits = rng.standard_normal((n_tokens, n_expert)).astype(np.float32) + synth.zipf_bias(n_expert)
+    ids = np.argsort(-logits, axis=1, kind="stable")[:, :min(k, n_expert)].astype(np.int32)
+    if seed == 4:
+        ids[5, 1] = -3            # out-of-range ids are dropped
+        ids[9, 0] = n_expert
+    resident = np.ones(n_expert, dtype=bool)
+    if n_expert >= 7:
+        resident[[1, 6]] = False  # experts that are not on the device are dropped
+    table = torch.from_numpy(np.where(resident, 4096 * (1 + np.arange(n_expert)), 0).astype(np.int64)).cuda()
+    p = pf.plan(dev(ids).reshape(-1), table)
+    torch.cuda.synchronize()
+    bounds, row_entry, entry_row = oracle.prefill_plan(ids, n_expert, resident)
+    assert np.array_equal(p.bounds.cpu().numpy(), bounds)
+    rows = int(bounds[-1])
+    assert np.array_equal(p.row_entry.cpu().numpy()[:rows], row_entry)
+    assert np.array_equal(p.entry_row.cpu().numpy(), entry_row)
+    # the tiles: every expert's rows exactly once, in runs of at most tile_rows
+    tr = pf.load().maya_moe_prefill_tile_rows()
+    nt = int(p.n_tiles.item())
+    te, t0 = p.tile_expert.cpu().numpy()[:nt], p.tile_row0.cpu().numpy()[:nt]
+    assert nt == sum((int(bounds[e + 1] - bounds[e]) + tr - 1) // tr for e in range(n_expert)) <= p.max_tiles
+    seen = np.zeros(rows, dtype=np.int32)
+    for e, r0 in zip(te, t0):
+        assert bounds[e] <= r0 < bounds[e + 1] and (r0 - bounds[e]) % tr == 0
+        seen[r0:min(r0 + tr, bounds[e + 1])] += 1
+    assert np.all(seen == 1)
+
+
+def test_quantized_rows_match_checker(pf, oracle):
+    rng = np.random.default_rng(21)
+    n_tokens, k, n_expert, n_embd = 19, 3, 6, 768
+    ids = np.stack([rng.permutation(n_expert)[:k] for _ in range(n_tokens)]).astype(np.int32)
+    x = rng.standard_normal((n_tokens, n_embd)).astype(np.float32)
+    x[3] = 0.0
+    x[4, :32] = [(-1) ** i * (i + 0.5) / 31.5 * 127 / 127 for i in range(32)]   # codes on exact halves: ties to even
+    table = torch.arange(1, n_expert + 1, dtype=torch.int64, device="cuda") * 4096
+    p = pf.plan(dev(ids).reshape(-1), table)
+    for xt in (torch.from_numpy(x), torch.from_numpy(x).to(torch.bfloat16), torch.from_numpy(x).to(torch.float16)):
+        a = pf.quant(xt.cuda(), p, k)
+        torch.cuda.synchronize()
+        xf = xt.to(torch.float32).numpy()
+        row_entry = p.row_entry.cpu().numpy()
+        q, d, s = a.q.cpu().numpy(), a.d.cpu().numpy(), a.s.cpu().numpy()
+        for r in range(n_tokens * k):
+            wq, wd = oracle.quant_i8x32(xf[row_entry[r] // k])
+            assert np.array_equal(q[r], wq) and np.array_equal(d[r], wd)
+            assert np.array_equal(s[r], wd * wq.reshape(-1, 32).sum(axis=1).astype(np.float32))
+
+
+LAYER_CASES = [
+    # n_embd, n_ff, n_expert, k, n_tokens, limit, encoded weights, experts that are not resident
+    (512, 256, 8, 2, 37, 0.0, False, ()),
+    (1024, 512, 16, 4, 200, 7.0, True, (2,)),
+    (768, 512, 4, 1, 1, 0.0, True, ()),
+    (512, 256, 3, 3, 150, 0.0, False, ()),       # every token on every expert: 150-row experts, 3 tiles each
+    (7168, 2048, 3, 2, 24, 0.0, True, ()),       # the full expert shape
+]
+
+
+@pytest.mark.parametrize("case", LAYER_CASES, ids=[str(c[:5]) for c in LAYER_CASES])
+def test_stages_and_layer_match_checker(pf, oracle, case):
+    from maya_amd import lib, synth
+    n_embd, n_ff, n_expert, k, n_tokens, limit, encoded, absent = case
+    blobs = make_blobs(oracle, n_expert, n_embd, n_ff, 50 + n_embd, encoded)
+    up_off, down_off, _ = synth.blob_offsets(Q4_K, Q4_K, n_embd, n_ff)
+    store = lib.ExpertStore(blobs)
+    table = store.table.clone()
+    resident = np.ones(n_expert, dtype=bool)
+    for e in absent:
+        table[e] = 0
+        resident[e] = False
+    rng = np.random.default_rng(n_tokens)
+    logits = (rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32)
+    x = rng.standard_normal((n_tokens, n_embd)).astype(np.float32)
+    want = oracle.prefill_layer(Q4_K, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit, resident)
+    layout, _ = lib.layout(Q4_K, Q4_K, n_embd, n_ff)
+
+    ids, w = lib.route_topk(dev(logits), k)
+    p = pf.plan(ids.reshape(-1), table)
+    xq = pf.quant(dev(x), p, k)
+    hq = pf.gate_up(layout, table, p, xq, limit)
+    part = pf.down(layout, table, p, hq)
+    out = pf.combine(p, w, part, n_tokens, k)
+    out16 = pf.combine(p, w, part, n_tokens, k, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    rows = int(want["bounds"][-1])
+    assert np.array_equal(ids.cpu().numpy(), want["ids"])
+    assert np.array_equal(p.row_entry.cpu().numpy()[:rows], want["row_entry"])
+    assert np.array_equal(xq.q.cpu().numpy()[:rows], want["xq"])
+
+    # H: the codes differ from the checker's by at most one step, rarely; the decoded rows agree to 1e-3
+    gq, gd = hq.q.cpu().numpy()[:rows].astype(np.int32), hq.d.cpu().numpy()[:rows]
+    diff = np.abs(gq - want["hq"].astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 5e-3
+    got_h = gq.reshape(rows, -1, 32) * gd[:, :, None]
+    want_h = want["hq"].astype(np.int32).reshape(rows, -1, 32) * want["hd"][:, :, None]
+    assert rel_l2(got_h, want_h) <= 1e-3
+    gs = hq.s.cpu().numpy()[:rows]
+    assert np.array_equal(gs, gd * gq.reshape(rows, -1, 32).sum(axis=2).astype(np.float32))
+
+    # down over the GPU's own H: only F32 rounding apart from the double products
+    mats = [blobs[e][down_off:] if want["bounds"][e + 1] > want["bounds"][e] else None for e in range(n_expert)]
+    want_part = oracle.grouped_ref(Q4_K, mats, want["bounds"], n_ff, n_embd, gq.astype(np.int8), gd)
+    assert rel_l2(part.cpu().numpy()[:rows], want_part) <= 1e-5
+
+    got = out.cpu().numpy()
+    for t in range(n_tokens):
+        assert rel_l2(got[t], want["out"][t]) <= 1e-3, t
+    assert torch.equal(out16, out.to(torch.bfloat16))
+
+    # the one-call layer gives the same bits as the stages
+    layer = pf.PrefillLayer(layout, n_expert, k, n_tokens, out_dtype=torch.float32)
+    got2 = layer.forward(table, dev(logits), dev(x), limit=limit)
+    torch.cuda.synchronize()
+    assert torch.equal(got2, out)
+
+
+def test_unsupported_and_bad_arguments(pf):
+    from maya_amd import lib
+    assert pf.load().maya_moe_prefill_supported(Q4_K) == 1 and pf.load().maya_moe_prefill_supported(22) == 0
+    table = torch.arange(1, 5, dtype=torch.int64, device="cuda") * 4096
+    ids = torch.zeros(8, dtype=torch.int32, device="cuda")
+    p = pf.plan(ids, table)
+    xq = pf.ActRows(8, 512)
+    iq, _ = lib.layout(22, 22, 512, 256)
+    with pytest.raises(lib.MayaError):
+        pf.gate_up(iq, table, p, xq)
+    bad, _ = lib.layout(Q4_K, Q4_K, 512, 256)
+    bad.n_ff = 200
+    with pytest.raises(lib.MayaError):
+        pf.gate_up(bad, table, p, xq)
