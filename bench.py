@@ -25,6 +25,10 @@ for _p in (os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle"),
 N_EMBD, N_FF, N_EXPERT, TOP_K = 7168, 2048, 256, 8
 IQ2_S = 22
 HBM_PEAK = 8.0e12
+# HBM bytes of one gate/up launch on this workload from rocprofv3's FETCH_SIZE and WRITE_SIZE (two runs, each scaled by
+# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,796.4 KiB read + 72.1 KiB written
+# (profiles/decode_iq2s_hbm_traffic_pmc.txt)
+GATE_UP_TRAFFIC_BYTES = int((73796.4 + 72.1) * 1024)
 
 
 def synth_experts_on_device(torch, n_expert, blob_bytes, seed):
@@ -134,6 +138,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus,
@@ -166,6 +173,13 @@ def main():
     rng = np.random.default_rng(11)
     x = torch.from_numpy(rng.standard_normal((1, N_EMBD)).astype(np.float32)).to(torch.bfloat16).cuda()
     torch.cuda.synchronize()
+
+    if args.calib_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     stream = torch.cuda.Stream()
     K, W = args.steps, args.warmup
@@ -275,8 +289,8 @@ def main():
                    "n_embd": N_EMBD, "n_ff": N_FF, "n_expert": N_EXPERT, "top_k": TOP_K, "tokens": 1,
                    "weight_bytes_per_step": w_bytes, "algorithmic_bytes_per_step": bytes_step,
                    "timed_as": "eager launches" if args.no_graph else "one HIP graph of the K steps", "device": info},
-        "roofline": {"bound": "hbm", "kernel": "gate_up_kernel<IQ2_S>", "achieved": round(gu_rate, 2), "peak": 8000.0,
-                     "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_pos_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
+                     "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 3)},
         "cpu_baseline": cpu,
         "parity_rel_l2_vs_cpu_path": err,

@@ -884,7 +884,8 @@ int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStrea
     static const int variant = tuning_variant("MAYA_DN_VARIANT", 0);
     if (variant == 1) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 2, 5>), grid, dim3(512), 0, s, a, st.cb);
     else if (variant == 2) hipLaunchKernelGGL((down_iq2s_pos_kernel<8, 1, 8>), dim3(grid.x * 2), dim3(512), 0, s, a, st.cb);
-    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 8>), grid, dim3(512), 0, s, a, st.cb);
+    else if (variant == 3) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 8>), grid, dim3(512), 0, s, a, st.cb);
+    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);   // 8 waves a SIMD spill
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
     return MAYA_OK;
 }

@@ -249,6 +249,25 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
     PfStage st;
     pf_fetch(a, row0, nrows, 0, st);
     pf_store(lds[0], st);
+    // the weights run one step (64 values of the 4 rows) ahead of the arithmetic, the block headers one super-block
+    uint64_t qcur[4], qnext[4];
+    uint32_t hdr[4][4];
+    auto load_q = [&](int sb, int j, uint64_t (&q)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) q[t] = *(const uint64_t*) (wrow[t] + (size_t) sb * 144 + 16 + 32 * j + 8 * g);
+    };
+    auto load_h = [&](int sb) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t* hp = (const uint32_t*) (wrow[t] + (size_t) sb * 144);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) hdr[t][i] = hp[i];
+        }
+    };
+    if (wave_on) {
+        load_h(0);
+        load_q(0, 0, qcur);
+    }
     __syncthreads();
     for (int sb = 0; sb < nsb; ++sb) {
         const uint8_t* buf = lds[sb & 1];
@@ -258,19 +277,19 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
             uint32_t sc[4][2], mn[4][2];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                const uint32_t* hp = (const uint32_t*) (wrow[t] + (size_t) sb * 144);
-                const uint32_t h0 = hp[0];
-                d[t] = f16_bits_to_f32((uint16_t) (h0 & 0xffffu));
-                dmin[t] = f16_bits_to_f32((uint16_t) (h0 >> 16));
-                q4k_unpack_scales(hp[1], hp[2], hp[3], sc[t], mn[t]);
+                d[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] & 0xffffu));
+                dmin[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] >> 16));
+                q4k_unpack_scales(hdr[t][1], hdr[t][2], hdr[t][3], sc[t], mn[t]);
             }
             const float* sxl = (const float*) (buf + kPfRows * kPfRowBytes);
             const float* ssl = sxl + 8 * kPfRows;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint64_t qw[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) qw[t] = *(const uint64_t*) (wrow[t] + (size_t) sb * 144 + 16 + 32 * j + 8 * g);
+                if (j < 3) load_q(sb, j + 1, qnext);
+                else if (sb + 1 < nsb) {
+                    load_q(sb + 1, 0, qnext);
+                    load_h(sb + 1);
+                }
 #pragma unroll
                 for (int nib = 0; nib < 2; ++nib) {
                     const int blk = 2 * j + nib;
@@ -278,7 +297,7 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
                     float dsc[4], dm[4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        wb[t] = (long) ((qw[t] >> (4 * nib)) & 0x0f0f0f0f0f0f0f0full);
+                        wb[t] = (long) ((qcur[t] >> (4 * nib)) & 0x0f0f0f0f0f0f0f0full);
                         dsc[t] = __fmul_rn(d[t], byte_f32(sc[t][blk >> 2], blk & 3));
                         dm[t] = __fmul_rn(dmin[t], byte_f32(mn[t][blk >> 2], blk & 3));
                     }
@@ -289,13 +308,15 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
                             const float4 sx = *(const float4*) (sxl + blk * kPfRows + 16 * m + 4 * g);
                             const float4 ss = *(const float4*) (ssl + blk * kPfRows + 16 * m + 4 * g);
                             const float sxa[4] = {sx.x, sx.y, sx.z, sx.w}, ssa[4] = {ss.x, ss.y, ss.z, ss.w};
+                            v4i dot[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) dot[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb[t], v4i{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
                             for (int t = 0; t < 4; ++t) {
-                                const v4i dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb[t], v4i{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
                                 for (int i = 0; i < 4; ++i) {
                                     float v = acc[t][m][i];
-                                    v = fmaf(__fmul_rn(dsc[t], sxa[i]), (float) dot[i], v);
+                                    v = fmaf(__fmul_rn(dsc[t], sxa[i]), (float) dot[t][i], v);
                                     v = fmaf(-dm[t], ssa[i], v);
                                     acc[t][m][i] = v;
                                 }
@@ -303,6 +324,8 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
                         }
                     }
                 }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) qcur[t] = qnext[t];
             }
         }
         if (sb + 1 < nsb) pf_store(lds[(sb + 1) & 1], st);
