@@ -217,3 +217,12 @@ def test_iq1_dequant_structure(oracle):
                     if vals <= {7 * m, 9 * m, m}:
                         ok = True
                 assert ok, (t, b, g, vals)
+
+
+def test_float_and_double_selection_agree(oracle):
+    # the kernel selects on float p, the reference's host test on double p: no disagreement on N(0,1) logits
+    rng = np.random.default_rng(8)
+    logits = rng.standard_normal((2000, 256)).astype(np.float32)
+    a, _ = oracle.router_topk(logits, 8)
+    b, _ = oracle.router_topk(logits, 8, f64=True)
+    assert np.array_equal(a, b)
