@@ -61,10 +61,12 @@ typedef struct maya_moe_layout {
     int32_t reserved;
 } maya_moe_layout;
 
-/* Row packings.  GGUF: the file's own block sequence.  STREAM: the same bytes of every row regrouped by field so that a
- * wavefront's loads are aligned and contiguous (IQ2_S rows: all (index word, sign word) pairs, then all (high-bit, scale)
- * byte pairs, then the block scales; other types are left as they are).  A row keeps its size and its position in the
- * blob, every field keeps its bits, so dequantized values are unchanged. */
+/* Row packings.  GGUF: the file's own block sequence.  STREAM: the same bytes regrouped so that a wavefront's loads are
+ * aligned, contiguous and addressed by position alone.  IQ2_S rows are taken four at a time (a quad; row counts are
+ * multiples of 4): with nu = k / 32 sub-blocks a row, the quad's 4 * row_bytes bytes hold, for sub-block u of row r of
+ * the quad, the (index word, sign word) pair at byte 8 (4 u + r), the (high-bit byte, scale byte) pair at
+ * 32 nu + 2 (4 u + r), and block b's FP16 scale at 40 nu + 2 (4 b + r).  Other types are left as they are.  A quad keeps
+ * its size and its position in the blob and every field keeps its bits, so dequantized values are unchanged. */
 #define MAYA_PACK_GGUF 0
 #define MAYA_PACK_STREAM 1
 
