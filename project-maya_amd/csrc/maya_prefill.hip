@@ -25,6 +25,7 @@ constexpr int kPlanThreads = 1024;
 constexpr int kPlanWaves = kPlanThreads / 64;
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // ---------------------------------------------------------------------------------------------------- the plan
 // One workgroup: counts per expert and per segment (a wave's contiguous share of the entries), the prefix sums, then
@@ -211,15 +212,10 @@ __device__ __forceinline__ float pf_swiglu(float g, float u, float limit) {
     return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
 }
 
-// grid (bands of weight rows, tiles at most)
-template <bool GU>
-__global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][kPfBufBytes];
-    const int tile = blockIdx.y;
-    if (tile >= *a.plan.n_tiles) return;
-    const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
-    const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
-    const int n_mt = (nrows + 15) >> 4;
+// one tile of NMT x 16 rows (the row count of the tile is a compile-time bound, so the inner loop is branch-free and
+// the compiler can move the LDS reads of a step above the arithmetic of the one before)
+template <bool GU, int NMT>
+__device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t (*lds)[kPfBufBytes], int ex, int row0, int nrows) {
     const uint8_t* blob = (const uint8_t*) a.table[ex];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 15, g = lane >> 4;
 
@@ -237,36 +233,54 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
     }
     const bool wave_on = n0 < a.n;   // (a.n is a multiple of the wave's rows: checked on the host)
 
-    float acc[4][kPfMt][4];
+    v4f acc[4][NMT];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int m = 0; m < kPfMt; ++m)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[t][m][i] = 0.0f;
+        for (int m = 0; m < NMT; ++m) acc[t][m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     const int nsb = (int) (a.k >> 8);
     PfStage st;
     pf_fetch(a, row0, nrows, 0, st);
     pf_store(lds[0], st);
-    // the weights run one step (64 values of the 4 rows) ahead of the arithmetic, the block headers one super-block
-    uint64_t qcur[4], qnext[4];
-    uint32_t hdr[4][4];
-    auto load_q = [&](int sb, int j, uint64_t (&q)[4]) {
+    // Weights run ahead of the arithmetic in registers.  Small tiles (1 or 2 groups of 16 rows) are bound by the weight
+    // stream: they keep a whole super-block in flight, and everything a lane needs of a row's 144-byte block (the 16-byte
+    // header and its four 8-byte slices of the codes) is requested in one burst, so the block's one or two cache lines are
+    // fetched once, not once per slice at different times.
+    // Tiles of 3 and 4 row groups have no registers to spare for a second block: their code slices run three slices
+    // ahead in a ring of four register sets instead (slice j in set j) and the header a block ahead.
+    constexpr bool kBurst = NMT <= 2;
+    uint64_t q[4][4], qn[kBurst ? 4 : 1][4];     // [slice j][row tile t]
+    uint32_t hdr[4][4], hdrn[kBurst ? 4 : 1][4];
+    auto load_q = [&](int sb, int j, uint64_t (&dst)[4]) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) q[t] = *(const uint64_t*) (wrow[t] + (size_t) sb * 144 + 16 + 32 * j + 8 * g);
+        for (int t = 0; t < 4; ++t) dst[t] = *(const uint64_t*) (wrow[t] + (size_t) sb * 144 + 16 + 32 * j + 8 * g);
     };
-    auto load_h = [&](int sb) {
+    auto load_h = [&](int sb, uint32_t (&dh)[4][4]) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const uint32_t* hp = (const uint32_t*) (wrow[t] + (size_t) sb * 144);
+            const uint4 h = *(const uint4*) (wrow[t] + (size_t) sb * 144);
+            dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
+        }
+    };
+    auto load_block = [&](int sb, uint64_t (&dq)[4][4], uint32_t (&dh)[4][4]) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) hdr[t][i] = hp[i];
+        for (int t = 0; t < 4; ++t) {
+            const uint8_t* blk = wrow[t] + (size_t) sb * 144;
+            const uint4 h = *(const uint4*) blk;
+            dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dq[j][t] = *(const uint64_t*) (blk + 16 + 32 * j + 8 * g);
         }
     };
     if (wave_on) {
-        load_h(0);
-        load_q(0, 0, qcur);
+        if constexpr (kBurst) load_block(0, q, hdr);
+        else {
+            load_h(0, hdr);
+            load_q(0, 0, q[0]);
+            load_q(0, 1, q[1]);
+            load_q(0, 2, q[2]);
+        }
     }
     __syncthreads();
     for (int sb = 0; sb < nsb; ++sb) {
@@ -281,51 +295,75 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
                 dmin[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] >> 16));
                 q4k_unpack_scales(hdr[t][1], hdr[t][2], hdr[t][3], sc[t], mn[t]);
             }
+            if (sb + 1 < nsb) {
+                if constexpr (kBurst) load_block(sb + 1, qn, hdrn);
+                else load_h(sb + 1, hdr);   // (decoded above: its registers are free)
+            }
             const float* sxl = (const float*) (buf + kPfRows * kPfRowBytes);
             const float* ssl = sxl + 8 * kPfRows;
+            // the minimums' term, -(dmin m) . s over the 8 sub-blocks, on the matrix cores in F32: A = the tokens' s
+            // (row = token, k = sub-block), B = this lane's row's -dmin m, accumulated straight into acc
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                float nb[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) nb[t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
+#pragma unroll
+                for (int m = 0; m < NMT; ++m) {
+                    const float sa = ssl[(4 * half + g) * kPfRows + 16 * m + ln];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa, nb[t], acc[t][m], 0, 0, 0);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if (j < 3) load_q(sb, j + 1, qnext);
-                else if (sb + 1 < nsb) {
-                    load_q(sb + 1, 0, qnext);
-                    load_h(sb + 1);
+                if constexpr (!kBurst) {   // slice (sb, j) + 3 into the set that slice (sb, j) - 1 has left
+                    const int jn = (j + 3) & 3, sbn = sb + ((j + 3) >> 2);
+                    if (sbn < nsb) load_q(sbn, jn, q[jn]);
                 }
 #pragma unroll
                 for (int nib = 0; nib < 2; ++nib) {
                     const int blk = 2 * j + nib;
                     long wb[4];
-                    float dsc[4], dm[4];
+                    float dsc[4];
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
-                        wb[t] = (long) ((qcur[t] >> (4 * nib)) & 0x0f0f0f0f0f0f0f0full);
-                        dsc[t] = __fmul_rn(d[t], byte_f32(sc[t][blk >> 2], blk & 3));
-                        dm[t] = __fmul_rn(dmin[t], byte_f32(mn[t][blk >> 2], blk & 3));
+                        wb[t] = (long) ((q[j][t] >> (4 * nib)) & 0x0f0f0f0f0f0f0f0full);
+                        // (the scale word is made opaque here: converted up front for all 8 sub-blocks, the 32 products
+                        // would sit in registers for the whole super-block)
+                        uint32_t scw = sc[t][blk >> 2];
+                        asm volatile("" : "+v"(scw));
+                        dsc[t] = __fmul_rn(d[t], byte_f32(scw, blk & 3));
                     }
 #pragma unroll
-                    for (int m = 0; m < kPfMt; ++m) {
-                        if (m < n_mt) {
-                            const long xa = *(const long*) (buf + (16 * m + ln) * kPfRowBytes + blk * 32 + 8 * g);
-                            const float4 sx = *(const float4*) (sxl + blk * kPfRows + 16 * m + 4 * g);
-                            const float4 ss = *(const float4*) (ssl + blk * kPfRows + 16 * m + 4 * g);
-                            const float sxa[4] = {sx.x, sx.y, sx.z, sx.w}, ssa[4] = {ss.x, ss.y, ss.z, ss.w};
-                            v4i dot[4];
+                    for (int m = 0; m < NMT; ++m) {
+                        const long xa = *(const long*) (buf + (16 * m + ln) * kPfRowBytes + blk * 32 + 8 * g);
+                        const float4 sx = *(const float4*) (sxl + blk * kPfRows + 16 * m + 4 * g);
+                        const float sxa[4] = {sx.x, sx.y, sx.z, sx.w};
+                        v4i dot[4];
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) dot[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb[t], v4i{0, 0, 0, 0}, 0, 0, 0);
+                        for (int t = 0; t < 4; ++t) dot[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb[t], v4i{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) {
+                        for (int t = 0; t < 4; ++t) {
 #pragma unroll
-                                for (int i = 0; i < 4; ++i) {
-                                    float v = acc[t][m][i];
-                                    v = fmaf(__fmul_rn(dsc[t], sxa[i]), (float) dot[t][i], v);
-                                    v = fmaf(-dm[t], ssa[i], v);
-                                    acc[t][m][i] = v;
-                                }
-                            }
+                            for (int i = 0; i < 4; ++i)
+                                acc[t][m][i] = fmaf(__fmul_rn(dsc[t], sxa[i]), (float) dot[t][i], acc[t][m][i]);
+                            // (pinned: left free, the optimizer issues every dot of the super-block first and holds
+                            // their 128 results in registers)
+                            asm volatile("" : "+v"(acc[t][m]));
                         }
                     }
+                    __builtin_amdgcn_sched_barrier(0);   // a sub-block's work stays together
                 }
+            }
+            if constexpr (kBurst) {
+                if (sb + 1 < nsb) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) qcur[t] = qnext[t];
+                    for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i], q[i][t] = qn[i][t];
+                    }
+                }
             }
         }
         if (sb + 1 < nsb) pf_store(lds[(sb + 1) & 1], st);
@@ -335,8 +373,7 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
 
     // outputs: lane (ln, g) holds weight row ln of each tile for the tokens 16 m + 4 g + i
 #pragma unroll
-    for (int m = 0; m < kPfMt; ++m) {
-        if (m >= n_mt) continue;
+    for (int m = 0; m < NMT; ++m) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = 16 * m + 4 * g + i;
@@ -370,6 +407,22 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
                 for (int t = 0; t < 4; ++t) o[16 * t] = acc[t][m][i];
             }
         }
+    }
+}
+
+// grid (bands of weight rows, tiles at most)
+template <bool GU>
+__global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][kPfBufBytes];
+    const int tile = blockIdx.y;
+    if (tile >= *a.plan.n_tiles) return;
+    const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
+    const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
+    switch ((nrows + 15) >> 4) {
+        case 1: pf_tile<GU, 1>(a, lds, ex, row0, nrows); break;
+        case 2: pf_tile<GU, 2>(a, lds, ex, row0, nrows); break;
+        case 3: pf_tile<GU, 3>(a, lds, ex, row0, nrows); break;
+        default: pf_tile<GU, 4>(a, lds, ex, row0, nrows); break;
     }
 }
 
@@ -459,7 +512,7 @@ static int prefill_check(const char* what, const maya_moe_layout* l, const uint6
     if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_UNSUPPORTED, "%s: GGUF packing only", what);
     if (l->n_embd <= 0 || l->n_ff <= 0 || l->n_embd % 256 || l->n_ff % 256)
         return fail(MAYA_E_SHAPE, "%s: n_embd %d / n_ff %d: multiples of 256 wanted", what, l->n_embd, l->n_ff);
-    if ((l->gate_off | l->up_off | l->down_off) & 7) return fail(MAYA_E_ARG, "%s: matrix offsets not 8-byte aligned", what);
+    if ((l->gate_off | l->up_off | l->down_off) & 15) return fail(MAYA_E_ARG, "%s: matrix offsets not 16-byte aligned", what);
     if (n_entries <= 0 || n_entries > 65535 * kPfRows || n_expert <= 0) return fail(MAYA_E_SHAPE, "%s: entries %d experts %d", what, n_entries, n_expert);
     return MAYA_OK;
 }
