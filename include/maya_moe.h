@@ -175,6 +175,9 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream);
 /* 1 when maya_moe_gate_up, given hq_sync, writes hq itself for these arguments (the caller then skips maya_quant_act
  * of h), 0 when it leaves hq alone. */
 int maya_moe_gate_up_fuses_hq(const maya_moe_args* a);
+/* 1 when maya_moe_down, given hq = {NULL, NULL, NULL}, rounds h to the down type's activation format itself for these
+ * arguments (native_quant_h's arithmetic, in the kernel's prologue; part may then be NULL), 0 when hq must be given. */
+int maya_moe_down_rounds_h(const maya_moe_args* a);
 int maya_moe_down(const maya_moe_args* a, void* stream);
 
 /* ---- the whole routed layer for a decode step / verify window of n_tokens <= MAYA_MAX_TOKENS tokens:

@@ -466,13 +466,54 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     __syncthreads();
     if (blob != 0ull) {
         int y[8];
-        const int4* q = (const int4*) (a.hq.q + (size_t) wave * 2048);
-        const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
-        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+        float dy8;
+        if (a.hq.q) {
+            const int4* q = (const int4*) (a.hq.q + (size_t) wave * 2048);
+            const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+            y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+            dy8 = a.hq.d[(size_t) wave * 64 + lane] * 0.125f;
+        } else {
+            // no rounded h given: the wave rounds its slot's h to Q8_K itself (quant_q8k_block's arithmetic): a lane holds
+            // sub-block `lane`, a 256-value block is 8 lanes; the block's signed maximum is the value at the FIRST largest
+            // magnitude - inside a lane the scan keeps the first, between lanes the lower lane wins a tie
+            const float4* hv = (const float4*) (a.h + (size_t) wave * 2048 + 32 * lane);
+            float v[32];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float4 t = hv[i];
+                v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+            }
+            float am = 0.0f, sv = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const float av = fabsf(v[i]);
+                if (av > am) am = av, sv = v[i];
+            }
+#pragma unroll
+            for (int o = 1; o < 8; o <<= 1) {
+                const float oa = __shfl_xor(am, o, kWave), os = __shfl_xor(sv, o, kWave);
+                if (oa > am || (oa == am && (lane & o))) am = oa, sv = os;
+            }
+            float iscale = 0.0f, d = 0.0f;
+            if (am > 0.0f) {
+                iscale = __fdiv_rn(-127.0f, sv);
+                d = __fdiv_rn(1.0f, iscale);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int c = am > 0.0f ? min(127, nearest_int(__fmul_rn(iscale, v[4 * i + b]))) : 0;
+                    w |= ((uint32_t) c & 0xffu) << (8 * b);
+                }
+                y[i] = (int) w;
+            }
+            dy8 = d * 0.125f;
+        }
         int yn[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
-        const float dy8 = a.hq.d[(size_t) wave * 64 + lane] * 0.125f;
         constexpr uint32_t qb = NU / 8 * 82 * 4;
         // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
         // scalar registers for the buffer resource

@@ -926,6 +926,12 @@ bool gate_up_fuses_hq(const maya_moe_args& a) {
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
 }
+// whether try_down_iq2s_1tok would take the position-mapped kernel, which can round h to Q8_K itself (hq.q == NULL)
+bool down_rounds_h(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    return l.down_type == kIQ2_S && fast_1tok(a) && a.k <= 8 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 &&
+           l.n_embd % 16 == 0;
+}
 int try_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
     const maya_moe_layout& l = a.layout;
     if (a.k > 8) return 0;
@@ -1155,11 +1161,16 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
 }
 
 int maya_moe_gate_up_fuses_hq(const maya_moe_args* a) { return a && a->hq_sync && gate_up_fuses_hq(*a) ? 1 : 0; }
+int maya_moe_down_rounds_h(const maya_moe_args* a) { return a && down_rounds_h(*a) ? 1 : 0; }
 
 int maya_moe_down(const maya_moe_args* a, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (const int rc = check_args(a)) return rc;
+    if (!a->hq.q && !a->hq.d && !a->hq.bsums && a->h && a->out && down_rounds_h(*a)) {
+        int rc = 0;   // the kernel rounds h itself
+        if (try_down_iq2s_1tok(*a, *st, as_stream(stream), &rc)) return rc;
+    }
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
     hipStream_t s = as_stream(stream);
     if (a->layout.down_type == kIQ2_S && fast_1tok(*a)) {
@@ -1260,7 +1271,7 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
             default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
         }
         MAYA_LAUNCHED("layer_head_kernel");
-        a.hq_sync = w.hq_sync;
+        a.hq_sync = down_rounds_h(a) ? nullptr : w.hq_sync;   // (the down kernel's own rounding of h is the cheaper one)
     } else {
         if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
         if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
@@ -1274,8 +1285,12 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
         a.n_groups = w.n_groups;
     }
     if ((rc = maya_moe_gate_up(&a, stream))) return rc;
-    if (!maya_moe_gate_up_fuses_hq(&a))
+    if (down_rounds_h(a)) {
+        a.hq = maya_act{nullptr, nullptr, nullptr};
+        a.part = nullptr;
+    } else if (!maya_moe_gate_up_fuses_hq(&a)) {
         if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
+    }
     return maya_moe_down(&a, stream);
 }
 

@@ -18,7 +18,7 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack",
-    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq",
+    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h",
 ]
 
 
@@ -76,6 +76,7 @@ def load():
     L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_gate_up_fuses_hq.argtypes = [C.POINTER(Args)]
+    L.maya_moe_down_rounds_h.argtypes = [C.POINTER(Args)]
     L.maya_moe_workspace_bytes.restype = sz
     L.maya_moe_workspace_bytes.argtypes = [C.POINTER(Layout), i32, i32]
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]

@@ -153,3 +153,43 @@ def test_unsupported_and_bad_shapes_fail_cleanly(lib):
     assert L.maya_moe_supported(22) == 1 and L.maya_moe_supported(10) == 0
     with pytest.raises(lib.MayaError):
         lib.route_topk(torch.zeros((1, 4), device="cuda"), 8)
+
+
+def test_down_rounds_h_itself_like_the_quantizer(lib):
+    """The stream-packed IQ2_S down kernel given no rounded h rounds it in its prologue: the same Q8_K codes as
+    maya_quant_act (ties, an all-zero block, equal magnitudes of both signs), so the same output bits."""
+    import ctypes as C
+    L = lib.load()
+    n_embd, n_ff, ne, k = 1024, 2048, 8, 8
+    blobs = make_experts(22, 22, n_embd, n_ff, ne, 77)
+    gguf, _ = lib.layout(22, 22, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf)
+    rng = np.random.default_rng(3)
+    h = rng.standard_normal((k, n_ff)).astype(np.float32)
+    h[0, 256:512] = 0.0
+    h[1, 512:768] = 0.5
+    h[2, 100], h[2, 200] = -7.0, 7.0          # the first (negative) maximum sets the sign of the scale
+    h[3, 900], h[3, 300] = 9.0, -9.0
+    h_d = dev(h)
+    hq = lib.quant_act(22, h_d)
+    w = dev(rng.uniform(0.05, 0.3, k).astype(np.float32))
+    plan = store.table.clone()
+    outs = []
+    for given in (True, False):
+        a = lib.Args()
+        a.layout = lib.copy_layout(gguf, lib.PACK_STREAM)
+        a.n_tokens, a.k = 1, k
+        a.plan_ptr, a.plan_w = plan.data_ptr(), w.data_ptr()
+        a.limit = float("inf")
+        a.h = h_d.data_ptr()
+        part = torch.zeros((k, n_embd), device="cuda")
+        out = torch.zeros((1, n_embd), device="cuda")
+        a.out = out.data_ptr()
+        if given:
+            a.hq, a.part = hq.c(), part.data_ptr()
+        assert L.maya_moe_down_rounds_h(C.byref(a)) == 1
+        lib.check(L.maya_moe_down(C.byref(a), lib._stream()))
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    assert np.array_equal(outs[0], outs[1])
+    assert np.abs(outs[0]).max() > 0
