@@ -358,50 +358,43 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     const float inv = (float) (1.0 / sm.sum);
     for (int e = tid; e < n_expert; e += 256) sm.p[e] = (float) (sm.ex[e] * (double) inv);
     __syncthreads();
-    for (int i = 0; i < k; ++i) {
-        float bv = -INFINITY;
-        int bi = n_expert;
-        for (int e = tid; e < n_expert; e += 256) {
-            const float pe = sm.p[e];
-            if (pe > bv) {
-                bv = pe;
-                bi = e;
-            }
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, kWave);
-            const int oi = __shfl_xor(bi, o, kWave);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        if ((tid & 63) == 0) {
-            sm.rv[tid >> 6] = bv;
-            sm.ri[tid >> 6] = bi;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            float v = sm.rv[0];
-            int ix = sm.ri[0];
-            for (int w = 1; w < 4; ++w)
-                if (sm.rv[w] > v || (sm.rv[w] == v && sm.ri[w] < ix)) {
-                    v = sm.rv[w];
-                    ix = sm.ri[w];
+    // k rounds of arg-max by the first wave alone (no workgroup barriers): a lane scans its experts lane, lane + 64, ...
+    // in ascending order with a strict >, the wave folds (value, index) pairs preferring the lower index on ties, the
+    // winner is struck out of LDS (a probability is >= 0)
+    if (tid < 64) {
+        for (int i = 0; i < k; ++i) {
+            float bv = -INFINITY;
+            int bi = n_expert;
+            for (int e = tid; e < n_expert; e += 64) {
+                const float pe = sm.p[e];
+                if (pe > bv) {
+                    bv = pe;
+                    bi = e;
                 }
-            if (ix >= n_expert) ix = 0;  // only when every remaining probability is NaN
-            sm.id[i] = ix;
-            sm.w[i] = sm.p[ix];
-            sm.p[ix] = -INFINITY;  // taken: never selected again (a probability is >= 0)
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(bv, o, kWave);
+                const int oi = __shfl_xor(bi, o, kWave);
+                if (ov > bv || (ov == bv && oi < bi)) {
+                    bv = ov;
+                    bi = oi;
+                }
+            }
+            if (bi >= n_expert) bi = 0;  // only when every remaining probability is NaN
+            if (tid == 0) {
+                sm.id[i] = bi;
+                sm.w[i] = sm.p[bi];
+                sm.p[bi] = -INFINITY;
+            }
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_s_waitcnt(0);   // the strike-out is in LDS before the next round's scan
         }
-        __syncthreads();
-    }
-    if (tid == 0) {
+        // renormalisation: the sum of the k weights in slot order in double, one division a lane
         double s = 0.0;
         for (int i = 0; i < k; ++i) s += (double) sm.w[i];
         const double sc = fmax(s, 6.103515625e-05);
-        for (int i = 0; i < k; ++i) sm.w[i] = (float) ((double) sm.w[i] / sc);
+        if (tid < k) sm.w[tid] = (float) ((double) sm.w[tid] / sc);
     }
     __syncthreads();
 }
@@ -428,16 +421,28 @@ __global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict
                                                          int32_t* __restrict__ counters, int n_counters) {
     __shared__ RouterLds sm;
     __shared__ int qs[264];
+    __shared__ uint64_t s_table[MAYA_MAX_EXPERTS];
     const int t = blockIdx.y;
     if (blockIdx.x == 0) {
         if (t == 0)
             for (int i = threadIdx.x; i < n_counters; i += 256) counters[i] = 0;
+        // the residency table rides along in registers while the token is routed: the plan's look-up then costs no second
+        // trip to memory after the ids are known
+        uint64_t tab[MAYA_MAX_EXPERTS / 256];
+#pragma unroll
+        for (int i = 0; i < MAYA_MAX_EXPERTS / 256; ++i) {
+            const int e = threadIdx.x + 256 * i;
+            tab[i] = e < n_expert ? table[e] : 0ull;
+        }
         route_token(logits + (size_t) t * n_expert, n_expert, k, sm);
+#pragma unroll
+        for (int i = 0; i < MAYA_MAX_EXPERTS / 256; ++i) s_table[threadIdx.x + 256 * i] = tab[i];
+        __syncthreads();
         if (threadIdx.x < k) {
             const int id = sm.id[threadIdx.x];
             ids[(size_t) t * k + threadIdx.x] = id;
             weights[(size_t) t * k + threadIdx.x] = sm.w[threadIdx.x];
-            plan[(size_t) t * k + threadIdx.x] = (id >= 0 && id < n_expert) ? table[id] : 0ull;
+            plan[(size_t) t * k + threadIdx.x] = (id >= 0 && id < n_expert) ? s_table[id] : 0ull;
         }
     } else {
         const int b = blockIdx.x - 1, j = threadIdx.x;
