@@ -138,6 +138,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-graph", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", default="decode_iq2s",
+                    help="decode_iq2s (configs[1], the default and the headline metric), or one of the other BASELINE "
+                         "configurations: single_q4k, batch8_mixed, prefill_q4k, exl3_verify")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters by)")
@@ -155,6 +158,18 @@ def main():
     lib.check(L.maya_init())
     info = L.maya_device_info().decode()
     torch.cuda.set_device(0)
+    if args.workload != "decode_iq2s":
+        from maya_amd import workloads
+        if args.workload not in workloads.WORKLOADS:
+            sys.exit("bench.py: unknown workload %r" % args.workload)
+        r = workloads.WORKLOADS[args.workload](args.steps, args.warmup)
+        r["config"]["device"] = info
+        line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
+                "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
+                "cpu_baseline": None}
+        print(json.dumps(line))
+        return
     layer = lib.MoeLayer(IQ2_S, IQ2_S, N_EMBD, N_FF, N_EXPERT, TOP_K, max_tokens=1, packing=lib.PACK_STREAM)
     blob_bytes = layer.blob_bytes
     # GGUF blobs are made on the device, then regrouped into the stream packing as an engine's upload would do;

@@ -373,16 +373,17 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
     const int u = is_up ? t - NU : t;
+    const int tok = e / a.k;   // the entry's token: its activation row
     int y[8];
     {
-        const int4* q = (const int4*) a.x.q;
+        const int4* q = (const int4*) (a.x.q + (size_t) tok * (32 * NU));
         const int4 ya = q[2 * u], yb = q[2 * u + 1];
         y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
     }
     int yn[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
-    const float dy8 = a.x.d[u] * 0.125f;
+    const float dy8 = a.x.d[(size_t) tok * NU + u] * 0.125f;
     constexpr uint32_t qb = NU / 8 * 82 * 4;  // bytes of a quad of rows
     const int n_ff = a.layout.n_ff, r0 = blockIdx.x * ROWS;
     // one resource over the expert's gate and up rows; the up rows ride in the lane offset
@@ -462,21 +463,23 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r0 = blockIdx.x * ROWS;
-    const uint64_t blob = wave < a.k ? a.plan_ptr[wave] : 0ull;
+    const int e0 = blockIdx.y * a.k;   // the token's first entry; wave w = its slot w
+    const int ent = e0 + wave;
+    const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
     __syncthreads();
     if (blob != 0ull) {
         int y[8];
         float dy8;
         if (a.hq.q) {
-            const int4* q = (const int4*) (a.hq.q + (size_t) wave * 2048);
+            const int4* q = (const int4*) (a.hq.q + (size_t) ent * 2048);
             const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
             y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
-            dy8 = a.hq.d[(size_t) wave * 64 + lane] * 0.125f;
+            dy8 = a.hq.d[(size_t) ent * 64 + lane] * 0.125f;
         } else {
             // no rounded h given: the wave rounds its slot's h to Q8_K itself (quant_q8k_block's arithmetic): a lane holds
             // sub-block `lane`, a 256-value block is 8 lanes; the block's signed maximum is the value at the FIRST largest
             // magnitude - inside a lane the scan keeps the first, between lanes the lower lane wins a tie
-            const float4* hv = (const float4*) (a.h + (size_t) wave * 2048 + 32 * lane);
+            const float4* hv = (const float4*) (a.h + (size_t) ent * 2048 + 32 * lane);
             float v[32];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -552,16 +555,17 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         float sum = 0.0f;
         bool first = true;
         for (int i = 0; i < a.k; ++i) {
-            if (a.plan_ptr[i] == 0ull) continue;
-            const float p = __fmul_rn(part[i][c], a.plan_w[i]);
+            if (a.plan_ptr[e0 + i] == 0ull) continue;
+            const float p = __fmul_rn(part[i][c], a.plan_w[e0 + i]);
             sum = first ? p : __fadd_rn(sum, p);
             first = false;
         }
-        if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[r0 + c]);
-        a.out[r0 + c] = sum;
+        const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
+        if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
+        a.out[o] = sum;
         if (a.part)
             for (int i = 0; i < a.k; ++i)
-                if (a.plan_ptr[i] != 0ull) a.part[(size_t) i * n_embd + r0 + c] = part[i][c];
+                if (a.plan_ptr[e0 + i] != 0ull) a.part[(size_t) (e0 + i) * n_embd + r0 + c] = part[i][c];
     }
 }
 

@@ -781,6 +781,7 @@ __global__ __launch_bounds__(256) void combine_kernel(maya_moe_args a) {
 }  // namespace maya
 
 #include "maya_fast.cuh"
+#include "maya_fastk.cuh"
 
 namespace maya {
 
@@ -874,7 +875,7 @@ int launch_gate_up_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipS
 template <int NW>
 int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
-    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) a.k);
+    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) (a.n_tokens * a.k));   // an entry a column of the grid
     static const int variant = tuning_variant("MAYA_GU_VARIANT", 0);
     if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 2, 5>), grid, dim3(64 * NW), 0, s, a, st.cb);
     else if (variant == 2) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 32, 1, 8>), dim3(grid.x / 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
@@ -885,10 +886,10 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 }
 int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
-    const dim3 grid((unsigned) (a.layout.n_embd / kRows));
+    const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
     static const int variant = tuning_variant("MAYA_DN_VARIANT", 0);
     if (variant == 1) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 2, 5>), grid, dim3(512), 0, s, a, st.cb);
-    else if (variant == 2) hipLaunchKernelGGL((down_iq2s_pos_kernel<8, 1, 8>), dim3(grid.x * 2), dim3(512), 0, s, a, st.cb);
+    else if (variant == 2) hipLaunchKernelGGL((down_iq2s_pos_kernel<8, 1, 8>), dim3(grid.x * 2, grid.y), dim3(512), 0, s, a, st.cb);
     else if (variant == 3) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 8>), grid, dim3(512), 0, s, a, st.cb);
     else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);   // 8 waves a SIMD spill
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
@@ -909,6 +910,9 @@ int launch_down_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipStre
 // single-token IQ2_S gate/up: 1 launched, 0 no specialised kernel for this shape (the caller takes the general one)
 int try_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
     const maya_moe_layout& l = a.layout;
+    if (l.packing != MAYA_PACK_STREAM && !fast_1tok(a)) return 0;
+    // (the position-mapped kernels take the entries of several tokens one by one, whether grouped or not: every entry
+    // is computed as its token alone would compute it)
     if (l.packing == MAYA_PACK_STREAM) {
         if (l.n_ff % 16 != 0) return 0;
         switch (l.n_embd / 1024 * (l.n_embd % 1024 == 0)) {
@@ -926,7 +930,7 @@ int try_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStre
 // whether try_gate_up_iq2s_1tok would take the position-mapped kernel, which can round h itself (hq_sync)
 bool gate_up_fuses_hq(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && fast_1tok(a) && l.packing == MAYA_PACK_STREAM)) return false;
+    if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && a.n_tokens == 1 && l.packing == MAYA_PACK_STREAM)) return false;
     if (l.n_ff % 256 != 0 || l.n_embd % 1024 != 0 || !q8k_act(l.down_type)) return false;
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
@@ -934,12 +938,13 @@ bool gate_up_fuses_hq(const maya_moe_args& a) {
 // whether try_down_iq2s_1tok would take the position-mapped kernel, which can round h to Q8_K itself (hq.q == NULL)
 bool down_rounds_h(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    return l.down_type == kIQ2_S && fast_1tok(a) && a.k <= 8 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 &&
-           l.n_embd % 16 == 0;
+    if (l.down_type == kQ4_K) return l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
+    return l.down_type == kIQ2_S && a.k <= 8 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 && l.n_embd % 16 == 0;
 }
 int try_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
     const maya_moe_layout& l = a.layout;
     if (a.k > 8) return 0;
+    if (l.packing != MAYA_PACK_STREAM && !fast_1tok(a)) return 0;
     if (l.packing == MAYA_PACK_STREAM) {
         if (l.n_ff != 2048 || l.n_embd % 16 != 0) return 0;
         *rc = launch_down_iq2s_pos(a, st, s);
@@ -949,6 +954,48 @@ int try_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_
     *rc = launch_down_iq2s_gguf(a, st, s);
     return 1;
 }
+
+// ---- Q4_K in the stream packing (its own GGUF order, blobs 16-byte aligned): the position-mapped kernels
+bool gate_up_q4k_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (!(l.gate_type == kQ4_K && l.up_type == kQ4_K && l.packing == MAYA_PACK_STREAM)) return false;
+    if (l.n_embd % 1024 != 0 || l.n_ff % 16 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
+    const int nw = l.n_embd / 1024;
+    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+}
+bool down_q4k_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    return l.down_type == kQ4_K && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 &&
+           (l.down_off & 15) == 0;
+}
+int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
+    constexpr int kRows = 16;
+    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) (a.n_tokens * a.k));
+    switch (a.layout.n_embd / 1024) {
+        case 4: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<4, kRows, 8>), grid, dim3(256), 0, s, a); break;
+        case 6: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<6, kRows, 8>), grid, dim3(384), 0, s, a); break;
+        case 7: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<7, kRows, 8>), grid, dim3(448), 0, s, a); break;
+        default: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<8, kRows, 8>), grid, dim3(512), 0, s, a); break;
+    }
+    MAYA_LAUNCHED("gate_up_q4k_pos_kernel");
+    return MAYA_OK;
+}
+int launch_down_q4k_pos(const maya_moe_args& a, hipStream_t s) {
+    constexpr int kRows = 16;
+    const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
+    hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8>), grid, dim3(512), 0, s, a);
+    MAYA_LAUNCHED("down_q4k_pos_kernel");
+    return MAYA_OK;
+}
+// whether the gate/up (down) call is served entry by entry (no use for the groups of a window)
+bool gate_up_by_entries(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (gate_up_q4k_pos_ok(a)) return true;
+    if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM) || l.n_ff % 16 != 0 || l.n_embd % 1024 != 0) return false;
+    const int nw = l.n_embd / 1024;
+    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+}
+bool down_by_entries(const maya_moe_args& a) { return down_q4k_pos_ok(a) || down_rounds_h(a); }
 
 }  // namespace maya
 
@@ -1146,10 +1193,11 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
     hipStream_t s = as_stream(stream);
     const int tg = a->layout.gate_type, tu = a->layout.up_type;
-    if (tg == kIQ2_S && tu == kIQ2_S && fast_1tok(*a)) {
+    if (tg == kIQ2_S && tu == kIQ2_S) {
         int rc = 0;
         if (try_gate_up_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
+    if (gate_up_q4k_pos_ok(*a)) return launch_gate_up_q4k_pos(*a, s);
 #define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
     MAYA_GU(kIQ2_S, kIQ2_S)
     MAYA_GU(kQ4_K, kQ4_K)
@@ -1174,14 +1222,16 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     if (const int rc = check_args(a)) return rc;
     if (!a->hq.q && !a->hq.d && !a->hq.bsums && a->h && a->out && down_rounds_h(*a)) {
         int rc = 0;   // the kernel rounds h itself
+        if (a->layout.down_type == kQ4_K) return launch_down_q4k_pos(*a, as_stream(stream));
         if (try_down_iq2s_1tok(*a, *st, as_stream(stream), &rc)) return rc;
     }
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
     hipStream_t s = as_stream(stream);
-    if (a->layout.down_type == kIQ2_S && fast_1tok(*a)) {
+    if (a->layout.down_type == kIQ2_S) {
         int rc = 0;
         if (try_down_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
+    if (down_q4k_pos_ok(*a)) return launch_down_q4k_pos(*a, s);
     int rc;
     switch (a->layout.down_type) {
         case kIQ2_S: rc = launch_down_t<kIQ2_S>(*a, *st, s); break;
@@ -1282,7 +1332,7 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
         if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }
-    if (n_tokens > 1) {
+    if (n_tokens > 1 && !(gate_up_by_entries(a) && down_by_entries(a))) {
         if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
         a.grp_ptr = w.grp_ptr;
         a.grp_start = w.grp_start;

@@ -1,0 +1,230 @@
+"""The BASELINE configurations other than the decode layer that bench.py times by default: synthetic inputs made on the
+device, K steps captured as one HIP graph, and the algorithmic bytes / operations of a step.  Each function returns the
+fields bench.py prints (metric, value, unit, ms_per_step, config, roofline)."""
+import ctypes as C
+import time
+
+import numpy as np
+import torch
+
+from . import exl3, lib, prefill, synth
+
+HBM_PEAK = 8.0e12
+INT8_PEAK = 5.0e15
+
+
+def random_blocks(n_bytes, block, fields, seed):
+    """Random bytes in `block`-byte blocks whose FP16 fields (byte offset -> (lo, hi)) are drawn uniformly."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    assert n_bytes % block == 0
+    pool = torch.empty(n_bytes, dtype=torch.uint8, device="cuda")
+    step = 1 << 28
+    for o in range(0, n_bytes, step):
+        n = min(step, n_bytes - o)
+        pool[o:o + n] = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    blocks = pool.view(-1, block)
+    for off, (lo, hi) in fields.items():
+        d = (torch.rand(blocks.shape[0], device="cuda", generator=g) * (hi - lo) + lo).to(torch.float16)
+        blocks[:, off:off + 2] = d.view(torch.uint8).view(-1, 2)
+    return pool
+
+
+def timed_graph(step, K, W, stream):
+    """W eager warm-up steps, then K steps as one HIP graph, one untimed replay, one timed; seconds of the K steps."""
+    with torch.cuda.stream(stream):
+        for i in range(W):
+            step(i)
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(K):
+                step(W + i)
+        g.replay()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        g.replay()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+
+def event_time(fn, reps, stream):
+    """Average seconds of fn() over reps launches in one graph, HIP events on the launch stream."""
+    with torch.cuda.stream(stream):
+        fn()
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for _ in range(reps):
+                fn()
+        g.replay()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        g.replay()
+        e1.record(stream)
+        stream.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def hbm_roofline(kernel, bytes_launch, seconds):
+    rate = bytes_launch / seconds / 1e9
+    return {"bound": "hbm", "kernel": kernel, "achieved": round(rate, 2), "peak": 8000.0, "unit": "GB/s",
+            "frac": round(rate * 1e9 / HBM_PEAK, 4), "traffic": None, "algorithmic_bytes_per_launch": int(bytes_launch),
+            "avg_launch_us": round(seconds * 1e6, 3)}
+
+
+def single_q4k(K, W):
+    """configs[0]: one Q4_K expert GLU, one token, F32 activation; 16 copies of the expert rotate (396 MB > the on-die
+    caches)."""
+    E, FF, copies = 7168, 2048, 16
+    layer = lib.MoeLayer(lib.Q4_K, lib.Q4_K, E, FF, copies, 1, max_tokens=1, packing=lib.PACK_STREAM)   # (Q4_K: GGUF order, aligned)
+    bb = layer.blob_bytes
+    pool = random_blocks(copies * bb, 144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}, 5)
+    table = torch.tensor([pool.data_ptr() + e * bb for e in range(copies)], dtype=torch.int64, device="cuda")
+    logits = torch.full((copies, copies), -30.0, device="cuda")
+    logits.fill_diagonal_(0.0)
+    x = torch.randn(1, E, device="cuda")
+    stream = torch.cuda.Stream()
+    dt = timed_graph(lambda i: layer.forward(table, logits[i % copies:i % copies + 1], x), K, W, stream)
+    nbytes = bb + E * 4 + E * 4
+    sec = dt / K
+    return {"metric": "expert_glu_hbm_gbps_1tok", "value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "ms_per_step": sec * 1e3,
+            "dtype": "int8",
+            "config": {"workload": "configs[0]: one expert GLU, gate/up [2048x7168] + down [7168x2048] Q4_K (constructed "
+                                   "blocks), 1 token F32; 16 copies of the expert rotate over the steps",
+                       "algorithmic_bytes_per_step": nbytes},
+            "roofline": hbm_roofline("layer (head + gate_up_kernel<Q4_K> + quant + down_kernel<Q4_K> + combine)", nbytes, sec)}
+
+
+def batch8_mixed(K, W):
+    """configs[2]: 8 tokens, 256 experts top-8, gate/up IQ2_S + down Q4_K, and a Q8_0 shared expert every token takes."""
+    E, FF, NE, TK, T = 7168, 2048, 256, 8, 8
+    layer = lib.MoeLayer(lib.IQ2_S, lib.Q4_K, E, FF, NE, TK, max_tokens=T, packing=lib.PACK_STREAM)
+    bb = layer.blob_bytes
+    l = layer.gguf_layout
+    pool = torch.empty(NE * bb, dtype=torch.uint8, device="cuda")
+    view = pool.view(NE, bb)
+    gu = random_blocks(NE * l.down_off, 82, {0: (2e-3, 6e-3)}, 6).view(NE, l.down_off)
+    dn = random_blocks(NE * (bb - l.down_off), 144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}, 7).view(NE, bb - l.down_off)
+    view[:, :l.down_off] = gu
+    view[:, l.down_off:] = dn
+    del gu, dn
+    staging = torch.empty(bb, dtype=torch.uint8, device="cuda")
+    for e in range(NE):   # the engine's upload: every blob regrouped into the stream packing
+        staging.copy_(view[e])
+        lib.repack(l, staging, view[e])
+    torch.cuda.synchronize()
+    table = torch.tensor([pool.data_ptr() + e * bb for e in range(NE)], dtype=torch.int64, device="cuda")
+    shared = lib.MoeLayer(lib.Q8_0, lib.Q8_0, E, FF, 1, 1, max_tokens=T)
+    n_sh = 4   # copies of the shared expert rotate too (4 x 46.8 MB)
+    sh_pool = random_blocks(n_sh * shared.blob_bytes, 34, {0: (1e-4, 4e-4)}, 8)
+    sh_tables = [torch.tensor([sh_pool.data_ptr() + c * shared.blob_bytes], dtype=torch.int64, device="cuda") for c in range(n_sh)]
+    sh_logits = torch.zeros((T, 1), device="cuda")
+    rng = np.random.default_rng(9)
+    n_sets = 8
+    logits = torch.from_numpy(rng.standard_normal((n_sets, T, NE)).astype(np.float32)).cuda()
+    x = torch.randn(T, E, device="cuda")
+    distinct = []
+    for s in range(n_sets):
+        ids, _ = lib.route_topk(logits[s], TK)
+        distinct.append(int(torch.unique(ids).numel()))
+    stream = torch.cuda.Stream()
+
+    def step(i):
+        sh = shared.forward(sh_tables[i % n_sh], sh_logits, x)
+        layer.forward(table, logits[i % n_sets], x, add=sh)
+
+    dt = timed_graph(step, K, W, stream)
+    d_avg = float(np.mean([distinct[(W + i) % n_sets] for i in range(K)]))
+    nbytes = d_avg * bb + shared.blob_bytes + T * (E * 4 + E * 4)
+    sec = dt / K
+    return {"metric": "moe_layer_decode_hbm_gbps_8tok", "value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "ms_per_step": sec * 1e3,
+            "dtype": "int8",
+            "config": {"workload": "configs[2]: 8 tokens, 256 experts top-8 (gate/up IQ2_S, down Q4_K) + a Q8_0 shared expert; "
+                                   "8 logit sets rotate", "distinct_experts_per_step": d_avg,
+                       "algorithmic_bytes_per_step": int(nbytes)},
+            "roofline": hbm_roofline("layer (routed gate_up_kernel<IQ2_S,8 tok> + down_kernel<Q4_K> + shared Q8_0 expert)", nbytes, sec)}
+
+
+def prefill_q4k(K, W):
+    """configs[3]: 512 tokens, 256 Q4_K experts top-8, Zipf(1.1)-skewed routing, per-32 int8 activations, bf16 out."""
+    E, FF, NE, TK, T = 7168, 2048, 256, 8, 512
+    layout, bb = lib.layout(lib.Q4_K, lib.Q4_K, E, FF)
+    pool = random_blocks(NE * bb, 144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}, 11)
+    table = torch.tensor([pool.data_ptr() + e * bb for e in range(NE)], dtype=torch.int64, device="cuda")
+    rng = np.random.default_rng(12)
+    logits = torch.from_numpy((rng.standard_normal((T, NE)) + synth.zipf_bias(NE)).astype(np.float32)).cuda()
+    x = torch.randn(T, E, device="cuda")
+    layer = prefill.PrefillLayer(layout, NE, TK, T, out_dtype=torch.bfloat16)
+    stream = torch.cuda.Stream()
+    dt = timed_graph(lambda i: layer.forward(table, logits, x), K, W, stream)
+    sec = dt / K
+    ids, w = lib.route_topk(logits, TK)
+    used = int(torch.unique(ids).numel())
+    ops = 2 * 3 * E * FF * T * TK
+    nbytes = used * bb + T * E * (1 + 4 / 32) + T * E * 2
+    # the dominant kernel alone: the gate/up GEMM (2/3 of the operations)
+    with torch.cuda.stream(stream):
+        p = prefill.plan(ids.reshape(-1), table)
+        xq = prefill.quant(x, p, TK)
+        hq = prefill.ActRows(p.n_entries, FF)
+        L = prefill.load()
+        sec_gu = event_time(lambda: lib.check(L.maya_moe_prefill_gate_up(C.byref(layout), lib._p(table), NE, C.byref(p.c), p.n_entries,
+                                                                         xq.c, 0.0, hq.c, lib._stream())), 8, stream)
+    ops_gu = 2 * 2 * E * FF * T * TK
+    tops_gu = ops_gu / sec_gu / 1e12
+    return {"metric": "prefill_int8_tops_512tok", "value": round(ops / sec / 1e12, 2), "unit": "TOP/s", "ms_per_step": sec * 1e3,
+            "dtype": "int8",
+            "config": {"workload": "configs[3]: prefill chunk of 512 tokens, 256 experts Q4_K top-8, logits N(0,1) - 1.1 ln(e+1), "
+                                   "per-32 int8 activations, bf16 out", "experts_with_rows": used, "int8_ops_per_step": ops,
+                       "algorithmic_bytes_per_step": int(nbytes), "weight_gbps": round(nbytes / sec / 1e9, 1),
+                       "pct_of_hbm_peak": round(100 * nbytes / sec / HBM_PEAK, 2)},
+            "roofline": {"bound": "mfma", "kernel": "prefill_q4k_kernel<gate_up>", "achieved": round(tops_gu, 2), "peak": 5000.0,
+                         "unit": "TOP/s", "frac": round(tops_gu * 1e12 / INT8_PEAK, 4), "traffic": None,
+                         "algorithmic_ops_per_launch": ops_gu, "avg_launch_us": round(sec_gu * 1e6, 1)}}
+
+
+def exl3_verify(K, W):
+    """configs[4]: 160 EXL3 experts (3 bits a weight: k2 = 6, mul1 codebook), top-8, hidden 6144, intermediate 1536, a
+    4-token verify window; 8 logit sets rotate."""
+    E, FF, NE, TK, T = 6144, 1536, 160, 8, 4
+    l, bb = exl3.make_layout(E, FF, 6, exl3.CB_MUL1)
+    stride = (bb + 255) & ~255
+    pool = random_blocks(NE * stride, 256, {}, 13)
+    view = pool.view(NE, stride)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(14)
+    for r in range(3):
+        k, n = exl3.matrix_of(l, r)
+        suh = (torch.randint(0, 2, (NE, k), device="cuda", generator=g) * 2 - 1).to(torch.float16)
+        svh = ((torch.randint(0, 2, (NE, n), device="cuda", generator=g) * 2 - 1) *
+               (torch.rand((NE, n), device="cuda", generator=g) + 0.5) / (k ** 0.5)).to(torch.float16)
+        view[:, l.suh[r]:l.suh[r] + 2 * k] = suh.view(torch.uint8).view(NE, -1)
+        view[:, l.svh[r]:l.svh[r] + 2 * n] = svh.view(torch.uint8).view(NE, -1)
+    table = torch.tensor([pool.data_ptr() + e * stride for e in range(NE)], dtype=torch.int64, device="cuda")
+    layer = exl3.Exl3Layer(l, NE, TK, max_tokens=T)
+    rng = np.random.default_rng(15)
+    n_sets = 8
+    logits = torch.from_numpy(rng.standard_normal((n_sets, T, NE)).astype(np.float32)).cuda()
+    x = torch.randn(T, E, device="cuda").to(torch.float16).to(torch.float32)   # FP16 activations, handed over as F32
+    distinct = []
+    for s in range(n_sets):
+        ids, _ = lib.route_topk(logits[s], TK)
+        distinct.append(int(torch.unique(ids).numel()))
+    stream = torch.cuda.Stream()
+    dt = timed_graph(lambda i: layer.forward(table, logits[i % n_sets], x), K, W, stream)
+    d_avg = float(np.mean([distinct[(W + i) % n_sets] for i in range(K)]))
+    nbytes = d_avg * bb + T * (E * 4 + E * 4)
+    sec = dt / K
+    return {"metric": "exl3_moe_layer_hbm_gbps_4tok", "value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "ms_per_step": sec * 1e3,
+            "dtype": "f16",
+            "config": {"workload": "configs[4]: EXL3 3-bit trellis experts (k2 6, mul1), 160 experts top-8, hidden 6144, "
+                                   "intermediate 1536, 4-token verify window; 8 logit sets rotate",
+                       "distinct_experts_per_step": d_avg, "algorithmic_bytes_per_step": int(nbytes)},
+            "roofline": hbm_roofline("layer (exl3_gate_up_kernel + exl3_down_kernel + combine)", nbytes, sec)}
+
+
+WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify}

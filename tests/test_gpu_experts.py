@@ -52,6 +52,12 @@ CASES = [
     (22, 22, 7168, 1024, 10, 8, 1),
     (22, 22, 7168, 2048, 9, 8, 1),
     (22, 22, 14336, 1024, 4, 3, 1),
+    # the position-mapped kernels on several tokens' entries, and the Q4_K ones (stream packing; n_ff 2048 for down)
+    (22, 22, 4096, 2048, 12, 8, 5),
+    (12, 12, 4096, 2048, 6, 4, 1),
+    (12, 12, 7168, 2048, 5, 3, 4),
+    (22, 12, 6144, 2048, 9, 8, 3),
+    (12, 22, 8192, 2048, 4, 2, 2),
 ]
 
 
@@ -123,7 +129,7 @@ def test_zero_input_and_bf16_input(lib, oracle):
     assert np.array_equal(ids, wi) and rel_l2(out, wout) <= TOL
 
 
-@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3)))
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3), (22, 12, 4096, 2048, 7, 4, 4)))
 def test_window_rows_equal_token_rows(lib, gt, dt, n_embd, n_ff, ne, k, nt):
     """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract), in either
     row packing."""
@@ -133,13 +139,13 @@ def test_window_rows_equal_token_rows(lib, gt, dt, n_embd, n_ff, ne, k, nt):
     x = rng.standard_normal((nt, n_embd)).astype(np.float32)
     _, _, win, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x)
     _, _, winp, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=1)
-    assert np.array_equal(win.view(np.uint32), winp.view(np.uint32))
     for t in range(nt):
         _, _, one, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits[t:t + 1], x[t:t + 1])
         assert np.array_equal(win[t].view(np.uint32), one[0].view(np.uint32)), t
-        # the stream packing's single-token kernels sum a row's sub-blocks in another order: same integers, float
-        # sums that differ in their last bits (and, rarely, one Q8_K code of h): held to the parity bar, not to the bit
         _, _, onep, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits[t:t + 1], x[t:t + 1], packing=1)
+        assert np.array_equal(winp[t].view(np.uint32), onep[0].view(np.uint32)), t
+        # the stream packing's kernels sum a row's sub-blocks in another order than the GGUF packing's: same integers,
+        # float sums that differ in their last bits (and, rarely, one Q8_K code of h): held to the parity bar
         assert rel_l2(onep[0], win[t]) <= TOL, t
 
 
