@@ -275,7 +275,8 @@ typedef struct maya_exl3_args {
     const float* x;     /* [n_tokens][x_stride] F32 */
     int64_t x_stride;   /* floats between tokens (0: n_embd) */
     float* h;           /* [n_tokens*k][n_ff] */
-    float* part;        /* [n_tokens*k][n_embd] */
+    float* part;        /* [n_tokens*k][n_embd]: down's per-entry outputs; given to maya_exl3_gate_up it also serves as
+                         * scratch for gate/up's partial outputs (the faster, split form); NULL there: the fused form */
     const float* add;   /* NULL or [n_tokens][n_embd] (shared expert / CPU lane part) */
     const int32_t* add_flag;
     float* out;         /* [n_tokens][n_embd] */

@@ -12,6 +12,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "maya_host.h"
 
 namespace maya {
@@ -155,6 +157,96 @@ __device__ __forceinline__ void walk_tiles(const uint32_t* __restrict__ trellis,
     }
 }
 
+// ---- the same walk with the bit rate a compile-time constant (K2 <= 10, the mul1 codebook): no LDS staging of the tile.
+// A lane's 4 windows span 16 + 3 K2 / 2 <= 31 bits, so they sit in the two words around the last window's end - two
+// dword buffer loads at lane-constant offsets, the tile's address in the scalar offset - and one 64-bit shift puts all
+// four into one register, where they are bit-field extracts at compile-time positions.  1024 + the byte sum is an FP16
+// whose bit pattern is 0x6400 + the byte sum (one v_sad_u8); values are made two at a time (v_pk_fma_f16) and meet the
+// FP16 activation pairs (rows 2q, 2q+1 and 2q+8, 2q+9 are adjacent) in v_dot2_f32_f16.
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+template <int K2> struct Taps {
+    static constexpr int end(int i) { return ((i + 1) * K2) / 2; }       // end bit of step i above the lane's 2 L K2
+    static constexpr int below(int i) { return end(3) - end(i); }        // how far window i ends before the last one
+};
+__device__ __forceinline__ h2 as_h2(uint32_t v) {
+    union { uint32_t u; h2 h; } c;
+    c.u = v;
+    return c.h;
+}
+template <int K2>
+__device__ __forceinline__ void tile_values(uint32_t wa, uint32_t wb, int sh, h2& w01, h2& w23) {
+    const uint32_t c = (uint32_t) ((((uint64_t) wa << 32) | (uint64_t) wb) >> sh);
+    uint32_t hb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t st = __builtin_amdgcn_ubfe(c, Taps<K2>::below(i), 16);
+        hb[i] = __builtin_amdgcn_sad_u8(st * 0x83DCD12Du, 0u, 0x6400u);   // the bits of FP16(1024 + byte sum)
+    }
+    const h2 kinv = as_h2(0x1eee1eeeu), kbias = as_h2(0xc931c931u);
+    w01 = __builtin_elementwise_fma(as_h2(hb[0] | (hb[1] << 16)), kinv, kbias);
+    w23 = __builtin_elementwise_fma(as_h2(hb[2] | (hb[3] << 16)), kinv, kbias);
+}
+template <int K2, int NT>
+__device__ __forceinline__ void walk_tiles_fast(const uint32_t* __restrict__ trellis, int k, int ld, int tc, int lane,
+                                                const __half* xr, int xr_stride, float (&acc)[NT]) {
+    static_assert(K2 >= 2 && K2 <= 10, "the four windows of a lane must fit 32 bits");
+    constexpr int W = 4 * K2;
+    const int E = 2 * lane * K2 + Taps<K2>::end(3);   // the end bit of the lane's last window: 1 .. 128 K2
+    const int ib = (E - 1) >> 5, ia = ib == 0 ? W - 1 : ib - 1;
+    const int sh = 32 * (ib + 1) - E;
+    const int q = (lane >> 1) & 3, nks = k >> 4;
+    const uint64_t base = (uint64_t) trellis;
+    const uint32_t b_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) base);
+    const uint32_t b_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (base >> 32));
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*) (((uint64_t) b_hi << 32) | b_lo), 0,
+                                                                         (int) ((uint32_t) nks * ld * W * 4), 0x00020000);
+    const uint32_t oa = 4u * ia, ob = 4u * ib, step = (uint32_t) ld * W * 4;
+    // (tc comes from the wave's index: uniform, but only readfirstlane tells the compiler so - a divergent scalar offset
+    // would turn every load into a loop over the lanes)
+    const uint32_t t_off = (uint32_t) __builtin_amdgcn_readfirstlane(tc) * W * 4;
+    // A wave's row tiles are ld * W * 4 bytes apart (a 96-byte read every 9 KB at 3 bits a weight): only many reads in
+    // flight keep the memory busy, so the walk runs kAhead tiles ahead in a ring of registers.
+    constexpr int kAhead = 8;   // (k is a multiple of 128: the row tiles come in eights)
+    uint32_t ra[kAhead], rb[kAhead];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+        ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, oa, t_off + (uint32_t) i * step, 0);
+        rb[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, ob, t_off + (uint32_t) i * step, 0);
+    }
+    const uint32_t* xw = (const uint32_t*) xr;   // pairs of FP16 activations
+    const int xs = xr_stride >> 1;
+#pragma unroll 1
+    for (int ks = 0; ks < nks; ks += kAhead) {
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            const uint32_t ca = ra[i], cb = rb[i];
+            const uint32_t nxt = t_off + (uint32_t) (ks + i + kAhead) * step;   // (past the matrix: the buffer returns 0)
+            ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, oa, nxt, 0);
+            rb[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, ob, nxt, 0);
+            h2 w01, w23;
+            tile_values<K2>(ca, cb, sh, w01, w23);
+            const int rw = (ks + i) * 8 + q;   // the word of rows 2q, 2q + 1 of this row tile
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                acc[t] = __builtin_amdgcn_fdot2(w01, as_h2(xw[t * xs + rw]), acc[t], false);
+                acc[t] = __builtin_amdgcn_fdot2(w23, as_h2(xw[t * xs + rw + 4]), acc[t], false);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        acc[t] += __shfl_xor(acc[t], 2, 64);
+        acc[t] += __shfl_xor(acc[t], 4, 64);
+    }
+}
+// K2 > 0: the compile-time walk; 0: the general one
+template <int CB, int NT, int K2>
+__device__ __forceinline__ void walk(const uint32_t* __restrict__ trellis, int k, int ld, int tc, int k2, int lane,
+                                     uint32_t* wt, const __half* xr, int xr_stride, float (&acc)[NT]) {
+    if constexpr (K2 > 0) walk_tiles_fast<K2, NT>(trellis, k, ld, tc, lane, xr, xr_stride, acc);
+    else walk_tiles<CB, NT>(trellis, k, ld, tc, k2, lane, wt, xr, xr_stride, acc);
+}
+
 __device__ __forceinline__ float ex_swiglu(float g, float u, float limit) {
     if (limit > 0.0f && limit < INFINITY) {
         g = fminf(g, limit);
@@ -165,7 +257,7 @@ __device__ __forceinline__ float ex_swiglu(float g, float u, float limit) {
 
 // dynamic LDS: [8 waves x 64 words of tile][NT x 2 x k halves of rotated inputs][max(k, NT*2*128) floats of scratch]
 // grid (n_ff / 128, groups)
-template <int CB, int NT>
+template <int CB, int NT, int K2>
 __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args a) {
     extern __shared__ uint32_t lds[];
     ExGroup gr;
@@ -178,54 +270,135 @@ __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args
     const int64_t xs = a.x_stride ? a.x_stride : k;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int tc = blockIdx.x * 8 + wave;
-    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
-        int ents[NT];
+    // the group's entries two at a time while two are left (one decode of the weights serves both), else one
+    auto chunk = [&](auto ntc, int c0) {
+        constexpr int NTC = decltype(ntc)::value;
+        int ents[NTC];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? ex_entry_of(a, gr, c0 + t) : -1;
+        for (int t = 0; t < NTC; ++t) ents[t] = ex_entry_of(a, gr, c0 + t);
         __syncthreads();
-        for (int t = 0; t < NT; ++t) {
-            if (ents[t] < 0) continue;
+        for (int t = 0; t < NTC; ++t) {
             const float* x = a.x + (size_t) (ents[t] / a.k) * xs;
             for (int role = 0; role < 2; ++role)
                 rotate_in(x, (const uint16_t*) (blob + a.layout.suh[role]), k, tmp, xr + ((size_t) t * 2 + role) * k);
         }
-        float raw[2][NT];
+        float raw[2][NTC];
 #pragma unroll
         for (int role = 0; role < 2; ++role) {
-            float acc[NT];
+            float acc[NTC];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
-            walk_tiles<CB, NT>((const uint32_t*) (blob + a.layout.trellis[role]), k, n >> 4, tc, a.layout.k2[role], lane, wt,
-                               xr + (size_t) role * k, 2 * k, acc);
+            for (int t = 0; t < NTC; ++t) acc[t] = 0.0f;
+            walk<CB, NTC, K2>((const uint32_t*) (blob + a.layout.trellis[role]), k, n >> 4, tc, a.layout.k2[role], lane, wt,
+                              xr + (size_t) role * k, 2 * k, acc);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) raw[role][t] = acc[t];
+            for (int t = 0; t < NTC; ++t) raw[role][t] = acc[t];
         }
         __syncthreads();
         // the lane with q = 0 of each column holds the sums: column (L >> 3) + 8 (L & 1) of the wave's tile
         if (((lane >> 1) & 3) == 0) {
             const int col = wave * 16 + (lane >> 3) + 8 * (lane & 1);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
+            for (int t = 0; t < NTC; ++t) {
                 tmp[(t * 2 + 0) * 128 + col] = raw[0][t];
                 tmp[(t * 2 + 1) * 128 + col] = raw[1][t];
             }
         }
         __syncthreads();
-        had128_lds(tmp, NT * 2);
+        had128_lds(tmp, NTC * 2);
         const uint16_t* svg = (const uint16_t*) (blob + a.layout.svh[0]) + blockIdx.x * 128;
         const uint16_t* svu = (const uint16_t*) (blob + a.layout.svh[1]) + blockIdx.x * 128;
-        for (int i = threadIdx.x; i < NT * 128; i += kExThreads) {
+        for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
             const int t = i >> 7, c = i & 127;
-            if (ents[t] < 0) continue;
             const float g = __fmul_rn(tmp[(t * 2 + 0) * 128 + c], f16_bits_to_f32(svg[c]));
             const float u = __fmul_rn(tmp[(t * 2 + 1) * 128 + c], f16_bits_to_f32(svu[c]));
             a.h[(size_t) ents[t] * n + blockIdx.x * 128 + c] = ex_swiglu(g, u, a.limit);
         }
+    };
+    for (int c0 = 0; c0 < gr.ne;) {
+        if (NT >= 2 && gr.ne - c0 >= 2) {
+            chunk(std::integral_constant<int, 2>{}, c0);
+            c0 += 2;
+        } else {
+            chunk(std::integral_constant<int, 1>{}, c0);
+            c0 += 1;
+        }
     }
 }
 
+// ---- gate/up split over more workgroups (the compile-time walk only): grid (n_ff / 128, groups, 2 KS), z = role KS + ks.
+// A workgroup takes one role (gate or up) and one of KS slices of the rows: it rotates its slice of the input, walks
+// its row tiles, rotates the 128 partial sums and scales them - rotation and scaling are linear, so the slices' partial
+// outputs simply add - and stores them to P[entry][role][ks][n_ff] (the caller's `part` scratch).  exl3_swiglu_kernel adds the
+// slices and applies the SwiGLU.  Twice 2 KS as many, shorter workgroups as the fused kernel: the chip fills evenly.
+// dynamic LDS: [NT x k/KS halves of rotated input][max(k/KS, NT*128) floats of scratch]
+template <int NT, int K2>
+__global__ __launch_bounds__(kExThreads) void exl3_gu_split_kernel(maya_exl3_args a, int KS) {
+    extern __shared__ uint32_t lds[];
+    ExGroup gr;
+    if (!ex_group_of(a, blockIdx.y, gr)) return;
+    const int role = blockIdx.z / KS, ks = blockIdx.z % KS;
+    const int k = a.layout.n_embd, n = a.layout.n_ff, kb = k / KS;
+    __half* xr = (__half*) lds;                         // [NT][kb]
+    float* tmp = (float*) (xr + (size_t) NT * kb);      // kb floats; later [NT][128]
+    const uint8_t* blob = (const uint8_t*) gr.blob;
+    const int64_t xs = a.x_stride ? a.x_stride : k;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tc = blockIdx.x * 8 + wave, ld = n >> 4;
+    const uint32_t* trellis = (const uint32_t*) (blob + a.layout.trellis[role]) + (size_t) ks * (kb >> 4) * ld * (4 * K2);
+    const uint16_t* suh = (const uint16_t*) (blob + a.layout.suh[role]) + (size_t) ks * kb;
+    const uint16_t* sv = (const uint16_t*) (blob + a.layout.svh[role]) + blockIdx.x * 128;
+    auto chunk = [&](auto ntc, int c0) {
+        constexpr int NTC = decltype(ntc)::value;
+        int ents[NTC];
+#pragma unroll
+        for (int t = 0; t < NTC; ++t) ents[t] = ex_entry_of(a, gr, c0 + t);
+        __syncthreads();
+        for (int t = 0; t < NTC; ++t)
+            rotate_in(a.x + (size_t) (ents[t] / a.k) * xs + (size_t) ks * kb, suh, kb, tmp, xr + (size_t) t * kb);
+        float acc[NTC];
+#pragma unroll
+        for (int t = 0; t < NTC; ++t) acc[t] = 0.0f;
+        walk_tiles_fast<K2, NTC>(trellis, kb, ld, tc, lane, xr, kb, acc);
+        __syncthreads();
+        if (((lane >> 1) & 3) == 0) {
+            const int col = wave * 16 + (lane >> 3) + 8 * (lane & 1);
+#pragma unroll
+            for (int t = 0; t < NTC; ++t) tmp[t * 128 + col] = acc[t];
+        }
+        __syncthreads();
+        had128_lds(tmp, NTC);
+        for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
+            const int t = i >> 7, c = i & 127;
+            a.part[(((size_t) ents[t] * 2 + role) * KS + ks) * n + blockIdx.x * 128 + c] = __fmul_rn(tmp[t * 128 + c], f16_bits_to_f32(sv[c]));
+        }
+    };
+    for (int c0 = 0; c0 < gr.ne;) {
+        if (NT >= 2 && gr.ne - c0 >= 2) {
+            chunk(std::integral_constant<int, 2>{}, c0);
+            c0 += 2;
+        } else {
+            chunk(std::integral_constant<int, 1>{}, c0);
+            c0 += 1;
+        }
+    }
+}
+// grid (n_ff / 256, entries): h = the clamped SwiGLU of the slices' sums (slice 0 first)
+__global__ __launch_bounds__(256) void exl3_swiglu_kernel(maya_exl3_args a, int KS) {
+    if (a.skip && *a.skip) return;
+    const int e = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x, n = a.layout.n_ff;
+    if (c >= n || a.plan_ptr[e] == 0ull) return;
+    const float* pg = a.part + ((size_t) e * 2 + 0) * KS * n + c;
+    const float* pu = a.part + ((size_t) e * 2 + 1) * KS * n + c;
+    float g = pg[0], u = pu[0];
+    for (int s = 1; s < KS; ++s) {
+        g = __fadd_rn(g, pg[(size_t) s * n]);
+        u = __fadd_rn(u, pu[(size_t) s * n]);
+    }
+    a.h[(size_t) e * n + c] = ex_swiglu(g, u, a.limit);
+}
+
 // grid (n_embd / 128, groups): part[e][columns] = the down product of h[e]
-template <int CB, int NT>
+template <int CB, int NT, int K2>
 __global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a) {
     extern __shared__ uint32_t lds[];
     ExGroup gr;
@@ -237,31 +410,39 @@ __global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a)
     const uint8_t* blob = (const uint8_t*) gr.blob;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int tc = blockIdx.x * 8 + wave;
-    for (int c0 = 0; c0 < gr.ne; c0 += NT) {
-        int ents[NT];
+    auto chunk = [&](auto ntc, int c0) {
+        constexpr int NTC = decltype(ntc)::value;
+        int ents[NTC];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? ex_entry_of(a, gr, c0 + t) : -1;
+        for (int t = 0; t < NTC; ++t) ents[t] = ex_entry_of(a, gr, c0 + t);
         __syncthreads();
-        for (int t = 0; t < NT; ++t)
-            if (ents[t] >= 0)
-                rotate_in(a.h + (size_t) ents[t] * k, (const uint16_t*) (blob + a.layout.suh[2]), k, tmp, xr + (size_t) t * k);
-        float acc[NT];
+        for (int t = 0; t < NTC; ++t)
+            rotate_in(a.h + (size_t) ents[t] * k, (const uint16_t*) (blob + a.layout.suh[2]), k, tmp, xr + (size_t) t * k);
+        float acc[NTC];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
-        walk_tiles<CB, NT>((const uint32_t*) (blob + a.layout.trellis[2]), k, n >> 4, tc, a.layout.k2[2], lane, wt, xr, k, acc);
+        for (int t = 0; t < NTC; ++t) acc[t] = 0.0f;
+        walk<CB, NTC, K2>((const uint32_t*) (blob + a.layout.trellis[2]), k, n >> 4, tc, a.layout.k2[2], lane, wt, xr, k, acc);
         __syncthreads();
         if (((lane >> 1) & 3) == 0) {
             const int col = wave * 16 + (lane >> 3) + 8 * (lane & 1);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) tmp[t * 128 + col] = acc[t];
+            for (int t = 0; t < NTC; ++t) tmp[t * 128 + col] = acc[t];
         }
         __syncthreads();
-        had128_lds(tmp, NT);
+        had128_lds(tmp, NTC);
         const uint16_t* sv = (const uint16_t*) (blob + a.layout.svh[2]) + blockIdx.x * 128;
-        for (int i = threadIdx.x; i < NT * 128; i += kExThreads) {
+        for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
             const int t = i >> 7, c = i & 127;
-            if (ents[t] < 0) continue;
             a.part[(size_t) ents[t] * n + blockIdx.x * 128 + c] = __fmul_rn(tmp[t * 128 + c], f16_bits_to_f32(sv[c]));
+        }
+    };
+    for (int c0 = 0; c0 < gr.ne;) {
+        if (NT >= 2 && gr.ne - c0 >= 2) {
+            chunk(std::integral_constant<int, 2>{}, c0);
+            c0 += 2;
+        } else {
+            chunk(std::integral_constant<int, 1>{}, c0);
+            c0 += 1;
         }
     }
 }
@@ -309,17 +490,71 @@ int launch_exl3_gate_up(const maya_exl3_args& a, const DeviceState& st, hipStrea
     const size_t lds = 8 * 64 * 4 + (size_t) NT * 2 * k * 2 + scratch;
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
     const dim3 grid((unsigned) (a.layout.n_ff / 128), (unsigned) (a.n_tokens * a.k));
-#define MAYA_EX(CBV)                                                                                              \
+#define MAYA_EX(CBV, K2V)                                                                                         \
     {                                                                                                             \
-        auto kern = exl3_gate_up_kernel<CBV, NT>;                                                                 \
+        auto kern = exl3_gate_up_kernel<CBV, NT, K2V>;                                                            \
         if (lds > 65536) MAYA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
         hipLaunchKernelGGL(kern, grid, dim3(kExThreads), lds, s, a);                                              \
     }
-    if (a.layout.cb == 2) MAYA_EX(2) else if (a.layout.cb == 1) MAYA_EX(1) else MAYA_EX(0)
+    // the compile-time walk: mul1, gate and up at one bit rate of at most 5 bits a weight
+    const int k2f = a.layout.cb == 2 && a.layout.k2[0] == a.layout.k2[1] && a.layout.k2[0] <= 10 ? a.layout.k2[0] : 0;
+    switch (k2f) {
+        case 2: MAYA_EX(2, 2) break;
+        case 3: MAYA_EX(2, 3) break;
+        case 4: MAYA_EX(2, 4) break;
+        case 5: MAYA_EX(2, 5) break;
+        case 6: MAYA_EX(2, 6) break;
+        case 7: MAYA_EX(2, 7) break;
+        case 8: MAYA_EX(2, 8) break;
+        case 10: MAYA_EX(2, 10) break;
+        default:
+            if (a.layout.cb == 2) MAYA_EX(2, 0) else if (a.layout.cb == 1) MAYA_EX(1, 0) else MAYA_EX(0, 0)
+    }
 #undef MAYA_EX
     MAYA_LAUNCHED("exl3_gate_up_kernel");
     return MAYA_OK;
 }
+// the split gate/up when it applies (mul1, one bit rate <= 5 bits for gate and up, `part` given and large enough for the
+// partial outputs): 1 launched, 0 not applicable
+template <int NT>
+int try_exl3_gu_split(const maya_exl3_args& a, const DeviceState& st, hipStream_t s, int* rc) {
+    const maya_exl3_layout& l = a.layout;
+    if (l.cb != 2 || l.k2[0] != l.k2[1] || l.k2[0] > 10 || !a.part) return 0;
+    const int KS = (l.n_embd % 256 == 0 && l.n_embd >= 4 * l.n_ff) ? 2 : (l.n_embd >= 2 * l.n_ff ? 1 : 0);
+    if (KS == 0) return 0;
+    const int kb = l.n_embd / KS;
+    const size_t lds = (size_t) NT * kb * 2 + (size_t) (kb > NT * 128 ? kb : NT * 128) * 4;
+    if (lds > (size_t) st.lds_limit) return 0;
+    const dim3 grid((unsigned) (l.n_ff / 128), (unsigned) (a.n_tokens * a.k), (unsigned) (2 * KS));
+#define MAYA_EX(K2V)                                                                                              \
+    {                                                                                                             \
+        auto kern = exl3_gu_split_kernel<NT, K2V>;                                                                \
+        if (lds > 65536) {                                                                                        \
+            const hipError_t e_ = hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds); \
+            if (e_ != hipSuccess) { *rc = hip_fail(e_, "hipFuncSetAttribute"); return 1; }                        \
+        }                                                                                                         \
+        hipLaunchKernelGGL(kern, grid, dim3(kExThreads), lds, s, a, KS);                                          \
+    }
+    switch (l.k2[0]) {
+        case 2: MAYA_EX(2) break;
+        case 3: MAYA_EX(3) break;
+        case 4: MAYA_EX(4) break;
+        case 5: MAYA_EX(5) break;
+        case 6: MAYA_EX(6) break;
+        case 7: MAYA_EX(7) break;
+        case 8: MAYA_EX(8) break;
+        case 10: MAYA_EX(10) break;
+        default: return 0;
+    }
+#undef MAYA_EX
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { *rc = hip_fail(e, "exl3_gu_split_kernel"); return 1; }
+    hipLaunchKernelGGL(exl3_swiglu_kernel, dim3((unsigned) ((l.n_ff + 255) / 256), (unsigned) (a.n_tokens * a.k)), dim3(256), 0, s, a, KS);
+    e = hipGetLastError();
+    *rc = e != hipSuccess ? hip_fail(e, "exl3_swiglu_kernel") : MAYA_OK;
+    return 1;
+}
+
 template <int NT>
 int launch_exl3_down(const maya_exl3_args& a, const DeviceState& st, hipStream_t s) {
     const int k = a.layout.n_ff;
@@ -327,13 +562,25 @@ int launch_exl3_down(const maya_exl3_args& a, const DeviceState& st, hipStream_t
     const size_t lds = 8 * 64 * 4 + (size_t) NT * k * 2 + scratch;
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
     const dim3 grid((unsigned) (a.layout.n_embd / 128), (unsigned) (a.n_tokens * a.k));
-#define MAYA_EX(CBV)                                                                                              \
+#define MAYA_EX(CBV, K2V)                                                                                         \
     {                                                                                                             \
-        auto kern = exl3_down_kernel<CBV, NT>;                                                                    \
+        auto kern = exl3_down_kernel<CBV, NT, K2V>;                                                               \
         if (lds > 65536) MAYA_HIP(hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
         hipLaunchKernelGGL(kern, grid, dim3(kExThreads), lds, s, a);                                              \
     }
-    if (a.layout.cb == 2) MAYA_EX(2) else if (a.layout.cb == 1) MAYA_EX(1) else MAYA_EX(0)
+    const int k2f = a.layout.cb == 2 && a.layout.k2[2] <= 10 ? a.layout.k2[2] : 0;
+    switch (k2f) {
+        case 2: MAYA_EX(2, 2) break;
+        case 3: MAYA_EX(2, 3) break;
+        case 4: MAYA_EX(2, 4) break;
+        case 5: MAYA_EX(2, 5) break;
+        case 6: MAYA_EX(2, 6) break;
+        case 7: MAYA_EX(2, 7) break;
+        case 8: MAYA_EX(2, 8) break;
+        case 10: MAYA_EX(2, 10) break;
+        default:
+            if (a.layout.cb == 2) MAYA_EX(2, 0) else if (a.layout.cb == 1) MAYA_EX(1, 0) else MAYA_EX(0, 0)
+    }
 #undef MAYA_EX
     MAYA_LAUNCHED("exl3_down_kernel");
     return MAYA_OK;
@@ -369,6 +616,8 @@ int maya_exl3_gate_up(const maya_exl3_args* a, void* stream) {
     if (const int rc = exl3_check(a)) return rc;
     if (!a->x || !a->h) return fail(MAYA_E_ARG, "exl3 gate_up: null x or h");
     const int nt = a->grp_ptr && a->n_tokens >= 2 ? 2 : 1;
+    int rc = 0;
+    if (nt == 2 ? try_exl3_gu_split<2>(*a, *st, as_stream(stream), &rc) : try_exl3_gu_split<1>(*a, *st, as_stream(stream), &rc)) return rc;
     return nt == 2 ? launch_exl3_gate_up<2>(*a, *st, as_stream(stream)) : launch_exl3_gate_up<1>(*a, *st, as_stream(stream));
 }
 
