@@ -650,12 +650,19 @@ __device__ __forceinline__ float swiglu(float g, float u, float limit) {
     return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
 }
 
-constexpr int kGuThreads = 512, kGuRows = 32;   // a workgroup: 8 waves, 32 gate + 32 up rows
-constexpr int kDnThreads = 512, kDnRows = 64;   // 8 waves x 2 rows a pass, 4 passes
+constexpr int kGuThreads = 512, kGuRows = 32;   // a workgroup: 8 waves, at most 32 gate + 32 up rows
+constexpr int kDnThreads = 512, kDnRows = 64;   // 8 waves x 2 rows a pass, at most 4 passes
+// rows a workgroup takes (a multiple of `unit`, at most `most`): fewer when the call has few entries - a shared expert,
+// a single token - so that the grid still covers the chip
+inline int rows_per_wg(int n_rows, int entries, int unit, int most) {
+    int r = most;
+    while (r > unit && (long long) ((n_rows + r - 1) / r) * entries < 1024) r >>= 1;
+    return r < unit ? unit : r;
+}
 
 // grid (n_ff / kGuRows, groups): wave w takes row pairs w, w + 8, ...: lanes 0..31 the gate row, 32..63 the up row
 template <int TG, int TU, int NT>
-__global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Codebooks cb) {
+__global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Codebooks cb, int wg_rows) {
     extern __shared__ int lds[];
     GroupRef gr;
     if (!group_of(a, blockIdx.y, gr)) return;
@@ -691,7 +698,7 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
         __syncthreads();
         stage_act<TG, NT>(lds_act, k, a.x, rows, Fmt<TG>::kMin || Fmt<TU>::kMin);
         __syncthreads();
-        for (int r = blockIdx.x * kGuRows + wave; r < min(n_ff, (int) (blockIdx.x + 1) * kGuRows); r += kGuThreads / 64) {
+        for (int r = blockIdx.x * wg_rows + wave; r < min(n_ff, (int) (blockIdx.x + 1) * wg_rows); r += kGuThreads / 64) {
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
@@ -719,7 +726,7 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
 // grid (n_embd / kDnRows, groups): a wave takes 2 rows a pass, 32 lanes a row (the single-token kernel's split of a
 // row over lanes, so a window's rows get the token path's bits)
 template <int TD, int NT>
-__global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codebooks cb) {
+__global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codebooks cb, int wg_rows) {
     extern __shared__ int lds[];
     GroupRef gr;
     if (!group_of(a, blockIdx.y, gr)) return;
@@ -744,8 +751,8 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
         __syncthreads();
         stage_act<TD, NT>(lds_act, k, a.hq, ents, Fmt<TD>::kMin);
         __syncthreads();
-        const int r_end = min(n_embd, (int) (blockIdx.x + 1) * kDnRows);
-        for (int r = blockIdx.x * kDnRows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
+        const int r_end = min(n_embd, (int) (blockIdx.x + 1) * wg_rows);
+        for (int r = blockIdx.x * wg_rows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
@@ -833,10 +840,11 @@ int launch_gate_up_t(const maya_moe_args& a, const DeviceState& st, hipStream_t 
     const int cbw = codebook_words(TG) + (codebook_words(TG) == codebook_words(TU) ? 0 : codebook_words(TU));
     const size_t lds = (size_t) cbw * 4 + act_lds_bytes(a.layout.n_embd, nt);
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
-    const dim3 grid((unsigned) ((a.layout.n_ff + kGuRows - 1) / kGuRows), (unsigned) (a.n_tokens * a.k));
-    if (nt == 4) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 4>), grid, dim3(kGuThreads), lds, s, a, st.cb);
-    else if (nt == 2) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 2>), grid, dim3(kGuThreads), lds, s, a, st.cb);
-    else hipLaunchKernelGGL((gate_up_kernel<TG, TU, 1>), grid, dim3(kGuThreads), lds, s, a, st.cb);
+    const int wr = rows_per_wg(a.layout.n_ff, a.n_tokens * a.k, 8, kGuRows);
+    const dim3 grid((unsigned) ((a.layout.n_ff + wr - 1) / wr), (unsigned) (a.n_tokens * a.k));
+    if (nt == 4) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 4>), grid, dim3(kGuThreads), lds, s, a, st.cb, wr);
+    else if (nt == 2) hipLaunchKernelGGL((gate_up_kernel<TG, TU, 2>), grid, dim3(kGuThreads), lds, s, a, st.cb, wr);
+    else hipLaunchKernelGGL((gate_up_kernel<TG, TU, 1>), grid, dim3(kGuThreads), lds, s, a, st.cb, wr);
     MAYA_LAUNCHED("gate_up_kernel");
     return MAYA_OK;
 }
@@ -845,10 +853,11 @@ int launch_down_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) 
     const int nt = a.grp_ptr ? (a.n_tokens >= 4 ? 4 : a.n_tokens >= 2 ? 2 : 1) : 1;
     const size_t lds = (size_t) codebook_words(TD) * 4 + act_lds_bytes(a.layout.n_ff, nt);
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
-    const dim3 grid((unsigned) ((a.layout.n_embd + kDnRows - 1) / kDnRows), (unsigned) (a.n_tokens * a.k));
-    if (nt == 4) hipLaunchKernelGGL((down_kernel<TD, 4>), grid, dim3(kDnThreads), lds, s, a, st.cb);
-    else if (nt == 2) hipLaunchKernelGGL((down_kernel<TD, 2>), grid, dim3(kDnThreads), lds, s, a, st.cb);
-    else hipLaunchKernelGGL((down_kernel<TD, 1>), grid, dim3(kDnThreads), lds, s, a, st.cb);
+    const int wr = rows_per_wg(a.layout.n_embd, a.n_tokens * a.k, 16, kDnRows);
+    const dim3 grid((unsigned) ((a.layout.n_embd + wr - 1) / wr), (unsigned) (a.n_tokens * a.k));
+    if (nt == 4) hipLaunchKernelGGL((down_kernel<TD, 4>), grid, dim3(kDnThreads), lds, s, a, st.cb, wr);
+    else if (nt == 2) hipLaunchKernelGGL((down_kernel<TD, 2>), grid, dim3(kDnThreads), lds, s, a, st.cb, wr);
+    else hipLaunchKernelGGL((down_kernel<TD, 1>), grid, dim3(kDnThreads), lds, s, a, st.cb, wr);
     MAYA_LAUNCHED("down_kernel");
     return MAYA_OK;
 }
