@@ -26,9 +26,9 @@ N_EMBD, N_FF, N_EXPERT, TOP_K = 7168, 2048, 256, 8
 IQ2_S = 22
 HBM_PEAK = 8.0e12
 # HBM bytes of one gate/up launch on this workload from rocprofv3's FETCH_SIZE and WRITE_SIZE (two runs, each scaled by
-# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,796.4 KiB read + 72.1 KiB written
+# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,783.1 KiB read + 64.0 KiB written
 # (profiles/decode_iq2s_hbm_traffic_pmc.txt)
-GATE_UP_TRAFFIC_BYTES = int((73796.4 + 72.1) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((73783.1 + 64.0) * 1024)
 
 
 def synth_experts_on_device(torch, n_expert, blob_bytes, seed):
