@@ -72,22 +72,24 @@ __global__ __launch_bounds__(256) void exl3_inner_kernel(const uint32_t* __restr
     dst[(ks * 16 + r) * n + tc * 16 + c] = __half_as_ushort(v);
 }
 
-// ---- the blockwise Hadamard transform of LDS data: v holds nb blocks of 128 floats; every thread of the workgroup calls
-// it.  The butterflies and their order are the reference's (src/kernels/cpu/exl3_ref.cpp:61-75): the same bits.
-__device__ __forceinline__ void had128_lds(float* v, int nb) {
-    for (int h = 1; h < 128; h <<= 1) {
-        for (int idx = threadIdx.x; idx < nb * 64; idx += kExThreads) {
-            const int blk = idx >> 6, j = idx & 63;
-            const int lo = blk * 128 + (j / h) * 2 * h + (j % h);
-            const float a = v[lo], c = v[lo + h];
-            v[lo] = __fadd_rn(a, c);
-            v[lo + h] = __fsub_rn(a, c);
-        }
-        __syncthreads();
+// ---- the blockwise Hadamard transform H / sqrt(128) of one 128-value block inside a wave: lane L holds values L and L + 64.
+// Stage h < 64 pairs lane L with lane L ^ h (the lower index adds, the upper takes lower - upper), stage 64 pairs the
+// lane's own two values: the butterflies, their order and every rounding are the reference's
+// (src/kernels/cpu/exl3_ref.cpp:61-75), so the same bits.
+__device__ __forceinline__ void had128_wave(float& v0, float& v1, int lane) {
+#pragma unroll
+    for (int h = 1; h < 64; h <<= 1) {
+        const float p0 = __shfl_xor(v0, h, 64), p1 = __shfl_xor(v1, h, 64);
+        const bool upper = (lane & h) != 0;
+        v0 = upper ? __fsub_rn(p0, v0) : __fadd_rn(v0, p0);
+        v1 = upper ? __fsub_rn(p1, v1) : __fadd_rn(v1, p1);
     }
+    const float a = v0, c = v1;
+    v0 = __fadd_rn(a, c);
+    v1 = __fsub_rn(a, c);
     const float s = 1.0f / sqrtf(128.0f);
-    for (int i = threadIdx.x; i < nb * 128; i += kExThreads) v[i] = __fmul_rn(v[i], s);
-    __syncthreads();
+    v0 = __fmul_rn(v0, s);
+    v1 = __fmul_rn(v1, s);
 }
 
 struct ExGroup {
@@ -113,13 +115,30 @@ __device__ __forceinline__ int ex_entry_of(const maya_exl3_args& a, const ExGrou
     return a.grp_ptr ? a.grp_ent[r.e0 + i] : r.e0;
 }
 
-// xr = FP16(H(x * suh)) of one activation into LDS (as FP16 pairs); `tmp` is k floats of LDS scratch
+// xr = FP16(H(x * suh)) of one activation into LDS; every wave of the workgroup takes blocks of 128 values (`tmp` is not
+// used: the transform runs in registers)
 __device__ __forceinline__ void rotate_in(const float* __restrict__ x, const uint16_t* __restrict__ suh, int k, float* tmp,
                                           __half* xr) {
-    for (int i = threadIdx.x; i < k; i += kExThreads) tmp[i] = __fmul_rn(x[i], f16_bits_to_f32(suh[i]));
+    (void) tmp;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int b = wave; b < (k >> 7); b += kExThreads / 64) {
+        const int i0 = b * 128 + lane;
+        float v0 = __fmul_rn(x[i0], f16_bits_to_f32(suh[i0])), v1 = __fmul_rn(x[i0 + 64], f16_bits_to_f32(suh[i0 + 64]));
+        had128_wave(v0, v1, lane);
+        xr[i0] = __float2half_rn(v0);
+        xr[i0 + 64] = __float2half_rn(v1);
+    }
     __syncthreads();
-    had128_lds(tmp, k >> 7);
-    for (int i = threadIdx.x; i < k; i += kExThreads) xr[i] = __float2half_rn(tmp[i]);
+}
+// the output rotation of nb blocks of 128 values in LDS, block b by wave b (nb <= 8), in place
+__device__ __forceinline__ void had128_out(float* v, int nb) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wave < nb) {
+        float v0 = v[wave * 128 + lane], v1 = v[wave * 128 + lane + 64];
+        had128_wave(v0, v1, lane);
+        v[wave * 128 + lane] = v0;
+        v[wave * 128 + lane + 64] = v1;
+    }
     __syncthreads();
 }
 
@@ -255,7 +274,7 @@ __device__ __forceinline__ float ex_swiglu(float g, float u, float limit) {
     return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
 }
 
-// dynamic LDS: [8 waves x 64 words of tile][NT x 2 x k halves of rotated inputs][max(k, NT*2*128) floats of scratch]
+// dynamic LDS: [8 waves x 64 words of tile][NT x 2 x k halves of rotated inputs][NT*2*128 floats of raw outputs]
 // grid (n_ff / 128, groups)
 template <int CB, int NT, int K2>
 __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args a) {
@@ -265,7 +284,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args
     const int k = a.layout.n_embd, n = a.layout.n_ff;
     uint32_t* wt = lds + (threadIdx.x >> 6) * 64;
     __half* xr = (__half*) (lds + 8 * 64);                       // [NT][2][k]
-    float* tmp = (float*) (xr + (size_t) NT * 2 * k);            // k floats; later the raw outputs [NT][2][128]
+    float* tmp = (float*) (xr + (size_t) NT * 2 * k);            // the raw outputs [NT][2][128]
     const uint8_t* blob = (const uint8_t*) gr.blob;
     const int64_t xs = a.x_stride ? a.x_stride : k;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -304,7 +323,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args
             }
         }
         __syncthreads();
-        had128_lds(tmp, NTC * 2);
+        had128_out(tmp, NTC * 2);
         const uint16_t* svg = (const uint16_t*) (blob + a.layout.svh[0]) + blockIdx.x * 128;
         const uint16_t* svu = (const uint16_t*) (blob + a.layout.svh[1]) + blockIdx.x * 128;
         for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
@@ -330,7 +349,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args
 // its row tiles, rotates the 128 partial sums and scales them - rotation and scaling are linear, so the slices' partial
 // outputs simply add - and stores them to P[entry][role][ks][n_ff] (the caller's `part` scratch).  exl3_swiglu_kernel adds the
 // slices and applies the SwiGLU.  Twice 2 KS as many, shorter workgroups as the fused kernel: the chip fills evenly.
-// dynamic LDS: [NT x k/KS halves of rotated input][max(k/KS, NT*128) floats of scratch]
+// dynamic LDS: [NT x k/KS halves of rotated input][NT*128 floats of raw outputs]
 template <int NT, int K2>
 __global__ __launch_bounds__(kExThreads) void exl3_gu_split_kernel(maya_exl3_args a, int KS) {
     extern __shared__ uint32_t lds[];
@@ -339,7 +358,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gu_split_kernel(maya_exl3_arg
     const int role = blockIdx.z / KS, ks = blockIdx.z % KS;
     const int k = a.layout.n_embd, n = a.layout.n_ff, kb = k / KS;
     __half* xr = (__half*) lds;                         // [NT][kb]
-    float* tmp = (float*) (xr + (size_t) NT * kb);      // kb floats; later [NT][128]
+    float* tmp = (float*) (xr + (size_t) NT * kb);      // the raw outputs [NT][128]
     const uint8_t* blob = (const uint8_t*) gr.blob;
     const int64_t xs = a.x_stride ? a.x_stride : k;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -366,7 +385,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gu_split_kernel(maya_exl3_arg
             for (int t = 0; t < NTC; ++t) tmp[t * 128 + col] = acc[t];
         }
         __syncthreads();
-        had128_lds(tmp, NTC);
+        had128_out(tmp, NTC);
         for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
             const int t = i >> 7, c = i & 127;
             a.part[(((size_t) ents[t] * 2 + role) * KS + ks) * n + blockIdx.x * 128 + c] = __fmul_rn(tmp[t * 128 + c], f16_bits_to_f32(sv[c]));
@@ -406,7 +425,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a)
     const int k = a.layout.n_ff, n = a.layout.n_embd;
     uint32_t* wt = lds + (threadIdx.x >> 6) * 64;
     __half* xr = (__half*) (lds + 8 * 64);             // [NT][k]
-    float* tmp = (float*) (xr + (size_t) NT * k);      // k floats; later [NT][128]
+    float* tmp = (float*) (xr + (size_t) NT * k);      // the raw outputs [NT][128]
     const uint8_t* blob = (const uint8_t*) gr.blob;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int tc = blockIdx.x * 8 + wave;
@@ -429,7 +448,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a)
             for (int t = 0; t < NTC; ++t) tmp[t * 128 + col] = acc[t];
         }
         __syncthreads();
-        had128_lds(tmp, NTC);
+        had128_out(tmp, NTC);
         const uint16_t* sv = (const uint16_t*) (blob + a.layout.svh[2]) + blockIdx.x * 128;
         for (int i = threadIdx.x; i < NTC * 128; i += kExThreads) {
             const int t = i >> 7, c = i & 127;
@@ -486,7 +505,7 @@ int exl3_check(const maya_exl3_args* a) {
 template <int NT>
 int launch_exl3_gate_up(const maya_exl3_args& a, const DeviceState& st, hipStream_t s) {
     const int k = a.layout.n_embd;
-    const size_t scratch = (size_t) (k > NT * 256 ? k : NT * 256) * 4;
+    const size_t scratch = (size_t) NT * 256 * 4;
     const size_t lds = 8 * 64 * 4 + (size_t) NT * 2 * k * 2 + scratch;
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
     const dim3 grid((unsigned) (a.layout.n_ff / 128), (unsigned) (a.n_tokens * a.k));
@@ -523,7 +542,7 @@ int try_exl3_gu_split(const maya_exl3_args& a, const DeviceState& st, hipStream_
     const int KS = (l.n_embd % 256 == 0 && l.n_embd >= 4 * l.n_ff) ? 2 : (l.n_embd >= 2 * l.n_ff ? 1 : 0);
     if (KS == 0) return 0;
     const int kb = l.n_embd / KS;
-    const size_t lds = (size_t) NT * kb * 2 + (size_t) (kb > NT * 128 ? kb : NT * 128) * 4;
+    const size_t lds = (size_t) NT * kb * 2 + (size_t) NT * 128 * 4;
     if (lds > (size_t) st.lds_limit) return 0;
     const dim3 grid((unsigned) (l.n_ff / 128), (unsigned) (a.n_tokens * a.k), (unsigned) (2 * KS));
 #define MAYA_EX(K2V)                                                                                              \
@@ -558,7 +577,7 @@ int try_exl3_gu_split(const maya_exl3_args& a, const DeviceState& st, hipStream_
 template <int NT>
 int launch_exl3_down(const maya_exl3_args& a, const DeviceState& st, hipStream_t s) {
     const int k = a.layout.n_ff;
-    const size_t scratch = (size_t) (k > NT * 128 ? k : NT * 128) * 4;
+    const size_t scratch = (size_t) NT * 128 * 4;
     const size_t lds = 8 * 64 * 4 + (size_t) NT * k * 2 + scratch;
     if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "exl3 down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
     const dim3 grid((unsigned) (a.layout.n_embd / 128), (unsigned) (a.n_tokens * a.k));

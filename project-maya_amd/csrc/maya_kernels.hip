@@ -889,6 +889,8 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 2, 5>), grid, dim3(64 * NW), 0, s, a, st.cb);
     else if (variant == 2) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 32, 1, 8>), dim3(grid.x / 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
     else if (variant == 3) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 8, 1, 8>), dim3(grid.x * 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
+    else if (variant == 4) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 7>), grid, dim3(64 * NW), 0, s, a, st.cb);
+    else if (variant == 5) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 8, 1, 7>), dim3(grid.x * 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
     else hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 8>), grid, dim3(64 * NW), 0, s, a, st.cb);
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
