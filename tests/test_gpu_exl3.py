@@ -105,6 +105,8 @@ CASES = [
     (512, 128, (3, 5, 7), 2, 6, 3, 4, 0.0),
     (4096, 2048, 6, 2, 8, 8, 1, 7.0),
     (1024, 512, 4, 2, 4, 4, 8, 0.0),
+    (6144, 1536, 6, 2, 10, 8, 4, 0.0),      # the EXL3 configuration's expert shape and window
+    (2048, 512, (4, 4, 16), 2, 5, 3, 2, 0.0),   # split gate/up with a general-walk down (16 bits a step)
 ]
 
 
