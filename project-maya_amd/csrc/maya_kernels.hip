@@ -316,9 +316,10 @@ __global__ __launch_bounds__(256) void quant_i8x32_kernel(const void* __restrict
 // ------------------------------------------------------------------------------------------------ router
 
 // One workgroup a token (src/kernels/cuda/router_top10.cu:68-187): the maximum (exact in any order), the exponentials in
-// double in parallel, their sum ascending on one thread, p = (float)(ex * inv) with inv a float, k rounds of a
-// workgroup-wide arg-max with a strict > and the lower index on ties, renormalisation by max(sum, 2^-14) in double.
-struct RouterLds {
+// double in parallel, their sum ascending on one thread, p = (float)(ex * inv) with inv a float, the k largest p in the
+// order k rounds of a strict-> arg-max with the lower index on ties would pick them, renormalisation by
+// max(sum, 2^-14) in double.
+struct alignas(16) RouterLds {
     double ex[MAYA_MAX_EXPERTS];
     float p[MAYA_MAX_EXPERTS];
     float rv[4];
@@ -327,7 +328,7 @@ struct RouterLds {
     float w[MAYA_MAX_K];
     int id[MAYA_MAX_K];
 };
-// 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights (thread 0 wrote them)
+// 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights
 __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
     const int tid = threadIdx.x;
     float mx = -INFINITY;
@@ -340,60 +341,76 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     __syncthreads();
     for (int e = tid; e < n_expert; e += 256) sm.ex[e] = exp((double) l[e] - (double) mx);
     __syncthreads();
-    if (tid == 0) {
-        // ascending, one add after the other (the reference's order); the reads run eight ahead of the adds
+    if (tid < 64) {
+        // ascending, one add after the other (the reference's order).  The chain of dependent double adds is the router's
+        // critical path, so nothing else may sit on it: the first wave pulls the values into registers (lane L holds
+        // experts L, L + 64, ...), then every add takes its operand from a lane by v_readlane (scalar registers, no
+        // memory wait); all lanes carry the same sum.
         double sum = 0.0;
-        int e = 0;
-        for (; e + 8 <= n_expert; e += 8) {
-            double v[8];
+        for (int r0 = 0; r0 < n_expert; r0 += 256) {
+            int lo[4], hi[4];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = sm.ex[e + j];
+            for (int r = 0; r < 4; ++r) {
+                const int e = r0 + 64 * r + tid;
+                const double v = e < n_expert ? sm.ex[e] : 0.0;   // (+0.0 past the end: adding it changes nothing)
+                lo[r] = __double2loint(v);
+                hi[r] = __double2hiint(v);
+            }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) sum += v[j];
+            for (int r = 0; r < 4; ++r) {
+                if (r0 + 64 * r < n_expert) {
+#pragma unroll
+                    for (int j0 = 0; j0 < 64; j0 += 8) {   // eight operands fetched ahead of the eight adds that use them
+                        int sl[8], sh[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            sl[j] = __builtin_amdgcn_readlane(lo[r], j0 + j);
+                            sh[j] = __builtin_amdgcn_readlane(hi[r], j0 + j);
+                        }
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) sum += __hiloint2double(sh[j], sl[j]);
+                    }
+                }
+            }
         }
-        for (; e < n_expert; ++e) sum += sm.ex[e];
-        sm.sum = sum;
+        if (tid == 0) sm.sum = sum;
     }
     __syncthreads();
     const float inv = (float) (1.0 / sm.sum);
     for (int e = tid; e < n_expert; e += 256) sm.p[e] = (float) (sm.ex[e] * (double) inv);
     __syncthreads();
-    // k rounds of arg-max by the first wave alone (no workgroup barriers): a lane scans its experts lane, lane + 64, ...
-    // in ascending order with a strict >, the wave folds (value, index) pairs preferring the lower index on ties, the
-    // winner is struck out of LDS (a probability is >= 0)
-    if (tid < 64) {
-        for (int i = 0; i < k; ++i) {
-            float bv = -INFINITY;
-            int bi = n_expert;
-            for (int e = tid; e < n_expert; e += 64) {
-                const float pe = sm.p[e];
-                if (pe > bv) {
-                    bv = pe;
-                    bi = e;
-                }
-            }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float ov = __shfl_xor(bv, o, kWave);
-                const int oi = __shfl_xor(bi, o, kWave);
-                if (ov > bv || (ov == bv && oi < bi)) {
-                    bv = ov;
-                    bi = oi;
-                }
-            }
-            if (bi >= n_expert) bi = 0;  // only when every remaining probability is NaN
-            if (tid == 0) {
-                sm.id[i] = bi;
-                sm.w[i] = sm.p[bi];
-                sm.p[bi] = -INFINITY;
-            }
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_s_waitcnt(0);   // the strike-out is in LDS before the next round's scan
+    // The k largest by rank, all at once: expert e's rank = the experts that beat it (a larger probability - they are
+    // non-negative, so their bit patterns order like the values - or an equal one at a lower index) - exactly the order in which k rounds of a strict-> arg-max with the lower index on ties
+    // would pick them (src/kernels/cuda/router_top10.cu:140-176), without the k dependent rounds.  Every thread reads
+    // the same p[j] at the same time (an LDS broadcast).
+    // (64-bit keys, probability bits above the complemented index, make "beats" one unsigned compare; they take the
+    // place of the exponentials, which are no longer needed)
+    unsigned long long* key = (unsigned long long*) sm.ex;
+    for (int e = tid; e < n_expert; e += 256)
+        key[e] = ((unsigned long long) __float_as_uint(sm.p[e]) << 32) | (unsigned long long) (0xffffffffu - (unsigned) e);
+    __syncthreads();
+    for (int e = tid; e < n_expert; e += 256) {
+        const unsigned long long ke = key[e];
+        int rank = 0;
+        int j = 0;
+        for (; j + 2 <= n_expert; j += 2) {
+            const ulonglong2 kj = *(const ulonglong2*) (key + j);
+            rank += kj.x > ke ? 1 : 0;
+            rank += kj.y > ke ? 1 : 0;
         }
+        for (; j < n_expert; ++j) rank += key[j] > ke ? 1 : 0;
+        if (rank < k) {
+            sm.id[rank] = e;
+            sm.w[rank] = sm.p[e];
+        }
+    }
+    __syncthreads();
+    if (tid < 64) {
         // renormalisation: the sum of the k weights in slot order in double, one division a lane
         double s = 0.0;
         for (int i = 0; i < k; ++i) s += (double) sm.w[i];
         const double sc = fmax(s, 6.103515625e-05);
+        __builtin_amdgcn_wave_barrier();
         if (tid < k) sm.w[tid] = (float) ((double) sm.w[tid] / sc);
     }
     __syncthreads();
