@@ -881,11 +881,6 @@ int launch_down_t(const maya_moe_args& a, const DeviceState& st, hipStream_t s) 
 
 bool fast_1tok(const maya_moe_args& a) { return a.n_tokens == 1 && a.grp_ptr == nullptr; }
 
-int tuning_variant(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
-}
-
 int launch_gate_up_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 32;
     const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) a.k);
@@ -897,29 +892,19 @@ int launch_gate_up_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipS
     MAYA_LAUNCHED("gate_up_iq2s_1tok_kernel");
     return MAYA_OK;
 }
-// (MAYA_GU_VARIANT / MAYA_DN_VARIANT: tuning knobs for the row tile and the prefetch depth; unset = the measured best)
+// the position-mapped kernels: 16 rows a workgroup; gate/up at the 6 waves a SIMD its registers allow, down at 7 (8 spill)
 template <int NW>
 int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
     const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) (a.n_tokens * a.k));   // an entry a column of the grid
-    static const int variant = tuning_variant("MAYA_GU_VARIANT", 0);
-    if (variant == 1) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 2, 5>), grid, dim3(64 * NW), 0, s, a, st.cb);
-    else if (variant == 2) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 32, 1, 8>), dim3(grid.x / 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
-    else if (variant == 3) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 8, 1, 8>), dim3(grid.x * 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
-    else if (variant == 4) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 7>), grid, dim3(64 * NW), 0, s, a, st.cb);
-    else if (variant == 5) hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, 8, 1, 7>), dim3(grid.x * 2, grid.y), dim3(64 * NW), 0, s, a, st.cb);
-    else hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 8>), grid, dim3(64 * NW), 0, s, a, st.cb);
+    hipLaunchKernelGGL((gate_up_iq2s_pos_kernel<NW, kRows, 1, 8>), grid, dim3(64 * NW), 0, s, a, st.cb);
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
 }
 int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
     const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
-    static const int variant = tuning_variant("MAYA_DN_VARIANT", 0);
-    if (variant == 1) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 2, 5>), grid, dim3(512), 0, s, a, st.cb);
-    else if (variant == 2) hipLaunchKernelGGL((down_iq2s_pos_kernel<8, 1, 8>), dim3(grid.x * 2, grid.y), dim3(512), 0, s, a, st.cb);
-    else if (variant == 3) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 8>), grid, dim3(512), 0, s, a, st.cb);
-    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);   // 8 waves a SIMD spill
+    hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
     return MAYA_OK;
 }
@@ -997,14 +982,20 @@ bool down_q4k_pos_ok(const maya_moe_args& a) {
            (l.down_off & 15) == 0;
 }
 int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
-    constexpr int kRows = 16;
-    const dim3 grid((unsigned) (a.layout.n_ff / kRows), (unsigned) (a.n_tokens * a.k));
+    // 16 rows a workgroup, 8 when the call has so few entries that 16 would leave compute units idle
+    const bool small = (long long) (a.layout.n_ff / 16) * a.n_tokens * a.k < 512;
+    const int rows = small ? 8 : 16;
+    const dim3 grid((unsigned) (a.layout.n_ff / rows), (unsigned) (a.n_tokens * a.k));
+#define MAYA_Q4(NWV)                                                                                              \
+    if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 8>), grid, dim3(64 * NWV), 0, s, a);          \
+    else hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a);
     switch (a.layout.n_embd / 1024) {
-        case 4: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<4, kRows, 8>), grid, dim3(256), 0, s, a); break;
-        case 6: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<6, kRows, 8>), grid, dim3(384), 0, s, a); break;
-        case 7: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<7, kRows, 8>), grid, dim3(448), 0, s, a); break;
-        default: hipLaunchKernelGGL((gate_up_q4k_pos_kernel<8, kRows, 8>), grid, dim3(512), 0, s, a); break;
+        case 4: MAYA_Q4(4) break;
+        case 6: MAYA_Q4(6) break;
+        case 7: MAYA_Q4(7) break;
+        default: MAYA_Q4(8) break;
     }
+#undef MAYA_Q4
     MAYA_LAUNCHED("gate_up_q4k_pos_kernel");
     return MAYA_OK;
 }
