@@ -327,6 +327,9 @@ struct alignas(16) RouterLds {
     double sum;
     float w[MAYA_MAX_K];
     int id[MAYA_MAX_K];
+    // (more than 256 experts) the threads' best keys, the k-th largest of them, the keys at or above it
+    unsigned long long lb[256], thr, cand[MAYA_MAX_K * (MAYA_MAX_EXPERTS / 256)];
+    int nc;
 };
 // 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights
 __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
@@ -389,19 +392,54 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     for (int e = tid; e < n_expert; e += 256)
         key[e] = ((unsigned long long) __float_as_uint(sm.p[e]) << 32) | (unsigned long long) (0xffffffffu - (unsigned) e);
     __syncthreads();
-    for (int e = tid; e < n_expert; e += 256) {
-        const unsigned long long ke = key[e];
-        int rank = 0;
-        int j = 0;
-        for (; j + 2 <= n_expert; j += 2) {
-            const ulonglong2 kj = *(const ulonglong2*) (key + j);
-            rank += kj.x > ke ? 1 : 0;
-            rank += kj.y > ke ? 1 : 0;
+    if (n_expert <= 256) {
+        for (int e = tid; e < n_expert; e += 256) {
+            const unsigned long long ke = key[e];
+            int rank = 0;
+            int j = 0;
+            for (; j + 2 <= n_expert; j += 2) {
+                const ulonglong2 kj = *(const ulonglong2*) (key + j);
+                rank += kj.x > ke ? 1 : 0;
+                rank += kj.y > ke ? 1 : 0;
+            }
+            for (; j < n_expert; ++j) rank += key[j] > ke ? 1 : 0;
+            if (rank < k) {
+                sm.id[rank] = e;
+                sm.w[rank] = sm.p[e];
+            }
         }
-        for (; j < n_expert; ++j) rank += key[j] > ke ? 1 : 0;
-        if (rank < k) {
-            sm.id[rank] = e;
-            sm.w[rank] = sm.p[e];
+    } else {
+        // Wider routers: ranking every expert against every other grows with the square.  The k-th largest of the
+        // threads' best keys is a lower bound of the k-th largest key overall (those are k different experts), so only keys
+        // at or above it can be among the k largest, and every key that beats one of them is at or above it too: the few
+        // candidates (at most k threads' experts) are ranked among themselves.
+        unsigned long long best = 0ull;
+        for (int e = tid; e < n_expert; e += 256) best = key[e] > best ? key[e] : best;
+        sm.lb[tid] = best;
+        if (tid == 0) sm.nc = 0;
+        __syncthreads();
+        int rank = 0;
+        for (int j = 0; j < 256; j += 2) {
+            const ulonglong2 kj = *(const ulonglong2*) (sm.lb + j);
+            rank += kj.x > best ? 1 : 0;
+            rank += kj.y > best ? 1 : 0;
+        }
+        if (rank == k - 1) sm.thr = best;
+        __syncthreads();
+        const unsigned long long thr = sm.thr;
+        for (int e = tid; e < n_expert; e += 256)
+            if (key[e] >= thr) sm.cand[atomicAdd(&sm.nc, 1)] = key[e];
+        __syncthreads();
+        const int nc = sm.nc;
+        if (tid < nc) {
+            const unsigned long long kc = sm.cand[tid];
+            int r = 0;
+            for (int j = 0; j < nc; ++j) r += sm.cand[j] > kc ? 1 : 0;
+            if (r < k) {
+                const int e = (int) (0xffffffffu - (unsigned) (kc & 0xffffffffull));
+                sm.id[r] = e;
+                sm.w[r] = sm.p[e];
+            }
         }
     }
     __syncthreads();

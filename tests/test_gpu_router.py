@@ -48,6 +48,19 @@ def test_twelve_way_tie_and_dominant(lib, oracle):
     _check(lib, oracle, logits, 8)
 
 
+def test_wide_routers_ties_and_degenerate_rows(lib, oracle):
+    """More than 256 experts take the candidate path: ties by index, underflowed probabilities, k up to 16."""
+    rng = np.random.default_rng(15)
+    for ne, k in ((1024, 8), (512, 16), (384, 6)):
+        logits = rng.standard_normal((5, ne)).astype(np.float32)
+        logits[0, :] = 0.25                                   # all equal: ids 0 .. k-1
+        logits[1, rng.choice(ne, 20, replace=False)] = 5.0    # a 20-way tie at the top
+        logits[2, :] = -1e30
+        logits[2, ne - 3] = 0.0                               # one expert, every other probability exactly 0
+        logits[3] = np.round(logits[3] * 2) / 2
+        _check(lib, oracle, logits, k)
+
+
 def test_zipf_biased(lib, oracle):
     from maya_amd import synth
     rng = np.random.default_rng(6)
