@@ -96,8 +96,12 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
     const uint8_t* rp = w + (size_t) row * row_stride;
     float r;
     if constexpr (TYPE == kQ8_0) {
-        const uint8_t* blk = rp + (size_t) (v >> 5) * 34;
-        r = __fmul_rn((float) (int8_t) blk[2 + (v & 31)], f16_bits_to_f32(ld16(blk)));
+        if (packing == MAYA_PACK_STREAM) {   // a row = its k codes, then its k / 32 scales
+            r = __fmul_rn((float) (int8_t) rp[v], f16_bits_to_f32(ld16(rp + k + 2 * (v >> 5))));
+        } else {
+            const uint8_t* blk = rp + (size_t) (v >> 5) * 34;
+            r = __fmul_rn((float) (int8_t) blk[2 + (v & 31)], f16_bits_to_f32(ld16(blk)));
+        }
     } else if constexpr (TYPE == kQ4_K) {
         const uint8_t* blk = rp + (size_t) (v >> 8) * 144;
         const int i = (int) (v & 255), j = i >> 5, l = i & 31;
@@ -191,6 +195,28 @@ __global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restr
             gd[0] = qs[o_d];
             gd[1] = qs[o_d + 1];
         }
+    }
+}
+
+// Q8_0 rows between the GGUF block sequence (2-byte scale, 32 codes, ...) and the stream order (the row's codes, then its
+// scales); one thread a block, grid (k/32 blocks / 256, rows).  DIR 0: GGUF -> stream, 1: stream -> GGUF.
+template <int DIR>
+__global__ __launch_bounds__(256) void repack_q80_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t k,
+                                                         int64_t n_rows) {
+    const int64_t nb = k >> 5, rb = nb * 34;
+    const int64_t b = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (b >= nb || row >= n_rows) return;
+    const uint16_t* g = (const uint16_t*) ((DIR == 0 ? src : dst) + row * rb + b * 34);          // the GGUF block
+    const uint16_t* sq = (const uint16_t*) ((DIR == 0 ? dst : src) + row * rb + b * 32);         // the stream codes
+    const uint16_t* sd = (const uint16_t*) ((DIR == 0 ? dst : src) + row * rb + k + b * 2);      // the stream scale
+    if constexpr (DIR == 0) {
+        *(uint16_t*) sd = g[0];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ((uint16_t*) sq)[i] = g[1 + i];
+    } else {
+        ((uint16_t*) g)[0] = *sd;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ((uint16_t*) g)[1 + i] = sq[i];
     }
 }
 
@@ -628,6 +654,12 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
             float D;
             if (TYPE == kIQ2_S && stream_packed) {
                 if constexpr (TYPE == kIQ2_S) Fmt<kIQ2_S>::decode_stream(row, nu, rq, un, grid, u, D);
+            } else if (TYPE == kQ8_0 && stream_packed) {   // the row's codes, then its scales
+                const int* c = (const int*) (row + 32 * (size_t) un);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) u.q[i] = c[i];
+                u.s0 = u.s1 = 1;
+                D = f16_bits_to_f32(ld16(row + k + 2 * (size_t) un));
             } else {
                 Fmt<TYPE>::decode(blk, ib, grid, u);
                 D = Fmt<TYPE>::scale(blk);
@@ -759,14 +791,16 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
             // (stream packing: the row's quad and its place in it; the GGUF packing: the row itself)
             // (only IQ2_S rows have a stream order; the other types' rows stay where GGUF puts them)
-            const bool pg = packed && TG == kIQ2_S, pu = packed && TU == kIQ2_S;
+            // (IQ2_S rows are packed in quads, Q8_0 rows one by one)
+            const bool qg = packed && TG == kIQ2_S, qu = packed && TU == kIQ2_S;
+            const bool pg = packed && (TG == kIQ2_S || TG == kQ8_0), pu = packed && (TU == kIQ2_S || TU == kQ8_0);
             const int rq = r & 3;
             if constexpr (TG == TU) {
-                const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) (pg ? (r & ~3) : r) * grow;
+                const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) (qg ? (r & ~3) : r) * grow;
                 row_dot<TG, NT, 32>(row, k, sub, al, grid_g, acc, pg, rq);
             } else {
-                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) (pg ? (r & ~3) : r) * grow, k, sub, al, grid_g, acc, pg, rq);
-                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) (pu ? (r & ~3) : r) * urow, k, sub, al, grid_u, acc, pu, rq);
+                if (!is_up) row_dot<TG, NT, 32>(blob + a.layout.gate_off + (size_t) (qg ? (r & ~3) : r) * grow, k, sub, al, grid_g, acc, pg, rq);
+                else row_dot<TU, NT, 32>(blob + a.layout.up_off + (size_t) (qu ? (r & ~3) : r) * urow, k, sub, al, grid_u, acc, pu, rq);
             }
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -798,7 +832,8 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
     const uint8_t* base = (const uint8_t*) gr.blob + a.layout.down_off;
     const size_t drow = (size_t) (k / Fmt<TD>::kValues) * Fmt<TD>::kBytes;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
-    const bool packed = a.layout.packing == MAYA_PACK_STREAM && TD == kIQ2_S;
+    const bool quads = a.layout.packing == MAYA_PACK_STREAM && TD == kIQ2_S;
+    const bool packed = a.layout.packing == MAYA_PACK_STREAM && (TD == kIQ2_S || TD == kQ8_0);
     for (int c0 = 0; c0 < gr.ne; c0 += NT) {
         int ents[NT];
 #pragma unroll
@@ -811,7 +846,7 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
             float acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
-            row_dot<TD, NT, 32>(base + (size_t) (packed ? (r & ~3) : r) * drow, k, sub, al, grid, acc, packed, r & 3);
+            row_dot<TD, NT, 32>(base + (size_t) (quads ? (r & ~3) : r) * drow, k, sub, al, grid, acc, packed, r & 3);
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 const float s = group_sum<32>(acc[t]);
@@ -844,6 +879,7 @@ __global__ __launch_bounds__(256) void combine_kernel(maya_moe_args a) {
 
 #include "maya_fast.cuh"
 #include "maya_fastk.cuh"
+#include "maya_fastq.cuh"
 
 namespace maya {
 
@@ -1044,6 +1080,62 @@ int launch_down_q4k_pos(const maya_moe_args& a, hipStream_t s) {
     MAYA_LAUNCHED("down_q4k_pos_kernel");
     return MAYA_OK;
 }
+// ---- Q8_0 in the stream packing: the position-mapped kernels for the shapes they take
+bool gate_up_q80_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (!(l.gate_type == kQ8_0 && l.up_type == kQ8_0 && l.packing == MAYA_PACK_STREAM)) return false;
+    if (l.n_embd % 1024 != 0 || l.n_ff % 8 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
+    const int nw = l.n_embd / 1024;
+    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+}
+bool down_q80_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    return l.down_type == kQ8_0 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 && l.n_embd % 64 == 0 && (l.down_off & 15) == 0;
+}
+// tokens of a group served by one read of the weights: as many as the call can have in a group, rounded up to 1, 2, 4, 8
+inline int q80_group_tokens(const maya_moe_args& a) {
+    if (!a.grp_ptr) return 1;
+    return a.n_tokens >= 5 ? 8 : a.n_tokens >= 3 ? 4 : a.n_tokens >= 2 ? 2 : 1;
+}
+int launch_gate_up_q80_pos(const maya_moe_args& a, hipStream_t s) {
+    const int nt = q80_group_tokens(a);
+    const dim3 grid((unsigned) (a.layout.n_ff / 8), (unsigned) (a.n_tokens * a.k));
+#define MAYA_Q8(NWV)                                                                                              \
+    switch (nt) {                                                                                                 \
+        case 8: hipLaunchKernelGGL((gate_up_q80_pos_kernel<NWV, 8, 8>), grid, dim3(64 * NWV), 0, s, a); break;  \
+        case 4: hipLaunchKernelGGL((gate_up_q80_pos_kernel<NWV, 4, 8>), grid, dim3(64 * NWV), 0, s, a); break;  \
+        case 2: hipLaunchKernelGGL((gate_up_q80_pos_kernel<NWV, 2, 8>), grid, dim3(64 * NWV), 0, s, a); break;  \
+        default: hipLaunchKernelGGL((gate_up_q80_pos_kernel<NWV, 1, 8>), grid, dim3(64 * NWV), 0, s, a); break; \
+    }
+    switch (a.layout.n_embd / 1024) {
+        case 4: MAYA_Q8(4) break;
+        case 6: MAYA_Q8(6) break;
+        case 7: MAYA_Q8(7) break;
+        default: MAYA_Q8(8) break;
+    }
+#undef MAYA_Q8
+    MAYA_LAUNCHED("gate_up_q80_pos_kernel");
+    return MAYA_OK;
+}
+int launch_down_q80_pos(const maya_moe_args& a, hipStream_t s) {
+    const int nt = q80_group_tokens(a);
+    // a wave takes per_wave rows, a multiple of the 8 / nt rows of a step: 8 (64 rows a workgroup) unless the call has so
+    // few entries that the grid would not cover the chip
+    const int step = 8 / nt;
+    int per_wave = 8;
+    while (per_wave > step && (long long) (a.layout.n_embd / (per_wave * 8)) * a.n_tokens * a.k < 1024) per_wave >>= 1;
+    const int wg_rows = per_wave * 8;
+    const dim3 grid((unsigned) ((a.layout.n_embd + wg_rows - 1) / wg_rows), (unsigned) (a.n_tokens * a.k));
+    switch (nt) {
+        case 8: hipLaunchKernelGGL((down_q80_pos_kernel<8>), grid, dim3(512), 0, s, a, wg_rows); break;
+        case 4: hipLaunchKernelGGL((down_q80_pos_kernel<4>), grid, dim3(512), 0, s, a, wg_rows); break;
+        case 2: hipLaunchKernelGGL((down_q80_pos_kernel<2>), grid, dim3(512), 0, s, a, wg_rows); break;
+        default: hipLaunchKernelGGL((down_q80_pos_kernel<1>), grid, dim3(512), 0, s, a, wg_rows); break;
+    }
+    MAYA_LAUNCHED("down_q80_pos_kernel");
+    return MAYA_OK;
+}
+
 // whether the gate/up (down) call is served entry by entry (no use for the groups of a window)
 bool gate_up_by_entries(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
@@ -1122,6 +1214,10 @@ static int repack_impl(const maya_moe_layout* l, const void* src, void* dst, voi
             const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
             if (dir == 0) hipLaunchKernelGGL(repack_iq2s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
             else hipLaunchKernelGGL(repack_iq2s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+        } else if (r.type == kQ8_0) {
+            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
+            if (dir == 0) hipLaunchKernelGGL(repack_q80_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+            else hipLaunchKernelGGL(repack_q80_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
         } else {
             const size_t n = maya_moe_row_bytes(r.type, r.k) * (size_t) r.rows;
             hipLaunchKernelGGL(copy_bytes_kernel, dim3(1024), dim3(256), 0, s, sp, dp, n);
@@ -1255,6 +1351,7 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
         if (try_gate_up_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
     if (gate_up_q4k_pos_ok(*a)) return launch_gate_up_q4k_pos(*a, s);
+    if (gate_up_q80_pos_ok(*a)) return launch_gate_up_q80_pos(*a, s);
 #define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
     MAYA_GU(kIQ2_S, kIQ2_S)
     MAYA_GU(kQ4_K, kQ4_K)
@@ -1289,6 +1386,13 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
         if (try_down_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
     if (down_q4k_pos_ok(*a)) return launch_down_q4k_pos(*a, s);
+    if (down_q80_pos_ok(*a)) {
+        if (const int rc = launch_down_q80_pos(*a, s)) return rc;
+        const dim3 cgrid((unsigned) ((a->layout.n_embd + 255) / 256), (unsigned) a->n_tokens);
+        hipLaunchKernelGGL(combine_kernel, cgrid, dim3(256), 0, s, *a);
+        MAYA_LAUNCHED("combine_kernel");
+        return MAYA_OK;
+    }
     int rc;
     switch (a->layout.down_type) {
         case kIQ2_S: rc = launch_down_t<kIQ2_S>(*a, *st, s); break;

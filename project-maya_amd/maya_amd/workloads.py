@@ -118,9 +118,14 @@ def batch8_mixed(K, W):
         lib.repack(l, staging, view[e])
     torch.cuda.synchronize()
     table = torch.tensor([pool.data_ptr() + e * bb for e in range(NE)], dtype=torch.int64, device="cuda")
-    shared = lib.MoeLayer(lib.Q8_0, lib.Q8_0, E, FF, 1, 1, max_tokens=T)
+    shared = lib.MoeLayer(lib.Q8_0, lib.Q8_0, E, FF, 1, 1, max_tokens=T, packing=lib.PACK_STREAM)
     n_sh = 4   # copies of the shared expert rotate too (4 x 46.8 MB)
     sh_pool = random_blocks(n_sh * shared.blob_bytes, 34, {0: (1e-4, 4e-4)}, 8)
+    staging = torch.empty(shared.blob_bytes, dtype=torch.uint8, device="cuda")
+    for c in range(n_sh):
+        staging.copy_(sh_pool[c * shared.blob_bytes:(c + 1) * shared.blob_bytes])
+        lib.repack(shared.gguf_layout, staging, sh_pool[c * shared.blob_bytes:(c + 1) * shared.blob_bytes])
+    torch.cuda.synchronize()
     sh_tables = [torch.tensor([sh_pool.data_ptr() + c * shared.blob_bytes], dtype=torch.int64, device="cuda") for c in range(n_sh)]
     sh_logits = torch.zeros((T, 1), device="cuda")
     rng = np.random.default_rng(9)

@@ -58,6 +58,11 @@ CASES = [
     (12, 12, 7168, 2048, 5, 3, 4),
     (22, 12, 6144, 2048, 9, 8, 3),
     (12, 22, 8192, 2048, 4, 2, 2),
+    # stream-packed Q8_0 (the shared expert's format): one token, a window, mixed with other types
+    (8, 8, 4096, 2048, 5, 3, 1),
+    (8, 8, 7168, 2048, 3, 2, 7),
+    (8, 12, 6144, 2048, 4, 2, 3),
+    (22, 8, 4096, 2048, 6, 4, 2),
 ]
 
 
@@ -129,7 +134,7 @@ def test_zero_input_and_bf16_input(lib, oracle):
     assert np.array_equal(ids, wi) and rel_l2(out, wout) <= TOL
 
 
-@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3), (22, 12, 4096, 2048, 7, 4, 4)))
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3), (22, 12, 4096, 2048, 7, 4, 4), (8, 8, 4096, 2048, 1, 1, 8)))
 def test_window_rows_equal_token_rows(lib, gt, dt, n_embd, n_ff, ne, k, nt):
     """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract), in either
     row packing."""

@@ -103,7 +103,7 @@ def test_i8x32_quant_byte_exact(lib, oracle):
         assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
 
 
-@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8)))
+@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8)))
 def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
     """maya_moe_repack regroups bytes only: unpack(repack(blob)) == blob, and the packed rows dequantize to the same bits."""
     n_embd, n_ff = 1024, 512
@@ -124,7 +124,12 @@ def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
         a = src[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
         b = packed[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
         assert np.array_equal(np.sort(a, axis=1), np.sort(b, axis=1))
-        if t != 22:
+        if t == 8:
+            # Q8_0: a row's codes first, then its scales
+            g = src[off:off + rb * rows].view(rows, k // 32, 34).cpu().numpy()
+            p = packed[off:off + rb * rows].view(rows, rb).cpu().numpy()
+            assert np.array_equal(p[:, :k], g[:, :, 2:].reshape(rows, k)) and np.array_equal(p[:, k:], g[:, :, :2].reshape(rows, -1))
+        elif t != 22:
             assert np.array_equal(a, b)
         want = oracle.dequant_rows(t, blob[off:off + rb * 16], k, 16)
         got = lib.dequant_rows(t, packed[off:], k, 16, packing=1).cpu().numpy()
