@@ -468,6 +468,20 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
     __syncthreads();
     if (blob != 0ull) {
+        // the first rows' weights are requested before h is rounded: their latency hides behind that arithmetic
+        constexpr uint32_t qb = NU / 8 * 82 * 4;
+        // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
+        // scalar registers for the buffer resource
+        const uint64_t mat = blob + a.layout.down_off;
+        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
+        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
+        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
+        const QuadOffs qo = quad_offs<NU>(0u, lane);
+        const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+        constexpr int NQ = ROWS / 4;
+        QuadIQ2S ring[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
         int y[8];
         float dy8;
         if (a.hq.q) {
@@ -486,50 +500,13 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
                 const float4 t = hv[i];
                 v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
             }
-            float am = 0.0f, sv = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const float av = fabsf(v[i]);
-                if (av > am) am = av, sv = v[i];
-            }
-#pragma unroll
-            for (int o = 1; o < 8; o <<= 1) {
-                const float oa = __shfl_xor(am, o, kWave), os = __shfl_xor(sv, o, kWave);
-                if (oa > am || (oa == am && (lane & o))) am = oa, sv = os;
-            }
-            float iscale = 0.0f, d = 0.0f;
-            if (am > 0.0f) {
-                iscale = __fdiv_rn(-127.0f, sv);
-                d = __fdiv_rn(1.0f, iscale);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                uint32_t w = 0;
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const int c = am > 0.0f ? min(127, nearest_int(__fmul_rn(iscale, v[4 * i + b]))) : 0;
-                    w |= ((uint32_t) c & 0xffu) << (8 * b);
-                }
-                y[i] = (int) w;
-            }
+            float d;
+            q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
             dy8 = d * 0.125f;
         }
         int yn[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
-        constexpr uint32_t qb = NU / 8 * 82 * 4;
-        // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
-        // scalar registers for the buffer resource
-        const uint64_t mat = blob + a.layout.down_off;
-        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
-        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
-        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        const QuadOffs qo = quad_offs<NU>(0u, lane);
-        const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
-        constexpr int NQ = ROWS / 4;
-        QuadIQ2S ring[DEPTH];
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
         float acc[8];
 #pragma unroll 1
         for (int r = 0; r < ROWS; r += 8) {

@@ -127,6 +127,14 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
     if (blob != 0ull) {
         PosQ4K p;
         pos_q4k_init(p, lane, 0u);
+        // the first row's weights are requested before h is rounded: their latency hides behind that arithmetic
+        constexpr uint32_t rb = NU / 8 * 144;
+        const uint64_t mat = blob + a.layout.down_off;
+        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
+        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
+        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) n_embd * rb);
+        u32x4 hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) r0 * rb, 0);
+        u32x4 qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) r0 * rb, 0);
         if (a.hq.q) {
             pos_q4k_codes(p, lane, a.hq.q + (size_t) ent * 2048, a.hq.d + (size_t) ent * NU, a.hq.bsums + (size_t) ent * (2 * NU));
         } else {
@@ -142,46 +150,15 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
                 v[4 * i] = lo.x, v[4 * i + 1] = lo.y, v[4 * i + 2] = lo.z, v[4 * i + 3] = lo.w;
                 v[16 + 4 * i] = hi.x, v[16 + 4 * i + 1] = hi.y, v[16 + 4 * i + 2] = hi.z, v[16 + 4 * i + 3] = hi.w;
             }
-            float am = 0.0f, sv = 0.0f;
-            int ix = 0;
+            int y[8];
+            float d;
+            q8k_round_lane32(v, [&](int i) { return 64 * j + 16 * half + (i < 16 ? i : i + 16); }, y, d);
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {   // ascending index inside the lane: a strict > keeps the first
-                const float av = fabsf(v[i]);
-                if (av > am) am = av, sv = v[i], ix = v0 + (i < 16 ? i : i + 16);
-            }
-#pragma unroll
-            for (int o = 1; o < 8; o <<= 1) {
-                const float oa = __shfl_xor(am, o, kWave), os = __shfl_xor(sv, o, kWave);
-                const int oi = __shfl_xor(ix, o, kWave);
-                if (oa > am || (oa == am && oi < ix)) am = oa, sv = os, ix = oi;
-            }
-            float iscale = 0.0f, d = 0.0f;
-            if (am > 0.0f) {
-                iscale = __fdiv_rn(-127.0f, sv);
-                d = __fdiv_rn(1.0f, iscale);
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                uint32_t w = 0;
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const int c = am > 0.0f ? min(127, nearest_int(__fmul_rn(iscale, v[4 * i + b]))) : 0;
-                    w |= ((uint32_t) c & 0xffu) << (8 * b);
-                }
-                if (i < 4) p.ylo[i] = (int) w;
-                else p.yhi[i - 4] = (int) w;
-            }
+            for (int i = 0; i < 4; ++i) p.ylo[i] = y[i], p.yhi[i] = y[4 + i];
             p.dx = d;
             p.slo = dot4(0x01010101, p.ylo[0], dot4(0x01010101, p.ylo[1], dot4(0x01010101, p.ylo[2], dot4(0x01010101, p.ylo[3], 0))));
             p.shi = dot4(0x01010101, p.yhi[0], dot4(0x01010101, p.yhi[1], dot4(0x01010101, p.yhi[2], dot4(0x01010101, p.yhi[3], 0))));
         }
-        constexpr uint32_t rb = NU / 8 * 144;
-        const uint64_t mat = blob + a.layout.down_off;
-        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
-        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
-        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) n_embd * rb);
-        u32x4 hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) r0 * rb, 0);
-        u32x4 qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) r0 * rb, 0);
         float acc[8];
 #pragma unroll 1
         for (int r = 0; r < ROWS; r += 8) {

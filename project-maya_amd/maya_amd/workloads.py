@@ -96,7 +96,7 @@ def single_q4k(K, W):
             "config": {"workload": "configs[0]: one expert GLU, gate/up [2048x7168] + down [7168x2048] Q4_K (constructed "
                                    "blocks), 1 token F32; 16 copies of the expert rotate over the steps",
                        "algorithmic_bytes_per_step": nbytes},
-            "roofline": hbm_roofline("layer (head + gate_up_kernel<Q4_K> + quant + down_kernel<Q4_K> + combine)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (layer_head_kernel + gate_up_q4k_pos_kernel + down_q4k_pos_kernel)", nbytes, sec)}
 
 
 def batch8_mixed(K, W):
@@ -151,7 +151,7 @@ def batch8_mixed(K, W):
             "config": {"workload": "configs[2]: 8 tokens, 256 experts top-8 (gate/up IQ2_S, down Q4_K) + a Q8_0 shared expert; "
                                    "8 logit sets rotate", "distinct_experts_per_step": d_avg,
                        "algorithmic_bytes_per_step": int(nbytes)},
-            "roofline": hbm_roofline("layer (routed gate_up_kernel<IQ2_S,8 tok> + down_kernel<Q4_K> + shared Q8_0 expert)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (routed gate_up_iq2s_pos_kernel + down_q4k_pos_kernel over 64 entries, shared expert gate_up_q80_pos_kernel + down_q80_pos_kernel)", nbytes, sec)}
 
 
 def prefill_q4k(K, W):
@@ -229,7 +229,7 @@ def exl3_verify(K, W):
             "config": {"workload": "configs[4]: EXL3 3-bit trellis experts (k2 6, mul1), 160 experts top-8, hidden 6144, "
                                    "intermediate 1536, 4-token verify window; 8 logit sets rotate",
                        "distinct_experts_per_step": d_avg, "algorithmic_bytes_per_step": int(nbytes)},
-            "roofline": hbm_roofline("layer (exl3_gate_up_kernel + exl3_down_kernel + combine)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (exl3_gu_split_kernel + exl3_swiglu_kernel + exl3_down_kernel + exl3_combine_kernel)", nbytes, sec)}
 
 
 WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify}

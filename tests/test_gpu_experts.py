@@ -166,14 +166,16 @@ def test_unsupported_and_bad_shapes_fail_cleanly(lib):
         lib.route_topk(torch.zeros((1, 4), device="cuda"), 8)
 
 
-def test_down_rounds_h_itself_like_the_quantizer(lib):
-    """The stream-packed IQ2_S down kernel given no rounded h rounds it in its prologue: the same Q8_K codes as
-    maya_quant_act (ties, an all-zero block, equal magnitudes of both signs), so the same output bits."""
+@pytest.mark.parametrize("dt", (22, 12))
+def test_down_rounds_h_itself_like_the_quantizer(lib, dt):
+    """The stream-packed IQ2_S / Q4_K down kernels given no rounded h round it in their prologue: the same Q8_K codes as
+    maya_quant_act (an all-zero block, equal magnitudes of both signs inside a lane's values, across lanes, and where
+    the lower index sits in the higher lane), so the same output bits."""
     import ctypes as C
     L = lib.load()
     n_embd, n_ff, ne, k = 1024, 2048, 8, 8
-    blobs = make_experts(22, 22, n_embd, n_ff, ne, 77)
-    gguf, _ = lib.layout(22, 22, n_embd, n_ff)
+    blobs = make_experts(22, dt, n_embd, n_ff, ne, 77)
+    gguf, _ = lib.layout(22, dt, n_embd, n_ff)
     store = lib.ExpertStore(blobs, pack_layout=gguf)
     rng = np.random.default_rng(3)
     h = rng.standard_normal((k, n_ff)).astype(np.float32)
@@ -181,8 +183,15 @@ def test_down_rounds_h_itself_like_the_quantizer(lib):
     h[1, 512:768] = 0.5
     h[2, 100], h[2, 200] = -7.0, 7.0          # the first (negative) maximum sets the sign of the scale
     h[3, 900], h[3, 300] = 9.0, -9.0
+    h[4, 300], h[4, 310] = 9.0, -9.0          # both in one run of 32
+    h[4, 600], h[4, 590] = 8.0, -8.0
+    h[5, 256 + 44], h[5, 256 + 20] = -5.0, 5.0
+    h[5, 512 + 20], h[5, 512 + 44] = -5.0, 5.0
+    h[6, 1024:1280] = -0.0
+    h[7, 1030] = -6.5                         # the largest magnitude of its block, and negative: no tie
+    h[7, 1100] = 6.25
     h_d = dev(h)
-    hq = lib.quant_act(22, h_d)
+    hq = lib.quant_act(22, h_d)           # Q8_K serves both down types
     w = dev(rng.uniform(0.05, 0.3, k).astype(np.float32))
     plan = store.table.clone()
     outs = []
