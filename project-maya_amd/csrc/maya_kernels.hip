@@ -419,6 +419,81 @@ struct alignas(16) RouterLds {
     unsigned long long lb[256], thr, cand[MAYA_MAX_K * (MAYA_MAX_EXPERTS / 256)];
     int nc;
 };
+// The largest of a wave's values, in every lane's scalar copy: exchanges inside the rows of 16 lanes (lane ^ 1, lane ^ 2,
+// the half-row and row mirrors), then lane 15 of a row to the next row and lane 31 to the upper half; lane 63 has it.
+__device__ __forceinline__ int wave_max_i32(int v) {
+    v = max(v, dpp_i<0xB1>(v));
+    v = max(v, dpp_i<0x4E>(v));
+    v = max(v, dpp_i<0x141>(v));
+    v = max(v, dpp_i<0x140>(v));
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x142, 0xa, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x143, 0xc, 0xf, false));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
+// Up to 256 experts, ONE wave, sm.ex filled: lane L keeps experts L, L + 64, L + 128, L + 192 in registers from the sum
+// to the weights, so nothing but the result touches LDS and no workgroup barrier sits on the path.
+//  * the sum: ascending, one add after the other (the reference's order).  The chain of dependent double adds is the
+//    critical path, so every add takes its operand from a lane by v_readlane, eight fetched ahead; all lanes carry the sum.
+//  * the k largest: k rounds of the reference's strict-> arg-max with the lower index on ties
+//    (src/kernels/cuda/router_top10.cu:140-176).  Probabilities are non-negative, so their bit patterns order like the
+//    values as signed integers and -1 marks "taken" or "no such expert"; a round is a 4-way maximum a lane, the wave
+//    maximum, and the first lane (lowest expert: lower register first, then lower lane) that holds it.
+//  * renormalisation: the k weights summed in slot order in double, one division a lane.
+__device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm) {
+    const int lane = threadIdx.x;
+    double ex[4];
+    int lo[4], hi[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int e = 64 * r + lane;
+        ex[r] = e < n_expert ? sm.ex[e] : 0.0;   // (+0.0 past the end: adding it changes nothing)
+        lo[r] = __double2loint(ex[r]);
+        hi[r] = __double2hiint(ex[r]);
+    }
+    double sum = 0.0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (64 * r < n_expert) {
+#pragma unroll
+            for (int j0 = 0; j0 < 64; j0 += 8) {
+                int sl[8], sh[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    sl[j] = __builtin_amdgcn_readlane(lo[r], j0 + j);
+                    sh[j] = __builtin_amdgcn_readlane(hi[r], j0 + j);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sum += __hiloint2double(sh[j], sl[j]);
+            }
+        }
+    }
+    const float inv = (float) (1.0 / sum);
+    int key[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) key[r] = 64 * r + lane < n_expert ? __float_as_int((float) (ex[r] * (double) inv)) : -1;
+    int my_id = 0, my_w = 0;
+    for (int i = 0; i < k; ++i) {
+        const int top = wave_max_i32(max(max(key[0], key[1]), max(key[2], key[3])));
+        unsigned long long b = __ballot(key[0] == top);
+        int r = 0;
+        if (b == 0ull) b = __ballot(key[1] == top), r = 1;
+        if (b == 0ull) b = __ballot(key[2] == top), r = 2;
+        if (b == 0ull) b = __ballot(key[3] == top), r = 3;
+        const int at = __builtin_ctzll(b);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) key[q] = (q == r && lane == at) ? -1 : key[q];
+        if (lane == i) my_id = 64 * r + at, my_w = top;
+    }
+    double s = 0.0;
+    for (int i = 0; i < k; ++i) s += (double) __int_as_float(__builtin_amdgcn_readlane(my_w, i));
+    const double sc = fmax(s, 6.103515625e-05);
+    if (lane < k) {
+        sm.id[lane] = my_id;
+        sm.w[lane] = (float) ((double) __int_as_float(my_w) / sc);
+    }
+}
+
 // 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights
 __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
     const int tid = threadIdx.x;
@@ -432,6 +507,11 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     __syncthreads();
     for (int e = tid; e < n_expert; e += 256) sm.ex[e] = exp((double) l[e] - (double) mx);
     __syncthreads();
+    if (n_expert <= 256) {
+        if (tid < 64) route_narrow(n_expert, k, sm);
+        __syncthreads();
+        return;
+    }
     if (tid < 64) {
         // ascending, one add after the other (the reference's order).  The chain of dependent double adds is the router's
         // critical path, so nothing else may sit on it: the first wave pulls the values into registers (lane L holds
@@ -470,34 +550,17 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     const float inv = (float) (1.0 / sm.sum);
     for (int e = tid; e < n_expert; e += 256) sm.p[e] = (float) (sm.ex[e] * (double) inv);
     __syncthreads();
-    // The k largest by rank, all at once: expert e's rank = the experts that beat it (a larger probability - they are
-    // non-negative, so their bit patterns order like the values - or an equal one at a lower index) - exactly the order in which k rounds of a strict-> arg-max with the lower index on ties
-    // would pick them (src/kernels/cuda/router_top10.cu:140-176), without the k dependent rounds.  Every thread reads
-    // the same p[j] at the same time (an LDS broadcast).
-    // (64-bit keys, probability bits above the complemented index, make "beats" one unsigned compare; they take the
-    // place of the exponentials, which are no longer needed)
+    // More than 256 experts: the k largest by rank.  Expert e's rank = the experts that beat it (a larger probability -
+    // they are non-negative, so their bit patterns order like the values - or an equal one at a lower index): exactly
+    // the order in which k rounds of a strict-> arg-max with the lower index on ties would pick them
+    // (src/kernels/cuda/router_top10.cu:140-176).  64-bit keys, probability bits above the complemented index, make
+    // "beats" one unsigned compare; they take the place of the exponentials, which are no longer needed.
     unsigned long long* key = (unsigned long long*) sm.ex;
     for (int e = tid; e < n_expert; e += 256)
         key[e] = ((unsigned long long) __float_as_uint(sm.p[e]) << 32) | (unsigned long long) (0xffffffffu - (unsigned) e);
     __syncthreads();
-    if (n_expert <= 256) {
-        for (int e = tid; e < n_expert; e += 256) {
-            const unsigned long long ke = key[e];
-            int rank = 0;
-            int j = 0;
-            for (; j + 2 <= n_expert; j += 2) {
-                const ulonglong2 kj = *(const ulonglong2*) (key + j);
-                rank += kj.x > ke ? 1 : 0;
-                rank += kj.y > ke ? 1 : 0;
-            }
-            for (; j < n_expert; ++j) rank += key[j] > ke ? 1 : 0;
-            if (rank < k) {
-                sm.id[rank] = e;
-                sm.w[rank] = sm.p[e];
-            }
-        }
-    } else {
-        // Wider routers: ranking every expert against every other grows with the square.  The k-th largest of the
+    {
+        // Ranking every expert against every other grows with the square.  The k-th largest of the
         // threads' best keys is a lower bound of the k-th largest key overall (those are k different experts), so only keys
         // at or above it can be among the k largest, and every key that beats one of them is at or above it too: the few
         // candidates (at most k threads' experts) are ranked among themselves.
