@@ -180,6 +180,28 @@ int maya_moe_gate_up_fuses_hq(const maya_moe_args* a);
 int maya_moe_down_rounds_h(const maya_moe_args* a);
 int maya_moe_down(const maya_moe_args* a, void* stream);
 
+/* ---- dense quantized mat-vecs beside the routed block (the shared expert's and the dense layers' projections):
+ * glmf::mv / glmf::MvJob (include/strata/kernels/glm_fast.hpp:23-55): y[c][r] = alpha * (W_r . x[c]) + (bias ? bias[r] : 0)
+ * for r in [0, n_out), c in [0, ncol).  The same weights meet ncol activations (a verify window's tokens); each column's
+ * sum is the single-column call's, bit for bit, and a row's weights are decoded once for up to 4 columns.  The
+ * activations are in the weight type's activation format (maya_quant_act: Q8_K for the K- and I-quants, Q8_0 for Q8_0 -
+ * the CPU path's contract; the reference's GPU form takes q8_1).  Up to MAYA_MV_MAX_JOBS independent jobs a call; jobs
+ * of one weight type share a launch.  n_in a multiple of 256, ncol <= MAYA_MAX_TOKENS. */
+#define MAYA_MV_MAX_JOBS 8
+typedef struct maya_mv_job {
+    const void* w;        /* n_out rows of n_in values of `type`, MAYA_PACK_GGUF or (IQ2_S: n_out a multiple of 4) MAYA_PACK_STREAM */
+    int32_t type, packing;
+    int32_t n_in, n_out;
+    int32_t ncol;
+    float alpha;
+    maya_act x;           /* [ncol][n_in] quantized activations */
+    const float* bias;    /* [n_out] or NULL */
+    float* y;             /* column c at y + c * y_stride */
+    int64_t y_stride;     /* floats; >= n_out */
+} maya_mv_job;
+int maya_mv_supported(int type);                                              /* glmf::mv_supported (glm_fast.hpp:52) */
+int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream);               /* glmf::mv / mv_nt (glm_fast.hpp:45-50) */
+
 /* ---- the whole routed layer for a decode step / verify window of n_tokens <= MAYA_MAX_TOKENS tokens:
  * route -> plan -> group -> quantize x -> gate/up -> quantize h -> down -> combine, every step on `stream`, nothing on
  * the host (the sequence of glm_fast_path.cu:2688-2691 and ds4_gguf.cu:1903-1971).

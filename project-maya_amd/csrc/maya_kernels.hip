@@ -1000,6 +1000,66 @@ __global__ __launch_bounds__(256) void combine_kernel(maya_moe_args a) {
     a.out[(size_t) t * n + c] = sum;
 }
 
+// ---- dense mat-vec jobs (glmf::mv, include/strata/kernels/glm_fast.hpp:23-55): the down kernel's row split - a wave
+// takes 2 rows a pass, 32 lanes a row, the activations staged in LDS, NT columns sharing one decode of a row - without
+// plan or groups; grid (rows / wg_rows, jobs).  y = alpha * dot + bias, each operation rounded.
+struct MvJobDev {
+    const uint8_t* w;
+    maya_act x;
+    const float* bias;
+    float* y;
+    long long y_stride;
+    float alpha;
+    int n_in, n_out, ncol, packing;
+};
+struct MvBatch {
+    MvJobDev job[MAYA_MV_MAX_JOBS];
+};
+template <int T, int NT>
+__global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb, int wg_rows) {
+    extern __shared__ int lds[];
+    const MvJobDev& j = b.job[blockIdx.y];
+    const int k = j.n_in, n_out = j.n_out;
+    if ((int) blockIdx.x * wg_rows >= n_out) return;
+    constexpr int cbw = Fmt<T>::kLdsWords;
+    if constexpr (cbw > 0) {
+        const int* src = (const int*) codebook_of<T>(cb);
+        for (int i = threadIdx.x; i < cbw; i += kDnThreads) lds[i] = src[i];
+    }
+    const uint2* grid = (const uint2*) lds;
+    int* lds_act = lds + cbw;
+    const int kq = k >> 2, kd = k >> 5;
+    ActLds al{lds_act, (const float*) (lds_act + NT * kq), lds_act + NT * kq + NT * kd, kq, kd};
+    const size_t drow = (size_t) (k / Fmt<T>::kValues) * Fmt<T>::kBytes;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
+    const bool quads = j.packing == MAYA_PACK_STREAM && T == kIQ2_S;
+    const bool packed = j.packing == MAYA_PACK_STREAM && (T == kIQ2_S || T == kQ8_0);
+    for (int c0 = 0; c0 < j.ncol; c0 += NT) {
+        int cols[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) cols[t] = c0 + t < j.ncol ? c0 + t : -1;
+        __syncthreads();
+        stage_act<T, NT>(lds_act, k, j.x, cols, Fmt<T>::kMin);
+        __syncthreads();
+        const int r_end = min(n_out, (int) (blockIdx.x + 1) * wg_rows);
+        for (int r = blockIdx.x * wg_rows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
+            float acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+            row_dot<T, NT, 32>(j.w + (size_t) (quads ? (r & ~3) : r) * drow, k, sub, al, grid, acc, packed, r & 3);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float sum = group_sum<32>(acc[t]);
+                if (sub == 0 && cols[t] >= 0) {
+                    float v = __fmul_rn(j.alpha, sum);
+                    if (j.bias) v = __fadd_rn(v, j.bias[r]);
+                    j.y[(size_t) cols[t] * j.y_stride + r] = v;
+                }
+            }
+        }
+    }
+}
+
 }  // namespace maya
 
 #include "maya_fast.cuh"
@@ -1271,6 +1331,21 @@ bool gate_up_by_entries(const maya_moe_args& a) {
 }
 bool down_by_entries(const maya_moe_args& a) { return down_q4k_pos_ok(a) || down_rounds_h(a); }
 
+template <int T>
+int launch_mv_t(const MvBatch& b, int n, int max_in, int max_out, int max_col, const DeviceState& st, hipStream_t s) {
+    int nt = max_col >= 4 ? 4 : max_col >= 2 ? 2 : 1;
+    while (nt > 1 && (size_t) codebook_words(T) * 4 + act_lds_bytes(max_in, nt) > (size_t) st.lds_limit) nt >>= 1;   // long rows: fewer columns a pass
+    const size_t lds = (size_t) codebook_words(T) * 4 + act_lds_bytes(max_in, nt);
+    if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "mv needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    const int wr = rows_per_wg(max_out, n, 16, kDnRows);
+    const dim3 grid((unsigned) ((max_out + wr - 1) / wr), (unsigned) n);
+    if (nt == 4) hipLaunchKernelGGL((mv_kernel<T, 4>), grid, dim3(kDnThreads), lds, s, b, st.cb, wr);
+    else if (nt == 2) hipLaunchKernelGGL((mv_kernel<T, 2>), grid, dim3(kDnThreads), lds, s, b, st.cb, wr);
+    else hipLaunchKernelGGL((mv_kernel<T, 1>), grid, dim3(kDnThreads), lds, s, b, st.cb, wr);
+    MAYA_LAUNCHED("mv_kernel");
+    return MAYA_OK;
+}
+
 }  // namespace maya
 
 using namespace maya;
@@ -1530,6 +1605,51 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     const dim3 grid((unsigned) ((a->layout.n_embd + 255) / 256), (unsigned) a->n_tokens);
     hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, s, *a);
     MAYA_LAUNCHED("combine_kernel");
+    return MAYA_OK;
+}
+
+int maya_mv_supported(int type) { return type_ok(type) ? 1 : 0; }
+
+int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!jobs || n_jobs < 1 || n_jobs > MAYA_MV_MAX_JOBS) return fail(MAYA_E_ARG, "mv: %d jobs outside 1..%d", n_jobs, MAYA_MV_MAX_JOBS);
+    for (int i = 0; i < n_jobs; ++i) {   // nothing is launched unless every job is covered
+        const maya_mv_job& j = jobs[i];
+        if (!type_ok(j.type)) return fail(MAYA_E_UNSUPPORTED, "mv: job %d: weight type %d is not covered", i, j.type);
+        if (j.packing != MAYA_PACK_GGUF && j.packing != MAYA_PACK_STREAM) return fail(MAYA_E_ARG, "mv: job %d: packing %d", i, j.packing);
+        if (j.n_in < 256 || j.n_in % 256 || j.n_in > 16384 || j.n_out < 1)
+            return fail(MAYA_E_SHAPE, "mv: job %d: n_in %d (a multiple of 256 up to 16384) / n_out %d", i, j.n_in, j.n_out);
+        if (j.ncol < 1 || j.ncol > MAYA_MAX_TOKENS) return fail(MAYA_E_SHAPE, "mv: job %d: ncol %d outside 1..%d", i, j.ncol, MAYA_MAX_TOKENS);
+        if (j.packing == MAYA_PACK_STREAM && j.type == kIQ2_S && j.n_out % 4)
+            return fail(MAYA_E_SHAPE, "mv: job %d: stream-packed IQ2_S rows come in quads, n_out %d", i, j.n_out);
+        if (j.packing == MAYA_PACK_STREAM && ((uintptr_t) j.w & 15)) return fail(MAYA_E_ARG, "mv: job %d: stream-packed weights must be 16-byte aligned", i);
+        if (!j.w || !j.x.q || !j.x.d || (q8k_act(j.type) && !j.x.bsums) || !j.y) return fail(MAYA_E_ARG, "mv: job %d: null pointer", i);
+        if (j.y_stride < j.n_out && j.ncol > 1) return fail(MAYA_E_ARG, "mv: job %d: y_stride %lld below n_out %d", i, (long long) j.y_stride, j.n_out);
+    }
+    static const int kTypes[] = {kQ8_0, kQ4_K, kIQ1_S, kIQ2_S, kIQ1_M};
+    for (const int t : kTypes) {
+        MvBatch b{};
+        int n = 0, max_in = 0, max_out = 0, max_col = 0;
+        for (int i = 0; i < n_jobs; ++i) {
+            const maya_mv_job& j = jobs[i];
+            if (j.type != t) continue;
+            b.job[n++] = MvJobDev{(const uint8_t*) j.w, j.x, j.bias, j.y, (long long) j.y_stride, j.alpha, j.n_in, j.n_out, j.ncol, j.packing};
+            max_in = j.n_in > max_in ? j.n_in : max_in;
+            max_out = j.n_out > max_out ? j.n_out : max_out;
+            max_col = j.ncol > max_col ? j.ncol : max_col;
+        }
+        if (n == 0) continue;
+        int rc;
+        switch (t) {
+            case kQ8_0: rc = launch_mv_t<kQ8_0>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+            case kQ4_K: rc = launch_mv_t<kQ4_K>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+            case kIQ1_S: rc = launch_mv_t<kIQ1_S>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+            case kIQ2_S: rc = launch_mv_t<kIQ2_S>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+            default: rc = launch_mv_t<kIQ1_M>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+        }
+        if (rc) return rc;
+    }
     return MAYA_OK;
 }
 

@@ -18,7 +18,7 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack",
-    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h",
+    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
 
 
@@ -44,6 +44,13 @@ class Args(C.Structure):
                 ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", Act), ("h", C.c_void_p),
                 ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p),
                 ("hq_sync", C.c_void_p)]
+
+
+class MvJob(C.Structure):
+    """maya_mv_job: y[c] = alpha * W x[c] + bias (glmf::MvJob, include/strata/kernels/glm_fast.hpp:29-43)."""
+    _fields_ = [("w", C.c_void_p), ("type", C.c_int32), ("packing", C.c_int32), ("n_in", C.c_int32), ("n_out", C.c_int32),
+                ("ncol", C.c_int32), ("alpha", C.c_float), ("x", Act), ("bias", C.c_void_p), ("y", C.c_void_p),
+                ("y_stride", C.c_int64)]
 
 
 _lib = None
@@ -77,6 +84,8 @@ def load():
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_gate_up_fuses_hq.argtypes = [C.POINTER(Args)]
     L.maya_moe_down_rounds_h.argtypes = [C.POINTER(Args)]
+    L.maya_mv_supported.argtypes = [i32]
+    L.maya_mv.argtypes = [C.POINTER(MvJob), i32, vp]
     L.maya_moe_workspace_bytes.restype = sz
     L.maya_moe_workspace_bytes.argtypes = [C.POINTER(Layout), i32, i32]
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
@@ -252,3 +261,24 @@ class MoeLayer:
                                            dtype_id(x), nt, limit, _p(add), _p(self.ids), _p(self.weights), _p(self.out),
                                            _p(self.ws), self.ws_bytes, _stream(stream)))
         return self.out[:nt]
+
+
+def mv(jobs, stream=None):
+    """jobs: dicts with w (uint8 rows), type, x [ncol, n_in] float activations, n_out and optionally packing, alpha, bias,
+    y; quantizes each x to the type's activation format and runs ONE maya_mv call.  Returns the outputs [ncol, n_out]."""
+    arr = (MvJob * len(jobs))()
+    keep, outs = [], []
+    for i, j in enumerate(jobs):
+        x = j["x"]
+        act = j.get("act") or quant_act(j["type"], x, stream)
+        y = j.get("y")
+        if y is None:
+            y = torch.empty((x.shape[0], j["n_out"]), dtype=torch.float32, device=x.device)
+        bias = j.get("bias")
+        arr[i] = MvJob(j["w"].data_ptr(), j["type"], j.get("packing", PACK_GGUF), x.shape[1], j["n_out"], x.shape[0],
+                       float(j.get("alpha", 1.0)), act.c(), bias.data_ptr() if bias is not None else None, y.data_ptr(),
+                       y.stride(0))
+        keep.append(act)
+        outs.append(y)
+    check(load().maya_mv(arr, len(jobs), _stream(stream)))
+    return outs
