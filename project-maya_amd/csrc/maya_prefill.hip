@@ -122,13 +122,11 @@ template <int DT> __device__ __forceinline__ float pf_load(const void* x, int64_
 }
 __device__ __forceinline__ int pf_rint(float f) { return (int) rintf(f); }
 
-// grid (k / 256, n_entries): row blockIdx.y of the plan, if there is one
+// grid (k / 256, tokens): a token's block is rounded once and written to the rows of all its entries in the plan
 template <int DT>
 __global__ __launch_bounds__(256) void prefill_quant_kernel(const void* __restrict__ x, int64_t x_stride, maya_prefill_plan p,
-                                                            int n_expert, int top_k, int64_t k, maya_prefill_act o) {
-    const int row = blockIdx.y;
-    if (row >= p.bounds[n_expert]) return;
-    const int t = p.row_entry[row] / top_k;
+                                                            int top_k, int64_t k, maya_prefill_act o) {
+    const int t = blockIdx.y;
     const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;
     const float xv = pf_load<DT>(x, (int64_t) t * x_stride + v);
     float am = fabsf(xv);
@@ -139,11 +137,15 @@ __global__ __launch_bounds__(256) void prefill_quant_kernel(const void* __restri
     int sum = c;
 #pragma unroll
     for (int s = 16; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
-    o.q[(size_t) row * k + v] = (int8_t) c;
-    if ((threadIdx.x & 31) == 0) {
-        const float d = __fdiv_rn(am, 127.0f);
-        o.d[((size_t) row * k + v) >> 5] = d;
-        o.s[((size_t) row * k + v) >> 5] = __fmul_rn(d, (float) sum);
+    const float d = __fdiv_rn(am, 127.0f), ds = __fmul_rn(d, (float) sum);
+    for (int j = 0; j < top_k; ++j) {
+        const int row = p.entry_row[t * top_k + j];
+        if (row < 0) continue;   // an entry of an expert that is not resident
+        o.q[(size_t) row * k + v] = (int8_t) c;
+        if ((threadIdx.x & 31) == 0) {
+            o.d[((size_t) row * k + v) >> 5] = d;
+            o.s[((size_t) row * k + v) >> 5] = ds;
+        }
     }
 }
 
@@ -494,12 +496,13 @@ int maya_moe_prefill_quant(const void* x, int x_dtype, int64_t x_stride, const m
     if (n_entries <= 0 || n_entries > 65535 || k <= 0 || n_embd <= 0 || n_embd % 256 || n_expert <= 0)
         return fail(MAYA_E_SHAPE, "prefill_quant: entries %d k %d n_embd %lld", n_entries, k, (long long) n_embd);
     if (x_stride == 0) x_stride = n_embd;
-    const dim3 grid((unsigned) (n_embd / 256), (unsigned) n_entries);
+    if (n_entries % k) return fail(MAYA_E_SHAPE, "prefill_quant: %d entries are not whole tokens of %d", n_entries, k);
+    const dim3 grid((unsigned) (n_embd / 256), (unsigned) (n_entries / k));
     hipStream_t s = as_stream(stream);
     switch (x_dtype) {
-        case MAYA_DT_F32: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, x, x_stride, *plan, n_expert, k, n_embd, xq); break;
-        case MAYA_DT_BF16: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, x, x_stride, *plan, n_expert, k, n_embd, xq); break;
-        default: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, x, x_stride, *plan, n_expert, k, n_embd, xq); break;
+        case MAYA_DT_F32: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, x, x_stride, *plan, k, n_embd, xq); break;
+        case MAYA_DT_BF16: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, x, x_stride, *plan, k, n_embd, xq); break;
+        default: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, x, x_stride, *plan, k, n_embd, xq); break;
     }
     MAYA_LAUNCHED("prefill_quant_kernel");
     return MAYA_OK;
