@@ -233,12 +233,16 @@ typedef struct maya_prefill_plan {
     int32_t* tile_row0;   /* [maya_moe_prefill_max_tiles()] */
     int32_t* n_tiles;     /* [1] */
 } maya_prefill_plan;
-/* Rows of activations as int8 codes with one F32 scale per 32 values, c = rint(x * (127 / amax)), d = amax / 127, and
- * s = d * (the 32 codes' sum) for the formats with a minimum. */
+/* Rows of activations in the CPU expert path's format for the K-quants, Q8_K (src/kernels/cuda/quantize_act.cu:161-207):
+ * int8 codes c = min(127, nearest_int(x * (-127 / max))) with max the signed value at the first largest magnitude of a
+ * 256-value block, one F32 scale d = 1 / (-127 / max) per block, and s = d * (the sum of every 32 codes), which the
+ * minimums of a Q4_K sub-block multiply.  The reference's two GPU prefill forms round per 32 values instead (q8_1,
+ * src/kernels/cuda/moe_mmq.cu:120; int8 + F32, src/prefill/moe_fused_rdna4.cu:87-109); this one reproduces the integer
+ * sums of the CPU path, which is what its results are checked against. */
 typedef struct maya_prefill_act {
     int8_t* q; /* [rows][k], 16-byte aligned */
-    float* d;  /* [rows][k / 32] */
-    float* s;  /* [rows][k / 32] */
+    float* d;  /* [rows][k / 256] */
+    float* s;  /* [rows][k / 32], 16-byte aligned */
 } maya_prefill_act;
 
 int maya_moe_prefill_tile_rows(void);
@@ -250,10 +254,12 @@ int maya_moe_prefill_plan(const int32_t* ids, int n_entries, const uint64_t* exp
 /* row r = the quantized x[row_entry[r] / k] for the plan's rows (rows past bounds[n_expert] are left alone) */
 int maya_moe_prefill_quant(const void* x, int x_dtype, int64_t x_stride, const maya_prefill_plan* plan, int n_entries,
                            int n_expert, int k, int64_t n_embd, maya_prefill_act xq, void* stream);
-/* hq row r = the per-32 int8 of swiglu(gate_e . x_r, up_e . x_r) (clamped by limit), e the row's expert; int8 MFMA over
- * the 4-bit codes and the activation codes, F32 scales per 32.  Expert blobs 8-byte aligned (GGUF packing). */
+/* h row r [n_ff] F32 = swiglu(gate_e . x_r, up_e . x_r) (clamped by limit), e the row's expert, and hq = its rounding
+ * (both written): int8 MFMA over two planes of the weights (their 4-bit codes times the low and the high 3 bits of
+ * their 6-bit sub-block scales) and the activation codes, int32 over a 256-value block - ggml_vec_dot_q4_K_q8_K's
+ * integer sums - then the two F32 scales of the block.  Matrix offsets 16-byte aligned (GGUF packing). */
 int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, const maya_prefill_plan* plan,
-                             int n_entries, maya_prefill_act xq, float limit, maya_prefill_act hq, void* stream);
+                             int n_entries, maya_prefill_act xq, float limit, float* h, maya_prefill_act hq, void* stream);
 /* part row r [n_embd] F32 = down_e . h_r */
 int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, const maya_prefill_plan* plan,
                           int n_entries, maya_prefill_act hq, float* part, void* stream);

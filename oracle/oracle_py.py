@@ -183,6 +183,10 @@ def vec_dot(t, row, k, act):
 
 
 def rows(t, w, k, n, act):
+    return rows_of(t, w, k, n, act)
+
+
+def rows_of(t, w, k, n, act):
     """w: n rows of type t; act: quantized activation bytes -> float32 [n]."""
     w = np.ascontiguousarray(w, dtype=np.uint8)
     rb = row_bytes(t, k)
@@ -306,35 +310,38 @@ def swiglu_rows(g, u, limit):
 
 
 def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=0.0, resident=None, nthreads=8):
-    """A prompt chunk's routed experts the way the reference's fused prefill defines them
-    (src/prefill/moe_fused_rdna4.cu:87-109, 620-660; tests/hip/prefill_fused_parity.cpp:150-175): per-32 int8 rows of
-    x, double products with the dequantized gate / up rows, the clamped SwiGLU in F32, H requantized per 32, double
-    products with the down rows, the weighted sum in slot order.  Returns a dict of every stage."""
+    """A prompt chunk's routed experts as the reference's CPU expert path computes each of them (Q8_K rows of x, the
+    gate / up row dots, the clamped SwiGLU, h rounded to Q8_K, the down row dots: src/kernels/cpu/native_expert.cpp:306-442)
+    in the plan's row order (src/kernels/cuda/glm_batch.cu:2102-2133), and the weighted sum in slot order.  Returns a dict
+    of every stage: xq / xd / xs = the rows' codes, block scales and d * (sum of every 32 codes); h = the SwiGLU values."""
     ids, w = router_topk(logits, k)
     ne = len(blobs)
     bounds, row_entry, entry_row = prefill_plan(ids, ne, resident)
     rows = row_entry.size
+    lim = float(limit) if limit and limit > 0 else float("inf")
     xq = np.zeros((rows, n_embd), dtype=np.int8)
-    xd = np.zeros((rows, n_embd // 32), dtype=np.float32)
-    cache = {}
+    xd = np.zeros((rows, n_embd // 256), dtype=np.float32)
+    xs = np.zeros((rows, n_embd // 32), dtype=np.float32)
+    h = np.zeros((rows, n_ff), dtype=np.float32)
+    part = np.zeros((rows, n_embd), dtype=np.float32)
+    acts = {}
+    sw = lib().mo_swiglu
     for r in range(rows):
-        tok = int(row_entry[r]) // k
-        if tok not in cache:
-            cache[tok] = quant_i8x32(x[tok])
-        xq[r], xd[r] = cache[tok]
-    used = [bounds[e + 1] > bounds[e] for e in range(ne)]
-    gate = grouped_ref(t, [blobs[e] if used[e] else None for e in range(ne)], bounds, n_embd, n_ff, xq, xd, nthreads)
-    up = grouped_ref(t, [blobs[e][up_off:] if used[e] else None for e in range(ne)], bounds, n_embd, n_ff, xq, xd, nthreads)
-    h = swiglu_rows(gate, up, limit)
-    hq = np.zeros((rows, n_ff), dtype=np.int8)
-    hd = np.zeros((rows, n_ff // 32), dtype=np.float32)
-    for r in range(rows):
-        hq[r], hd[r] = quant_i8x32(h[r])
-    part = grouped_ref(t, [blobs[e][down_off:] if used[e] else None for e in range(ne)], bounds, n_ff, n_embd, hq, hd, nthreads)
+        tok, e = int(row_entry[r]) // k, int(ids.reshape(-1)[row_entry[r]])
+        if tok not in acts:
+            a = quant_act(t, x[tok])
+            d, q, bs = q8k_fields(a)
+            acts[tok] = (a, q, d, (d[:, None] * (bs[:, 0::2] + bs[:, 1::2]).astype(np.float32)).reshape(-1))
+        a, xq[r], xd[r], xs[r] = acts[tok]
+        b = blobs[e]
+        g = rows_of(t, b, n_embd, n_ff, a)
+        u = rows_of(t, b[up_off:], n_embd, n_ff, a)
+        h[r] = [sw(float(gv), float(uv), lim) for gv, uv in zip(g, u)]
+        part[r] = rows_of(t, b[down_off:], n_ff, n_embd, quant_act(t, h[r]))
     out = np.zeros((x.shape[0], n_embd), dtype=np.float32)
     for tok in range(x.shape[0]):
         sel = [j for j in range(k) if entry_row[tok * k + j] >= 0]
         if sel:
             out[tok] = combine(np.stack([part[entry_row[tok * k + j]] for j in sel]), np.array([w[tok, j] for j in sel]))
-    return dict(ids=ids, w=w, bounds=bounds, row_entry=row_entry, entry_row=entry_row, xq=xq, xd=xd, h=h, hq=hq, hd=hd,
+    return dict(ids=ids, w=w, bounds=bounds, row_entry=row_entry, entry_row=entry_row, xq=xq, xd=xd, xs=xs, h=h,
                 part=part, out=out)

@@ -20,7 +20,6 @@ namespace maya {
 
 constexpr int kPfRows = 64;        // rows of a tile
 constexpr int kPfMt = kPfRows / 16;
-constexpr int kPfRowBytes = 272;   // a staged row of 256 codes: 4 banks' offset a row keeps the 8-byte reads apart
 constexpr int kPlanThreads = 1024;
 constexpr int kPlanWaves = kPlanThreads / 64;
 
@@ -122,34 +121,91 @@ template <int DT> __device__ __forceinline__ float pf_load(const void* x, int64_
 }
 __device__ __forceinline__ int pf_rint(float f) { return (int) rintf(f); }
 
+// ggml's nearest_int: the magic-number round (ties to even) of a product already rounded to F32
+__device__ __forceinline__ int pf_nearest_int(float f) {
+    const float v = __fadd_rn(f, 12582912.0f);
+    return (__float_as_int(v) & 0x007fffff) - 0x00400000;
+}
+// One 256-value block by the 256 threads of a workgroup (thread = value), Q8_K - the activation format of the
+// reference's CPU expert path for the K-quants (src/kernels/cuda/quantize_act.cu:161-207): the block's signed maximum
+// is the value at the FIRST largest magnitude, iscale = -127 / max, c = min(127, nearest_int(iscale x)), d = 1 / iscale;
+// s = d * (the sum of each 32 codes), what the minimums of a Q4_K sub-block multiply.  sm: 256 + 8 words.
+struct PfCodes {
+    int c;
+    float d, ds;
+};
+__device__ __forceinline__ PfCodes pf_quant_block(float xv, int* sm) {
+    const int j = threadIdx.x;
+    float am = fabsf(xv);
+    int ix = j;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float oa = __shfl_xor(am, o, 64);
+        const int oi = __shfl_xor(ix, o, 64);
+        if (oa > am || (oa == am && oi < ix)) am = oa, ix = oi;
+    }
+    float* s_x = (float*) sm;
+    float* s_am = (float*) (sm + 256);
+    int* s_ix = sm + 260;
+    s_x[j] = xv;
+    if ((j & 63) == 0) s_am[j >> 6] = am, s_ix[j >> 6] = ix;
+    __syncthreads();
+    am = s_am[0], ix = s_ix[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+        if (s_am[w] > am) am = s_am[w], ix = s_ix[w];   // (a later wave holds later indices: a tie keeps the earlier)
+    PfCodes o;
+    o.c = 0, o.d = 0.0f;
+    if (am > 0.0f) {
+        const float iscale = __fdiv_rn(-127.0f, s_x[ix]);
+        o.c = min(127, pf_nearest_int(__fmul_rn(iscale, xv)));
+        o.d = __fdiv_rn(1.0f, iscale);
+    }
+    int sum = o.c;
+#pragma unroll
+    for (int s = 16; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
+    o.ds = __fmul_rn(o.d, (float) sum);
+    __syncthreads();   // (sm is free for the next block)
+    return o;
+}
+__device__ __forceinline__ void pf_store_codes(const maya_prefill_act& o, size_t row, int64_t k, int64_t v, const PfCodes& c) {
+    const size_t at = row * (size_t) k + (size_t) v;
+    o.q[at] = (int8_t) c.c;
+    if ((threadIdx.x & 31) == 0) o.s[at >> 5] = c.ds;
+    if (threadIdx.x == 0) o.d[at >> 8] = c.d;
+}
+
 // grid (k / 256, tokens): a token's block is rounded once and written to the rows of all its entries in the plan
 template <int DT>
 __global__ __launch_bounds__(256) void prefill_quant_kernel(const void* __restrict__ x, int64_t x_stride, maya_prefill_plan p,
                                                             int top_k, int64_t k, maya_prefill_act o) {
+    __shared__ int sm[264];
     const int t = blockIdx.y;
     const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;
-    const float xv = pf_load<DT>(x, (int64_t) t * x_stride + v);
-    float am = fabsf(xv);
-#pragma unroll
-    for (int s = 16; s > 0; s >>= 1) am = fmaxf(am, __shfl_xor(am, s, 64));
-    const float inv = am > 0.0f ? __fdiv_rn(127.0f, am) : 0.0f;
-    const int c = pf_rint(__fmul_rn(xv, inv));
-    int sum = c;
-#pragma unroll
-    for (int s = 16; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
-    const float d = __fdiv_rn(am, 127.0f), ds = __fmul_rn(d, (float) sum);
+    const PfCodes c = pf_quant_block(pf_load<DT>(x, (int64_t) t * x_stride + v), sm);
     for (int j = 0; j < top_k; ++j) {
         const int row = p.entry_row[t * top_k + j];
         if (row < 0) continue;   // an entry of an expert that is not resident
-        o.q[(size_t) row * k + v] = (int8_t) c;
-        if ((threadIdx.x & 31) == 0) {
-            o.d[((size_t) row * k + v) >> 5] = d;
-            o.s[((size_t) row * k + v) >> 5] = ds;
-        }
+        pf_store_codes(o, (size_t) row, k, v, c);
     }
+}
+// grid (k / 256, rows at most): the plan's row blockIdx.y of an F32 matrix (the SwiGLU outputs)
+__global__ __launch_bounds__(256) void prefill_quant_rows_kernel(const float* __restrict__ x, maya_prefill_plan p, int n_expert,
+                                                                 int64_t k, maya_prefill_act o) {
+    __shared__ int sm[264];
+    const int row = blockIdx.y;
+    if (row >= p.bounds[n_expert]) return;
+    const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    const PfCodes c = pf_quant_block(x[(size_t) row * k + v], sm);
+    pf_store_codes(o, (size_t) row, k, v, c);
 }
 
 // ---------------------------------------------------------------------------------------------------- the GEMM
+// out[row][n] = sum over 256-value blocks b of (d_w[n][b] d_x[row][b]) * sum_j sc[n][j] (q[n] . c[row])_j  -  the
+// minimums' term: ggml_vec_dot_q4_K_q8_K's integer sums, exactly.  The 6-bit sub-block scale is split sc = 8 hi + lo, so
+// q sc = 8 (q hi) + (q lo) with both products <= 105: two int8 planes of the weights.  Their products with the codes run
+// on the int8 matrix cores and are accumulated in int32 over the whole 256-value block - the sub-block scales never leave
+// the integer domain, and the vector ALU converts and scales once per 256 values.
 struct PfGemm {
     const uint64_t* table;
     maya_prefill_plan plan;
@@ -157,43 +213,40 @@ struct PfGemm {
     int64_t k, n;          // inner length, weight rows of one matrix
     int64_t row_bytes;
     maya_prefill_act x;    // the tile rows' activations [rows][k]
-    maya_prefill_act h;    // gate/up: the requantized H [rows][n]
-    float* part;           // down: [rows][n]
+    float* out;            // gate/up: the SwiGLU outputs [rows][n] F32; down: part [rows][n]
     float limit;
 };
 
-struct PfStage {
-    uint4 q[4];
-    float4 sc;
-};
-// this thread's share of super-block sb of the tile's activations: 4 chunks of 16 codes, 4 scales (threads 0-127: d,
-// 128-255: s)
-__device__ __forceinline__ void pf_fetch(const PfGemm& a, int row0, int nrows, int sb, PfStage& st) {
-    const int tid = threadIdx.x;
+// LDS of one buffer: the codes [kPfRows][256] (16-byte chunk c of row r at position c ^ (r & 15): the 16 rows x 4
+// k-groups of a matrix-core operand read then hit distinct banks), s [kPfRows][8], d [kPfRows]
+constexpr int kPfPlane = kPfRows * 256;
+constexpr int kPfSOff = kPfPlane, kPfDOff = kPfSOff + kPfRows * 32;
+constexpr int kPfBufBytes = kPfDOff + kPfRows * 4;
+constexpr int kPfLdsBytes = 3 * kPfBufBytes;
+
+typedef const __attribute__((address_space(1))) void* pf_gptr;
+typedef __attribute__((address_space(3))) void* pf_lptr;
+// Super-block sb of the tile's activations, global memory -> LDS without passing registers (each lane's 16 bytes land
+// at the wave's base + 16 lane).  Rows past the tile's end repeat its last row (their results are never stored).
+template <int NMT>
+__device__ __forceinline__ void pf_dma(const PfGemm& a, uint8_t* buf, int row0, int nrows, int sb, int wave, int lane) {
+    const int last = nrows - 1;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int c = tid + 256 * i, r = c >> 4, col = c & 15;
-        st.q[i] = r < nrows ? *(const uint4*) (a.x.q + (size_t) (row0 + r) * a.k + (size_t) sb * 256 + col * 16) : make_uint4(0, 0, 0, 0);
+    for (int n = 0; n < NMT; ++n) {
+        const int i = wave + 4 * n;   // rows 4 i .. 4 i + 3
+        const int r = 4 * i + (lane >> 4), cp = lane & 15;
+        const size_t src = (size_t) (row0 + min(r, last)) * a.k + (size_t) sb * 256 + (size_t) ((cp ^ (r & 15)) * 16);
+        __builtin_amdgcn_global_load_lds((pf_gptr) (a.x.q + src), (pf_lptr) (buf + i * 1024), 16, 0, 0);
     }
-    const int r = (tid & 127) >> 1, half = tid & 1;
-    const float* src = (tid < 128 ? a.x.d : a.x.s) + (size_t) (row0 + r) * (a.k >> 5) + sb * 8 + half * 4;
-    st.sc = r < nrows ? *(const float4*) src : make_float4(0.f, 0.f, 0.f, 0.f);
-}
-// LDS of one buffer: codes [kPfRows][kPfRowBytes], d [8][kPfRows], s [8][kPfRows]
-constexpr int kPfBufBytes = kPfRows * kPfRowBytes + 2 * 8 * kPfRows * 4;
-__device__ __forceinline__ void pf_store(uint8_t* buf, const PfStage& st) {
-    const int tid = threadIdx.x;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int c = tid + 256 * i, r = c >> 4, col = c & 15;
-        *(uint4*) (buf + r * kPfRowBytes + col * 16) = st.q[i];
+    if (wave < 2 && 32 * wave < 16 * NMT) {   // s: 32 rows an instruction, 32 bytes a row
+        const int r = 32 * wave + (lane >> 1);
+        const float* src = a.x.s + (size_t) (row0 + min(r, last)) * (a.k >> 5) + sb * 8 + (lane & 1) * 4;
+        __builtin_amdgcn_global_load_lds((pf_gptr) src, (pf_lptr) (buf + kPfSOff + wave * 1024), 16, 0, 0);
     }
-    float* sc = (float*) (buf + kPfRows * kPfRowBytes) + (tid < 128 ? 0 : 8 * kPfRows);
-    const int r = (tid & 127) >> 1, half = tid & 1;
-    sc[(half * 4 + 0) * kPfRows + r] = st.sc.x;
-    sc[(half * 4 + 1) * kPfRows + r] = st.sc.y;
-    sc[(half * 4 + 2) * kPfRows + r] = st.sc.z;
-    sc[(half * 4 + 3) * kPfRows + r] = st.sc.w;
+    if (wave == 2) {
+        const float* src = a.x.d + (size_t) (row0 + min(lane, last)) * (a.k >> 8) + sb;
+        __builtin_amdgcn_global_load_lds((pf_gptr) src, (pf_lptr) (buf + kPfDOff), 4, 0, 0);
+    }
 }
 
 // the 8 six-bit scales and 8 six-bit minimums of a Q4_K block's 12 bytes, as bytes of two words each
@@ -204,7 +257,6 @@ __device__ __forceinline__ void q4k_unpack_scales(uint32_t s0, uint32_t s1, uint
     sc[1] = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
     mn[1] = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
 }
-__device__ __forceinline__ float byte_f32(uint32_t w, int i) { return (float) ((w >> (8 * i)) & 0xffu); }
 
 __device__ __forceinline__ float pf_swiglu(float g, float u, float limit) {
     if (limit > 0.0f && limit < INFINITY) {
@@ -214,60 +266,52 @@ __device__ __forceinline__ float pf_swiglu(float g, float u, float limit) {
     return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
 }
 
-// one tile of NMT x 16 rows (the row count of the tile is a compile-time bound, so the inner loop is branch-free and
-// the compiler can move the LDS reads of a step above the arithmetic of the one before)
-template <bool GU, int NMT>
-__device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t (*lds)[kPfBufBytes], int ex, int row0, int nrows) {
-    const uint8_t* blob = (const uint8_t*) a.table[ex];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+typedef unsigned short pf_u16x2 __attribute__((ext_vector_type(2)));
+// eight 4-bit codes (one a byte) times a factor <= 7: no byte overflows, so two packed 16-bit multiplies a word do it
+__device__ __forceinline__ long pf_scale_codes(uint64_t w, uint32_t f) {
+    const pf_u16x2 ff = {(unsigned short) f, (unsigned short) f};
+    const pf_u16x2 lo = __builtin_bit_cast(pf_u16x2, (uint32_t) w) * ff, hi = __builtin_bit_cast(pf_u16x2, (uint32_t) (w >> 32)) * ff;
+    return (long) (((uint64_t) __builtin_bit_cast(uint32_t, hi) << 32) | (uint64_t) __builtin_bit_cast(uint32_t, lo));
+}
 
-    // the 4 weight rows this lane feeds: gate/up: features f0 + ln and f0 + 16 + ln of gate, then of up
-    const uint8_t* wrow[4];
+// one tile of NMT x 16 rows against the wave's two tiles of 16 weight rows (gate/up: the gate and the up rows of 16
+// features)
+template <bool GU, int NMT>
+__device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, int row0, int nrows) {
+    const uint8_t* blob = (const uint8_t*) a.table[ex];
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const uint8_t* wrow[2];
     int64_t n0;   // the wave's first feature (gate/up) or output row (down)
     if constexpr (GU) {
+        n0 = (int64_t) blockIdx.x * 64 + wave * 16;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) wrow[t] = blob + a.off[t] + (size_t) (n0 + ln) * a.row_bytes;
+    } else {
         n0 = (int64_t) blockIdx.x * 128 + wave * 32;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) wrow[t] = blob + a.off[t >> 1] + (size_t) (n0 + 16 * (t & 1) + ln) * a.row_bytes;
-    } else {
-        n0 = (int64_t) blockIdx.x * 256 + wave * 64;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) wrow[t] = blob + a.off[0] + (size_t) (n0 + 16 * t + ln) * a.row_bytes;
+        for (int t = 0; t < 2; ++t) wrow[t] = blob + a.off[0] + (size_t) (n0 + 16 * t + ln) * a.row_bytes;
     }
     const bool wave_on = n0 < a.n;   // (a.n is a multiple of the wave's rows: checked on the host)
 
-    v4f acc[4][NMT];
+    v4f acc[2][NMT];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int m = 0; m < NMT; ++m) acc[t][m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     const int nsb = (int) (a.k >> 8);
-    PfStage st;
-    pf_fetch(a, row0, nrows, 0, st);
-    pf_store(lds[0], st);
-    // Weights run ahead of the arithmetic in registers.  Small tiles (1 or 2 groups of 16 rows) are bound by the weight
-    // stream: they keep a whole super-block in flight, and everything a lane needs of a row's 144-byte block (the 16-byte
-    // header and its four 8-byte slices of the codes) is requested in one burst, so the block's one or two cache lines are
-    // fetched once, not once per slice at different times.
-    // Tiles of 3 and 4 row groups have no registers to spare for a second block: their code slices run three slices
-    // ahead in a ring of four register sets instead (slice j in set j) and the header a block ahead.
-    constexpr bool kBurst = NMT <= 2;
-    uint64_t q[4][4], qn[kBurst ? 4 : 1][4];     // [slice j][row tile t]
-    uint32_t hdr[4][4], hdrn[kBurst ? 4 : 1][4];
-    auto load_q = [&](int sb, int j, uint64_t (&dst)[4]) {
+    // the activations run two super-blocks ahead through three LDS buffers, the weights one ahead in registers
+    pf_dma<NMT>(a, lds, row0, nrows, 0, wave, lane);
+    if (nsb > 1) pf_dma<NMT>(a, lds + kPfBufBytes, row0, nrows, 1, wave, lane);
+    // the weights of a super-block - the 16-byte header and the lane's four 8-byte slices of the codes of each of its two
+    // rows
+    uint64_t q[4][2], qn[4][2];     // [slice][row tile]
+    uint32_t hdr[2][4], hdrn[2][4];
+    auto load_block = [&](int sb, uint64_t (&dq)[4][2], uint32_t (&dh)[2][4]) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) dst[t] = *(const uint64_t*) (wrow[t] + (size_t) sb * 144 + 16 + 32 * j + 8 * g);
-    };
-    auto load_h = [&](int sb, uint32_t (&dh)[4][4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const uint4 h = *(const uint4*) (wrow[t] + (size_t) sb * 144);
-            dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
-        }
-    };
-    auto load_block = [&](int sb, uint64_t (&dq)[4][4], uint32_t (&dh)[4][4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < 2; ++t) {
             const uint8_t* blk = wrow[t] + (size_t) sb * 144;
             const uint4 h = *(const uint4*) blk;
             dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
@@ -275,101 +319,97 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t (*lds)[kPfBufBy
             for (int j = 0; j < 4; ++j) dq[j][t] = *(const uint64_t*) (blk + 16 + 32 * j + 8 * g);
         }
     };
-    if (wave_on) {
-        if constexpr (kBurst) load_block(0, q, hdr);
-        else {
-            load_h(0, hdr);
-            load_q(0, 0, q[0]);
-            load_q(0, 1, q[1]);
-            load_q(0, 2, q[2]);
-        }
-    }
+    if (wave_on) load_block(0, q, hdr);
+    const int a_base = ln * 256 + 8 * (g & 1), a_swz = (ln ^ (g >> 1)) << 4;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    int cur = 0;   // the buffer of super-block sb
     for (int sb = 0; sb < nsb; ++sb) {
-        const uint8_t* buf = lds[sb & 1];
-        if (sb + 1 < nsb) pf_fetch(a, row0, nrows, sb + 1, st);
+        const uint8_t* buf = lds + cur * kPfBufBytes;
+        const int nxt2 = cur == 0 ? 2 : cur - 1;   // the buffer of super-block sb + 2
+        float d[2], dmin[2];
+        uint32_t sc[2][2], mn[2][2];
         if (wave_on) {
-            float d[4], dmin[4];
-            uint32_t sc[4][2], mn[4][2];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < 2; ++t) {
                 d[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] & 0xffffu));
                 dmin[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] >> 16));
                 q4k_unpack_scales(hdr[t][1], hdr[t][2], hdr[t][3], sc[t], mn[t]);
             }
-            if (sb + 1 < nsb) {
-                if constexpr (kBurst) load_block(sb + 1, qn, hdrn);
-                else load_h(sb + 1, hdr);   // (decoded above: its registers are free)
-            }
-            const float* sxl = (const float*) (buf + kPfRows * kPfRowBytes);
-            const float* ssl = sxl + 8 * kPfRows;
+            if (sb + 1 < nsb) load_block(sb + 1, qn, hdrn);
+        }
+        // (after the weights' loads, so that waiting for everything but these copies covers the weights too)
+        if (sb + 2 < nsb) pf_dma<NMT>(a, lds + nxt2 * kPfBufBytes, row0, nrows, sb + 2, wave, lane);
+        if (wave_on) {
             // the minimums' term, -(dmin m) . s over the 8 sub-blocks, on the matrix cores in F32: A = the tokens' s
             // (row = token, k = sub-block), B = this lane's row's -dmin m, accumulated straight into acc
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                float nb[4];
+                float nb[2];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) nb[t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
+                for (int t = 0; t < 2; ++t) nb[t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
 #pragma unroll
                 for (int m = 0; m < NMT; ++m) {
-                    const float sa = ssl[(4 * half + g) * kPfRows + 16 * m + ln];
+                    const float sa = *(const float*) (buf + kPfSOff + (16 * m + ln) * 32 + (4 * half + g) * 4);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa, nb[t], acc[t][m], 0, 0, 0);
+                    for (int t = 0; t < 2; ++t) acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa, nb[t], acc[t][m], 0, 0, 0);
                 }
             }
+            // The two plane products of the block, int32: [t][m][0] = (q lo) . c, [1] = (q hi) . c.  One 64-deep matrix
+            // instruction takes the two sub-blocks of a 32-byte slice of the codes: a lane's first 8 operand bytes are the
+            // low nibbles (sub-block 2p, values 8 g .. 8 g + 7), its second 8 the high nibbles (sub-block 2p + 1, the same
+            // values), each times its own sub-block's factor; the activations' operand pairs the same two runs of 8 codes.
+            v4i dot[2][NMT][2];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if constexpr (!kBurst) {   // slice (sb, j) + 3 into the set that slice (sb, j) - 1 has left
-                    const int jn = (j + 3) & 3, sbn = sb + ((j + 3) >> 2);
-                    if (sbn < nsb) load_q(sbn, jn, q[jn]);
+            for (int p = 0; p < 4; ++p) {
+                v4i wl[2], wh[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint64_t w0 = q[p][t] & 0x0f0f0f0f0f0f0f0full, w1 = (q[p][t] >> 4) & 0x0f0f0f0f0f0f0f0full;
+                    const uint32_t s2 = sc[t][p >> 1] >> (16 * (p & 1));
+                    const uint32_t sa = s2 & 0x3fu, sb6 = (s2 >> 8) & 0x3fu;
+                    const long l0 = pf_scale_codes(w0, sa & 7u), l1 = pf_scale_codes(w1, sb6 & 7u);
+                    const long h0 = pf_scale_codes(w0, sa >> 3), h1 = pf_scale_codes(w1, sb6 >> 3);
+                    wl[t] = v4i{(int) l0, (int) (l0 >> 32), (int) l1, (int) (l1 >> 32)};
+                    wh[t] = v4i{(int) h0, (int) (h0 >> 32), (int) h1, (int) (h1 >> 32)};
                 }
+                const int at0 = a_base + (a_swz ^ (64 * p)), at1 = a_base + (a_swz ^ (64 * p + 32));
 #pragma unroll
-                for (int nib = 0; nib < 2; ++nib) {
-                    const int blk = 2 * j + nib;
-                    long wb[4];
-                    float dsc[4];
+                for (int m = 0; m < NMT; ++m) {
+                    const int2 x0 = *(const int2*) (buf + at0 + m * 4096), x1 = *(const int2*) (buf + at1 + m * 4096);
+                    const v4i xc = {x0.x, x0.y, x1.x, x1.y};
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        wb[t] = (long) ((q[j][t] >> (4 * nib)) & 0x0f0f0f0f0f0f0f0full);
-                        // (the scale word is made opaque here: converted up front for all 8 sub-blocks, the 32 products
-                        // would sit in registers for the whole super-block)
-                        uint32_t scw = sc[t][blk >> 2];
-                        asm volatile("" : "+v"(scw));
-                        dsc[t] = __fmul_rn(d[t], byte_f32(scw, blk & 3));
+                    for (int t = 0; t < 2; ++t) {
+                        const v4i z = {0, 0, 0, 0};
+                        dot[t][m][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xc, wl[t], p ? dot[t][m][0] : z, 0, 0, 0);
+                        dot[t][m][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xc, wh[t], p ? dot[t][m][1] : z, 0, 0, 0);
                     }
-#pragma unroll
-                    for (int m = 0; m < NMT; ++m) {
-                        const long xa = *(const long*) (buf + (16 * m + ln) * kPfRowBytes + blk * 32 + 8 * g);
-                        const float4 sx = *(const float4*) (sxl + blk * kPfRows + 16 * m + 4 * g);
-                        const float sxa[4] = {sx.x, sx.y, sx.z, sx.w};
-                        v4i dot[4];
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) dot[t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, wb[t], v4i{0, 0, 0, 0}, 0, 0, 0);
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                            for (int i = 0; i < 4; ++i)
-                                acc[t][m][i] = fmaf(__fmul_rn(dsc[t], sxa[i]), (float) dot[t][i], acc[t][m][i]);
-                            // (pinned: left free, the optimizer issues every dot of the super-block first and holds
-                            // their 128 results in registers)
-                            asm volatile("" : "+v"(acc[t][m]));
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);   // a sub-block's work stays together
                 }
             }
-            if constexpr (kBurst) {
-                if (sb + 1 < nsb) {
+            // once a block: lo + 8 hi = the block's integer sum (< 2^25), then its two scales
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
+            for (int m = 0; m < NMT; ++m) {
+                const float4 dx4 = *(const float4*) (buf + kPfDOff + (16 * m + 4 * g) * 4);
+                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i], q[i][t] = qn[i][t];
-                    }
+                for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[t][m][i] = fmaf(__fmul_rn(dx[i], d[t]), (float) (dot[t][m][0][i] + 8 * dot[t][m][1][i]), acc[t][m][i]);
+                }
+            }
+            if (sb + 1 < nsb) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i], q[i][t] = qn[i][t];
                 }
             }
         }
-        if (sb + 1 < nsb) pf_store(lds[(sb + 1) & 1], st);
+        // super-block sb + 1 has landed once only this iteration's copies (of sb + 2) may still be in flight
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NMT) : "memory");
         __syncthreads();
+        cur = cur == 2 ? 0 : cur + 1;
     }
     if (!wave_on) return;
 
@@ -379,35 +419,10 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t (*lds)[kPfBufBy
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = 16 * m + 4 * g + i;
-            const bool on = r < nrows;
-            if constexpr (GU) {
-                // 32 features of one token: this lane's 2, the 16 lanes of its group
-                const float h0 = pf_swiglu(acc[0][m][i], acc[2][m][i], a.limit);
-                const float h1 = pf_swiglu(acc[1][m][i], acc[3][m][i], a.limit);
-                float am = fmaxf(fabsf(h0), fabsf(h1));
-#pragma unroll
-                for (int s = 8; s > 0; s >>= 1) am = fmaxf(am, __shfl_xor(am, s, 64));
-                const float inv = am > 0.0f ? __fdiv_rn(127.0f, am) : 0.0f;
-                const int c0 = pf_rint(__fmul_rn(h0, inv)), c1 = pf_rint(__fmul_rn(h1, inv));
-                int sum = c0 + c1;
-#pragma unroll
-                for (int s = 8; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
-                if (on) {
-                    int8_t* q = a.h.q + (size_t) (row0 + r) * a.n + n0;
-                    q[ln] = (int8_t) c0;
-                    q[16 + ln] = (int8_t) c1;
-                    if (ln == 0) {
-                        const float dd = __fdiv_rn(am, 127.0f);
-                        const size_t b = ((size_t) (row0 + r) * a.n + n0) >> 5;
-                        a.h.d[b] = dd;
-                        a.h.s[b] = __fmul_rn(dd, (float) sum);
-                    }
-                }
-            } else if (on) {
-                float* o = a.part + (size_t) (row0 + r) * a.n + n0 + ln;
-#pragma unroll
-                for (int t = 0; t < 4; ++t) o[16 * t] = acc[t][m][i];
-            }
+            if (r >= nrows) continue;
+            float* o = a.out + (size_t) (row0 + r) * a.n + n0 + ln;
+            if constexpr (GU) o[0] = pf_swiglu(acc[0][m][i], acc[1][m][i], a.limit);
+            else o[0] = acc[0][m][i], o[16] = acc[1][m][i];
         }
     }
 }
@@ -415,16 +430,16 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t (*lds)[kPfBufBy
 // grid (bands of weight rows, tiles at most)
 template <bool GU>
 __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][kPfBufBytes];
+    extern __shared__ __attribute__((aligned(16))) uint8_t pf_lds[];
     const int tile = blockIdx.y;
     if (tile >= *a.plan.n_tiles) return;
     const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
     const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
     switch ((nrows + 15) >> 4) {
-        case 1: pf_tile<GU, 1>(a, lds, ex, row0, nrows); break;
-        case 2: pf_tile<GU, 2>(a, lds, ex, row0, nrows); break;
-        case 3: pf_tile<GU, 3>(a, lds, ex, row0, nrows); break;
-        default: pf_tile<GU, 4>(a, lds, ex, row0, nrows); break;
+        case 1: pf_tile<GU, 1>(a, pf_lds, ex, row0, nrows); break;
+        case 2: pf_tile<GU, 2>(a, pf_lds, ex, row0, nrows); break;
+        case 3: pf_tile<GU, 3>(a, pf_lds, ex, row0, nrows); break;
+        default: pf_tile<GU, 4>(a, pf_lds, ex, row0, nrows); break;
     }
 }
 
@@ -457,7 +472,21 @@ __global__ __launch_bounds__(256) void prefill_combine_kernel(const int32_t* __r
 static bool plan_ok(const maya_prefill_plan* p) {
     return p && p->bounds && p->row_entry && p->entry_row && p->tile_expert && p->tile_row0 && p->n_tiles;
 }
-static bool act_ok(const maya_prefill_act& a) { return a.q && a.d && a.s && ((uintptr_t) a.q & 15) == 0 && ((uintptr_t) a.d & 15) == 0 && ((uintptr_t) a.s & 15) == 0; }
+static bool act_ok(const maya_prefill_act& a) {
+    return a.q && a.d && a.s && (((uintptr_t) a.q | (uintptr_t) a.s) & 15) == 0 && ((uintptr_t) a.d & 3) == 0;
+}
+// the GEMM kernels' three LDS buffers are dynamic
+template <bool GU>
+static int pf_launch(const PfGemm& a, dim3 grid, hipStream_t s) {
+    constexpr int lds = kPfLdsBytes;
+    static bool raised[2] = {false, false};
+    if (!raised[GU]) {
+        MAYA_HIP(hipFuncSetAttribute((const void*) prefill_q4k_kernel<GU>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        raised[GU] = true;
+    }
+    hipLaunchKernelGGL(prefill_q4k_kernel<GU>, grid, dim3(256), lds, s, a);
+    return MAYA_OK;
+}
 
 }  // namespace maya
 
@@ -521,12 +550,11 @@ static int prefill_check(const char* what, const maya_moe_layout* l, const uint6
 }
 
 int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, const maya_prefill_plan* plan,
-                             int n_entries, maya_prefill_act xq, float limit, maya_prefill_act hq, void* stream) {
+                             int n_entries, maya_prefill_act xq, float limit, float* h, maya_prefill_act hq, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (const int rc = prefill_check("prefill_gate_up", l, expert_table, n_expert, plan, n_entries, l ? l->gate_type : 0, l ? l->up_type : 0)) return rc;
-    if (!act_ok(xq) || !act_ok(hq)) return fail(MAYA_E_ARG, "prefill_gate_up: null or misaligned activations");
-    if (l->n_ff % 128) return fail(MAYA_E_SHAPE, "prefill_gate_up: n_ff %d: a multiple of 128 wanted", l->n_ff);
+    if (!act_ok(xq) || !act_ok(hq) || !h) return fail(MAYA_E_ARG, "prefill_gate_up: null or misaligned activations");
     PfGemm a{};
     a.table = expert_table;
     a.plan = *plan;
@@ -536,11 +564,14 @@ int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_ta
     a.n = l->n_ff;
     a.row_bytes = (int64_t) (l->n_embd / 256) * 144;
     a.x = xq;
-    a.h = hq;
+    a.out = h;
     a.limit = limit;
-    const dim3 grid((unsigned) (l->n_ff / 128), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
-    hipLaunchKernelGGL(prefill_q4k_kernel<true>, grid, dim3(256), 0, as_stream(stream), a);
+    const dim3 grid((unsigned) (l->n_ff / 64), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
+    if (const int rc = pf_launch<true>(a, grid, as_stream(stream))) return rc;
     MAYA_LAUNCHED("prefill_q4k_kernel<gate_up>");
+    const dim3 qgrid((unsigned) (l->n_ff / 256), (unsigned) n_entries);
+    hipLaunchKernelGGL(prefill_quant_rows_kernel, qgrid, dim3(256), 0, as_stream(stream), (const float*) h, *plan, n_expert, (int64_t) l->n_ff, hq);
+    MAYA_LAUNCHED("prefill_quant_rows_kernel");
     return MAYA_OK;
 }
 
@@ -550,7 +581,7 @@ int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table
     if (const int rc = current_state(&st)) return rc;
     if (const int rc = prefill_check("prefill_down", l, expert_table, n_expert, plan, n_entries, l ? l->down_type : 0, l ? l->down_type : 0)) return rc;
     if (!act_ok(hq) || !part) return fail(MAYA_E_ARG, "prefill_down: null or misaligned pointer");
-    if (l->n_embd % 64) return fail(MAYA_E_SHAPE, "prefill_down: n_embd %d", l->n_embd);
+    if (l->n_embd % 32) return fail(MAYA_E_SHAPE, "prefill_down: n_embd %d", l->n_embd);
     PfGemm a{};
     a.table = expert_table;
     a.plan = *plan;
@@ -559,9 +590,9 @@ int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table
     a.n = l->n_embd;
     a.row_bytes = (int64_t) (l->n_ff / 256) * 144;
     a.x = hq;
-    a.part = part;
-    const dim3 grid((unsigned) ((l->n_embd + 255) / 256), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
-    hipLaunchKernelGGL(prefill_q4k_kernel<false>, grid, dim3(256), 0, as_stream(stream), a);
+    a.out = part;
+    const dim3 grid((unsigned) ((l->n_embd + 127) / 128), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
+    if (const int rc = pf_launch<false>(a, grid, as_stream(stream))) return rc;
     MAYA_LAUNCHED("prefill_q4k_kernel<down>");
     return MAYA_OK;
 }
@@ -587,7 +618,7 @@ int maya_moe_prefill_combine(const maya_prefill_plan* plan, const float* weights
 struct PrefillWs {
     maya_prefill_plan plan;
     maya_prefill_act x, h;
-    float* part;
+    float *hf, *part;
     size_t bytes;
 };
 static PrefillWs prefill_carve(const maya_moe_layout& l, int n_tokens, int k, int n_expert, uint8_t* base) {
@@ -606,12 +637,14 @@ static PrefillWs prefill_carve(const maya_moe_layout& l, int n_tokens, int k, in
     w.plan.tile_expert = (int32_t*) take(4 * mt);
     w.plan.tile_row0 = (int32_t*) take(4 * mt);
     w.plan.n_tiles = (int32_t*) take(4);
-    w.x.q = (int8_t*) take(ne * l.n_embd);
-    w.x.d = (float*) take(ne * (l.n_embd / 32) * 4);
-    w.x.s = (float*) take(ne * (l.n_embd / 32) * 4);
-    w.h.q = (int8_t*) take(ne * l.n_ff);
-    w.h.d = (float*) take(ne * (l.n_ff / 32) * 4);
-    w.h.s = (float*) take(ne * (l.n_ff / 32) * 4);
+    auto take_act = [&](maya_prefill_act& a, size_t k) {
+        a.q = (int8_t*) take(ne * k);
+        a.d = (float*) take(ne * (k / 256) * 4);
+        a.s = (float*) take(ne * (k / 32) * 4);
+    };
+    take_act(w.x, (size_t) l.n_embd);
+    take_act(w.h, (size_t) l.n_ff);
+    w.hf = (float*) take(ne * l.n_ff * 4);
     w.part = (float*) take(ne * l.n_embd * 4);
     w.bytes = off;
     return w;
@@ -634,7 +667,7 @@ int maya_moe_prefill_layer(const maya_moe_layout* l, const uint64_t* expert_tabl
     if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
     if ((rc = maya_moe_prefill_plan(ids, ne, expert_table, n_expert, &w.plan, stream))) return rc;
     if ((rc = maya_moe_prefill_quant(x, x_dtype, 0, &w.plan, ne, n_expert, k, l->n_embd, w.x, stream))) return rc;
-    if ((rc = maya_moe_prefill_gate_up(l, expert_table, n_expert, &w.plan, ne, w.x, limit, w.h, stream))) return rc;
+    if ((rc = maya_moe_prefill_gate_up(l, expert_table, n_expert, &w.plan, ne, w.x, limit, w.hf, w.h, stream))) return rc;
     if ((rc = maya_moe_prefill_down(l, expert_table, n_expert, &w.plan, ne, w.h, w.part, stream))) return rc;
     return maya_moe_prefill_combine(&w.plan, weights, w.part, n_tokens, k, l->n_embd, add, out, out_dtype, stream);
 }

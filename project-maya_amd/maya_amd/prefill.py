@@ -32,7 +32,7 @@ def load():
         lib.maya_moe_prefill_supported.argtypes = [i32]
         lib.maya_moe_prefill_plan.argtypes = [vp, i32, vp, i32, PP, vp]
         lib.maya_moe_prefill_quant.argtypes = [vp, i32, i64, PP, i32, i32, i32, i64, PAct, vp]
-        lib.maya_moe_prefill_gate_up.argtypes = [LP, vp, i32, PP, i32, PAct, f32, PAct, vp]
+        lib.maya_moe_prefill_gate_up.argtypes = [LP, vp, i32, PP, i32, PAct, f32, vp, PAct, vp]
         lib.maya_moe_prefill_down.argtypes = [LP, vp, i32, PP, i32, PAct, vp, vp]
         lib.maya_moe_prefill_combine.argtypes = [PP, vp, vp, i32, i32, i64, vp, vp, i32, vp]
         lib.maya_moe_prefill_workspace_bytes.restype = sz
@@ -63,7 +63,7 @@ class PlanBuf:
 class ActRows:
     def __init__(self, rows, k, device="cuda"):
         self.q = torch.zeros((rows, k), dtype=torch.int8, device=device)
-        self.d = torch.zeros((rows, k // 32), dtype=torch.float32, device=device)
+        self.d = torch.zeros((rows, k // 256), dtype=torch.float32, device=device)
         self.s = torch.zeros((rows, k // 32), dtype=torch.float32, device=device)
         self.c = PAct(self.q.data_ptr(), self.d.data_ptr(), self.s.data_ptr())
 
@@ -84,8 +84,9 @@ def quant(x, p, k, stream=None):
 
 def gate_up(layout, expert_table, p, xq, limit=0.0, stream=None):
     h = ActRows(p.n_entries, layout.n_ff, xq.q.device)
+    h.f32 = torch.zeros((p.n_entries, layout.n_ff), dtype=torch.float32, device=xq.q.device)   # the values before rounding
     L.check(load().maya_moe_prefill_gate_up(C.byref(layout), L._p(expert_table), p.n_expert, C.byref(p.c), p.n_entries, xq.c,
-                                            limit, h.c, L._stream(stream)))
+                                            limit, L._p(h.f32), h.c, L._stream(stream)))
     return h
 
 

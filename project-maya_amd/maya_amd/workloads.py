@@ -155,7 +155,7 @@ def batch8_mixed(K, W):
 
 
 def prefill_q4k(K, W):
-    """configs[3]: 512 tokens, 256 Q4_K experts top-8, Zipf(1.1)-skewed routing, per-32 int8 activations, bf16 out."""
+    """configs[3]: 512 tokens, 256 Q4_K experts top-8, Zipf(1.1)-skewed routing, int8 (Q8_K) activations, bf16 out."""
     E, FF, NE, TK, T = 7168, 2048, 256, 8, 512
     layout, bb = lib.layout(lib.Q4_K, lib.Q4_K, E, FF)
     pool = random_blocks(NE * bb, 144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}, 11)
@@ -170,21 +170,23 @@ def prefill_q4k(K, W):
     ids, w = lib.route_topk(logits, TK)
     used = int(torch.unique(ids).numel())
     ops = 2 * 3 * E * FF * T * TK
-    nbytes = used * bb + T * E * (1 + 4 / 32) + T * E * 2
+    nbytes = used * bb + T * E * 4 + T * E * 2
     # the dominant kernel alone: the gate/up GEMM (2/3 of the operations)
     with torch.cuda.stream(stream):
         p = prefill.plan(ids.reshape(-1), table)
         xq = prefill.quant(x, p, TK)
         hq = prefill.ActRows(p.n_entries, FF)
+        hf = torch.empty((p.n_entries, FF), dtype=torch.float32, device="cuda")
         L = prefill.load()
+        # (the call also rounds h: its small kernel rides in the measured time)
         sec_gu = event_time(lambda: lib.check(L.maya_moe_prefill_gate_up(C.byref(layout), lib._p(table), NE, C.byref(p.c), p.n_entries,
-                                                                         xq.c, 0.0, hq.c, lib._stream())), 8, stream)
+                                                                         xq.c, 0.0, lib._p(hf), hq.c, lib._stream())), 8, stream)
     ops_gu = 2 * 2 * E * FF * T * TK
     tops_gu = ops_gu / sec_gu / 1e12
     return {"metric": "prefill_int8_tops_512tok", "value": round(ops / sec / 1e12, 2), "unit": "TOP/s", "ms_per_step": sec * 1e3,
             "dtype": "int8",
             "config": {"workload": "configs[3]: prefill chunk of 512 tokens, 256 experts Q4_K top-8, logits N(0,1) - 1.1 ln(e+1), "
-                                   "per-32 int8 activations, bf16 out", "experts_with_rows": used, "int8_ops_per_step": ops,
+                                   "int8 activations in the CPU path's Q8_K rounding, bf16 out", "experts_with_rows": used, "int8_ops_per_step": ops,
                        "algorithmic_bytes_per_step": int(nbytes), "weight_gbps": round(nbytes / sec / 1e9, 1),
                        "pct_of_hbm_peak": round(100 * nbytes / sec / HBM_PEAK, 2)},
             "roofline": {"bound": "mfma", "kernel": "prefill_q4k_kernel<gate_up>", "achieved": round(tops_gu, 2), "peak": 5000.0,
