@@ -222,32 +222,41 @@ struct PfGemm {
 constexpr int kPfPlane = kPfRows * 256;
 constexpr int kPfSOff = kPfPlane, kPfDOff = kPfSOff + kPfRows * 32;
 constexpr int kPfBufBytes = kPfDOff + kPfRows * 4;
-constexpr int kPfLdsBytes = 3 * kPfBufBytes;
 
-typedef const __attribute__((address_space(1))) void* pf_gptr;
 typedef __attribute__((address_space(3))) void* pf_lptr;
-// Super-block sb of the tile's activations, global memory -> LDS without passing registers (each lane's 16 bytes land
-// at the wave's base + 16 lane).  Rows past the tile's end repeat its last row (their results are never stored).
+// The tile's activations go from global memory to LDS without passing registers (each lane's 16 bytes land at the
+// wave's base + 16 lane): buffer loads whose per-lane offsets are fixed for the tile - the super-block rides in the
+// scalar offset - so a copy costs no vector arithmetic.  Rows past the tile's end repeat its last row (their results
+// are never stored).
 template <int NMT>
-__device__ __forceinline__ void pf_dma(const PfGemm& a, uint8_t* buf, int row0, int nrows, int sb, int wave, int lane) {
-    const int last = nrows - 1;
+struct PfDma {
+    __amdgpu_buffer_rsrc_t rq, rs, rd;
+    uint32_t oq[NMT], os, od;
+    int wave;
+    __device__ __forceinline__ void init(const PfGemm& a, int row0, int nrows, int wave_, int lane) {
+        wave = wave_;
+        const int last = nrows - 1;
+        rq = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.q + (size_t) row0 * a.k), 0, (int) (nrows * a.k), 0x00020000);
+        rs = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.s + (size_t) row0 * (a.k >> 5)), 0, (int) (nrows * (a.k >> 5) * 4), 0x00020000);
+        rd = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.d + (size_t) row0 * (a.k >> 8)), 0, (int) (nrows * (a.k >> 8) * 4), 0x00020000);
 #pragma unroll
-    for (int n = 0; n < NMT; ++n) {
-        const int i = wave + 4 * n;   // rows 4 i .. 4 i + 3
-        const int r = 4 * i + (lane >> 4), cp = lane & 15;
-        const size_t src = (size_t) (row0 + min(r, last)) * a.k + (size_t) sb * 256 + (size_t) ((cp ^ (r & 15)) * 16);
-        __builtin_amdgcn_global_load_lds((pf_gptr) (a.x.q + src), (pf_lptr) (buf + i * 1024), 16, 0, 0);
+        for (int n = 0; n < NMT; ++n) {
+            const int r = 4 * (wave + 4 * n) + (lane >> 4), cp = lane & 15;   // rows 4 i .. 4 i + 3, i = wave + 4 n
+            oq[n] = (uint32_t) (min(r, last) * (int) a.k + ((cp ^ (r & 15)) * 16));
+        }
+        os = (uint32_t) (min(32 * wave + (lane >> 1), last) * (int) (a.k >> 5) * 4 + (lane & 1) * 16);
+        od = (uint32_t) (min(lane, last) * (int) (a.k >> 8) * 4);
     }
-    if (wave < 2 && 32 * wave < 16 * NMT) {   // s: 32 rows an instruction, 32 bytes a row
-        const int r = 32 * wave + (lane >> 1);
-        const float* src = a.x.s + (size_t) (row0 + min(r, last)) * (a.k >> 5) + sb * 8 + (lane & 1) * 4;
-        __builtin_amdgcn_global_load_lds((pf_gptr) src, (pf_lptr) (buf + kPfSOff + wave * 1024), 16, 0, 0);
+    // super-block sb into the buffer at `buf`
+    __device__ __forceinline__ void copy(uint8_t* buf, int sb) const {
+#pragma unroll
+        for (int n = 0; n < NMT; ++n)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (pf_lptr) (buf + (wave + 4 * n) * 1024), 16, oq[n], sb * 256, 0, 0);
+        if (wave < 2 && 32 * wave < 16 * NMT)   // s: 32 rows an instruction, 32 bytes a row
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (pf_lptr) (buf + kPfSOff + wave * 1024), 16, os, sb * 32, 0, 0);
+        if (wave == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (pf_lptr) (buf + kPfDOff), 4, od, sb * 4, 0, 0);
     }
-    if (wave == 2) {
-        const float* src = a.x.d + (size_t) (row0 + min(lane, last)) * (a.k >> 8) + sb;
-        __builtin_amdgcn_global_load_lds((pf_gptr) src, (pf_lptr) (buf + kPfDOff), 4, 0, 0);
-    }
-}
+};
 
 // the 8 six-bit scales and 8 six-bit minimums of a Q4_K block's 12 bytes, as bytes of two words each
 // (get_scale_min_k4, include/strata/artifact/dequant.hpp:162-172)
@@ -274,15 +283,60 @@ __device__ __forceinline__ long pf_scale_codes(uint64_t w, uint32_t f) {
     return (long) (((uint64_t) __builtin_bit_cast(uint32_t, hi) << 32) | (uint64_t) __builtin_bit_cast(uint32_t, lo));
 }
 
+// LDS reads of the GEMM loop are written out by hand.  The compiler cannot tell which LDS buffer a direct-to-LDS copy
+// fills, so before any LDS read of its own it waits for every copy in flight - here that would be the copy of the
+// super-block two ahead, issued moments earlier.  These reads it does not see; each group is followed by pf_lds_wait
+// on the registers it filled (the values pass through the wait, so nothing that uses them can move above it).
+typedef int pf_i2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pf_lds_addr(const void* p) {
+    return (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) void*) p;
+}
+template <int OFF> __device__ __forceinline__ pf_i2 pf_lds_b64(uint32_t addr) {
+    pf_i2 v;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> __device__ __forceinline__ float pf_lds_f32(uint32_t addr) {
+    float v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> __device__ __forceinline__ v4f pf_lds_f32x4(uint32_t addr) {
+    v4f v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int N, typename T> __device__ __forceinline__ void pf_lds_wait(T (&r)[N]) {
+    if constexpr (N == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]));
+    else if constexpr (N == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]));
+    else if constexpr (N == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]));
+    else if constexpr (N == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]));
+    else if constexpr (N == 6) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]));
+    else {
+        static_assert(N == 8, "1, 2, 3, 4, 6 or 8 registers");
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+    }
+}
+// (compile-time loops over the row groups of a tile)
+template <int M, int NMT, typename F> __device__ __forceinline__ void pf_for_m(F&& f) {
+    if constexpr (M < NMT) {
+        f(std::integral_constant<int, M>{});
+        pf_for_m<M + 1, NMT>(f);
+    }
+}
+
 // one tile of NMT x 16 rows against the wave's two tiles of 16 weight rows (gate/up: the gate and the up rows of 16
 // features)
 template <bool GU, int NMT>
-__device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, int row0, int nrows) {
-    const uint8_t* blob = (const uint8_t*) a.table[ex];
+__device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b1, uint8_t* b2, int ex, int row0, int nrows) {
+    // (global address space: a generic pointer's loads would count as LDS operations too, and every wait for them
+    // would also wait for the copies into LDS behind them)
+    typedef const __attribute__((address_space(1))) uint8_t* wptr;
+    wptr blob = (wptr) a.table[ex];
     const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const uint8_t* wrow[2];
+    wptr wrow[2];
     int64_t n0;   // the wave's first feature (gate/up) or output row (down)
     if constexpr (GU) {
         n0 = (int64_t) blockIdx.x * 64 + wave * 16;
@@ -302,9 +356,13 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
         for (int m = 0; m < NMT; ++m) acc[t][m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
     const int nsb = (int) (a.k >> 8);
-    // the activations run two super-blocks ahead through three LDS buffers, the weights one ahead in registers
-    pf_dma<NMT>(a, lds, row0, nrows, 0, wave, lane);
-    if (nsb > 1) pf_dma<NMT>(a, lds + kPfBufBytes, row0, nrows, 1, wave, lane);
+    // The activations run two super-blocks ahead through three LDS buffers, the weights one ahead in registers.  The
+    // buffers are three separate arrays and the loop below is unrolled over them, so that the compiler can tell a read
+    // of one from a copy into another (it would otherwise wait for every copy in flight before each LDS read).
+    PfDma<NMT> dma;
+    dma.init(a, row0, nrows, wave, lane);
+    dma.copy(b0, 0);
+    if (nsb > 1) dma.copy(b1, 1);
     // the weights of a super-block - the 16-byte header and the lane's four 8-byte slices of the codes of each of its two
     // rows
     uint64_t q[4][2], qn[4][2];     // [slice][row tile]
@@ -312,21 +370,19 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
     auto load_block = [&](int sb, uint64_t (&dq)[4][2], uint32_t (&dh)[2][4]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const uint8_t* blk = wrow[t] + (size_t) sb * 144;
-            const uint4 h = *(const uint4*) blk;
+            wptr blk = wrow[t] + (size_t) sb * 144;
+            typedef uint32_t w4 __attribute__((ext_vector_type(4)));
+            const w4 h = *(const __attribute__((address_space(1))) w4*) blk;
             dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) dq[j][t] = *(const uint64_t*) (blk + 16 + 32 * j + 8 * g);
+            for (int j = 0; j < 4; ++j) dq[j][t] = *(const __attribute__((address_space(1))) uint64_t*) (blk + 16 + 32 * j + 8 * g);
         }
     };
     if (wave_on) load_block(0, q, hdr);
     const int a_base = ln * 256 + 8 * (g & 1), a_swz = (ln ^ (g >> 1)) << 4;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    int cur = 0;   // the buffer of super-block sb
-    for (int sb = 0; sb < nsb; ++sb) {
-        const uint8_t* buf = lds + cur * kPfBufBytes;
-        const int nxt2 = cur == 0 ? 2 : cur - 1;   // the buffer of super-block sb + 2
+    auto step = [&](int sb, const uint8_t* buf, uint8_t* buf2) {   // super-block sb from buf; sb + 2 is copied into buf2
         float d[2], dmin[2];
         uint32_t sc[2][2], mn[2][2];
         if (wave_on) {
@@ -339,21 +395,32 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
             if (sb + 1 < nsb) load_block(sb + 1, qn, hdrn);
         }
         // (after the weights' loads, so that waiting for everything but these copies covers the weights too)
-        if (sb + 2 < nsb) pf_dma<NMT>(a, lds + nxt2 * kPfBufBytes, row0, nrows, sb + 2, wave, lane);
+        if (sb + 2 < nsb) dma.copy(buf2, sb + 2);
         if (wave_on) {
             // the minimums' term, -(dmin m) . s over the 8 sub-blocks, on the matrix cores in F32: A = the tokens' s
             // (row = token, k = sub-block), B = this lane's row's -dmin m, accumulated straight into acc
+            const uint32_t lbuf = pf_lds_addr(buf);
+            {
+                float sa[2 * NMT];
+                const uint32_t at = lbuf + kPfSOff + ln * 32 + g * 4;
+                pf_for_m<0, NMT>([&](auto mc) {
+                    constexpr int m = decltype(mc)::value;
+                    sa[2 * m] = pf_lds_f32<m * 512>(at);
+                    sa[2 * m + 1] = pf_lds_f32<m * 512 + 16>(at);
+                });
+                float nb[2][2];
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                float nb[2];
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) nb[t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
+                    for (int t = 0; t < 2; ++t) nb[half][t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
+                pf_lds_wait(sa);
 #pragma unroll
-                for (int m = 0; m < NMT; ++m) {
-                    const float sa = *(const float*) (buf + kPfSOff + (16 * m + ln) * 32 + (4 * half + g) * 4);
+                for (int half = 0; half < 2; ++half)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa, nb[t], acc[t][m], 0, 0, 0);
-                }
+                    for (int m = 0; m < NMT; ++m)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[2 * m + half], nb[half][t], acc[t][m], 0, 0, 0);
             }
             // The two plane products of the block, int32: [t][m][0] = (q lo) . c, [1] = (q hi) . c.  One 64-deep matrix
             // instruction takes the two sub-blocks of a 32-byte slice of the codes: a lane's first 8 operand bytes are the
@@ -362,6 +429,15 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
             v4i dot[2][NMT][2];
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
+                pf_i2 xr[2 * NMT];
+                {
+                    const uint32_t at0 = lbuf + a_base + (a_swz ^ (64 * p)), at1 = lbuf + a_base + (a_swz ^ (64 * p + 32));
+                    pf_for_m<0, NMT>([&](auto mc) {
+                        constexpr int m = decltype(mc)::value;
+                        xr[2 * m] = pf_lds_b64<m * 4096>(at0);
+                        xr[2 * m + 1] = pf_lds_b64<m * 4096>(at1);
+                    });
+                }
                 v4i wl[2], wh[2];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
@@ -373,11 +449,10 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
                     wl[t] = v4i{(int) l0, (int) (l0 >> 32), (int) l1, (int) (l1 >> 32)};
                     wh[t] = v4i{(int) h0, (int) (h0 >> 32), (int) h1, (int) (h1 >> 32)};
                 }
-                const int at0 = a_base + (a_swz ^ (64 * p)), at1 = a_base + (a_swz ^ (64 * p + 32));
+                pf_lds_wait(xr);
 #pragma unroll
                 for (int m = 0; m < NMT; ++m) {
-                    const int2 x0 = *(const int2*) (buf + at0 + m * 4096), x1 = *(const int2*) (buf + at1 + m * 4096);
-                    const v4i xc = {x0.x, x0.y, x1.x, x1.y};
+                    const v4i xc = {xr[2 * m].x, xr[2 * m].y, xr[2 * m + 1].x, xr[2 * m + 1].y};
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
                         const v4i z = {0, 0, 0, 0};
@@ -387,10 +462,15 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
                 }
             }
             // once a block: lo + 8 hi = the block's integer sum (< 2^25), then its two scales
+            v4f dxr[NMT];
+            pf_for_m<0, NMT>([&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                dxr[m] = pf_lds_f32x4<kPfDOff + m * 64>(lbuf + 16 * g);
+            });
+            pf_lds_wait(dxr);
 #pragma unroll
             for (int m = 0; m < NMT; ++m) {
-                const float4 dx4 = *(const float4*) (buf + kPfDOff + (16 * m + 4 * g) * 4);
-                const float dx[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
+                const float dx[4] = {dxr[m][0], dxr[m][1], dxr[m][2], dxr[m][3]};
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
@@ -407,9 +487,13 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
             }
         }
         // super-block sb + 1 has landed once only this iteration's copies (of sb + 2) may still be in flight
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NMT) : "memory");
-        __syncthreads();
-        cur = cur == 2 ? 0 : cur + 1;
+        // (a bare barrier: __syncthreads() would first wait for every memory operation of the wave, these copies included)
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NMT) : "memory");
+    };
+    for (int sb = 0; sb < nsb; sb += 3) {
+        step(sb, b0, b2);
+        if (sb + 1 < nsb) step(sb + 1, b1, b0);
+        if (sb + 2 < nsb) step(sb + 2, b2, b1);
     }
     if (!wave_on) return;
 
@@ -430,16 +514,16 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* lds, int ex, i
 // grid (bands of weight rows, tiles at most)
 template <bool GU>
 __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t pf_lds[];
+    __shared__ __attribute__((aligned(16))) uint8_t b0[kPfBufBytes], b1[kPfBufBytes], b2[kPfBufBytes];
     const int tile = blockIdx.y;
     if (tile >= *a.plan.n_tiles) return;
     const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
     const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
     switch ((nrows + 15) >> 4) {
-        case 1: pf_tile<GU, 1>(a, pf_lds, ex, row0, nrows); break;
-        case 2: pf_tile<GU, 2>(a, pf_lds, ex, row0, nrows); break;
-        case 3: pf_tile<GU, 3>(a, pf_lds, ex, row0, nrows); break;
-        default: pf_tile<GU, 4>(a, pf_lds, ex, row0, nrows); break;
+        case 1: pf_tile<GU, 1>(a, b0, b1, b2, ex, row0, nrows); break;
+        case 2: pf_tile<GU, 2>(a, b0, b1, b2, ex, row0, nrows); break;
+        case 3: pf_tile<GU, 3>(a, b0, b1, b2, ex, row0, nrows); break;
+        default: pf_tile<GU, 4>(a, b0, b1, b2, ex, row0, nrows); break;
     }
 }
 
@@ -475,16 +559,9 @@ static bool plan_ok(const maya_prefill_plan* p) {
 static bool act_ok(const maya_prefill_act& a) {
     return a.q && a.d && a.s && (((uintptr_t) a.q | (uintptr_t) a.s) & 15) == 0 && ((uintptr_t) a.d & 3) == 0;
 }
-// the GEMM kernels' three LDS buffers are dynamic
 template <bool GU>
 static int pf_launch(const PfGemm& a, dim3 grid, hipStream_t s) {
-    constexpr int lds = kPfLdsBytes;
-    static bool raised[2] = {false, false};
-    if (!raised[GU]) {
-        MAYA_HIP(hipFuncSetAttribute((const void*) prefill_q4k_kernel<GU>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        raised[GU] = true;
-    }
-    hipLaunchKernelGGL(prefill_q4k_kernel<GU>, grid, dim3(256), lds, s, a);
+    hipLaunchKernelGGL(prefill_q4k_kernel<GU>, grid, dim3(256), 0, s, a);
     return MAYA_OK;
 }
 
