@@ -363,16 +363,10 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     dma.init(a, row0, nrows, wave, lane);
     dma.copy(b0, 0);
     if (nsb > 1) dma.copy(b1, 1);
-    // The weights of a super-block - the 16-byte header and the lane's four 8-byte slices of the codes of each of its two
-    // rows - wait in registers.  Tiles of one or two row groups are bound by the weight stream and have registers to
-    // spare: they keep two super-blocks in flight in three register sets that rotate with the LDS buffers; the larger
-    // tiles keep one, in two sets.
-    constexpr bool kDeep = NMT <= 2;
-    struct WSet {
-        uint64_t q[4][2];     // [slice][row tile]
-        uint32_t hdr[2][4];
-    };
-    WSet ws[3];
+    // the weights of a super-block - the 16-byte header and the lane's four 8-byte slices of the codes of each of its two
+    // rows
+    uint64_t q[4][2], qn[4][2];     // [slice][row tile]
+    uint32_t hdr[2][4], hdrn[2][4];
     auto load_block = [&](int sb, uint64_t (&dq)[4][2], uint32_t (&dh)[2][4]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -384,19 +378,13 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
             for (int j = 0; j < 4; ++j) dq[j][t] = *(const __attribute__((address_space(1))) uint64_t*) (blk + 16 + 32 * j + 8 * g);
         }
     };
-    if (wave_on) {
-        load_block(0, ws[0].q, ws[0].hdr);
-        if (kDeep && nsb > 1) load_block(1, ws[1].q, ws[1].hdr);
-    }
+    if (wave_on) load_block(0, q, hdr);
     const int a_base = ln * 256 + 8 * (g & 1), a_swz = (ln ^ (g >> 1)) << 4;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    // super-block sb from buf and the register set wc; sb + 2 is copied into buf2 and (kDeep) loaded into the set wn
-    auto step = [&](int sb, const uint8_t* buf, uint8_t* buf2, WSet& wc, WSet& wn) {
+    auto step = [&](int sb, const uint8_t* buf, uint8_t* buf2) {   // super-block sb from buf; sb + 2 is copied into buf2
         float d[2], dmin[2];
         uint32_t sc[2][2], mn[2][2];
-        uint64_t (&q)[4][2] = wc.q;
-        uint32_t (&hdr)[2][4] = wc.hdr;
         if (wave_on) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
@@ -404,11 +392,7 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
                 dmin[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] >> 16));
                 q4k_unpack_scales(hdr[t][1], hdr[t][2], hdr[t][3], sc[t], mn[t]);
             }
-            if constexpr (kDeep) {
-                if (sb + 2 < nsb) load_block(sb + 2, wn.q, wn.hdr);
-            } else {
-                if (sb + 1 < nsb) load_block(sb + 1, wn.q, wn.hdr);
-            }
+            if (sb + 1 < nsb) load_block(sb + 1, qn, hdrn);
         }
         // (after the weights' loads, so that waiting for everything but these copies covers the weights too)
         if (sb + 2 < nsb) dma.copy(buf2, sb + 2);
@@ -494,31 +478,22 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
                         acc[t][m][i] = fmaf(__fmul_rn(dx[i], d[t]), (float) (dot[t][m][0][i] + 8 * dot[t][m][1][i]), acc[t][m][i]);
                 }
             }
-            if constexpr (!kDeep) {
-                if (sb + 1 < nsb) {
+            if (sb + 1 < nsb) {
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
+                for (int t = 0; t < 2; ++t) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) wc.hdr[t][i] = wn.hdr[t][i], wc.q[i][t] = wn.q[i][t];
-                    }
+                    for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i], q[i][t] = qn[i][t];
                 }
             }
         }
         // super-block sb + 1 has landed once only this iteration's copies (of sb + 2) may still be in flight
         // (a bare barrier: __syncthreads() would first wait for every memory operation of the wave, these copies included)
-        // (and, kDeep, this iteration's 10 weight loads, issued before them)
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NMT + (kDeep ? 10 : 0)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NMT) : "memory");
     };
     for (int sb = 0; sb < nsb; sb += 3) {
-        if constexpr (kDeep) {
-            step(sb, b0, b2, ws[0], ws[2]);
-            if (sb + 1 < nsb) step(sb + 1, b1, b0, ws[1], ws[0]);
-            if (sb + 2 < nsb) step(sb + 2, b2, b1, ws[2], ws[1]);
-        } else {
-            step(sb, b0, b2, ws[0], ws[1]);
-            if (sb + 1 < nsb) step(sb + 1, b1, b0, ws[0], ws[1]);
-            if (sb + 2 < nsb) step(sb + 2, b2, b1, ws[0], ws[1]);
-        }
+        step(sb, b0, b2);
+        if (sb + 1 < nsb) step(sb + 1, b1, b0);
+        if (sb + 2 < nsb) step(sb + 2, b2, b1);
     }
     if (!wave_on) return;
 
