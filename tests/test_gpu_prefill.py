@@ -159,6 +159,27 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
     assert torch.equal(got2, out)
 
 
+def test_chunk_tokens_equal_the_decode_layer(pf):
+    """Two independent GPU paths, one contract: a token's row of the prompt chunk (grouped int8-MFMA GEMMs) is what the
+    decode layer (dot-product mat-vecs) gives for that token alone - the same Q8_K codes and integer sums, F32 sums in
+    another order."""
+    from maya_amd import lib, synth
+    n_embd, n_ff, n_expert, k, n_tokens = 7168, 2048, 6, 3, 40
+    rng = np.random.default_rng(77)
+    blobs = [synth.expert_blob(Q4_K, Q4_K, n_embd, n_ff, rng) for _ in range(n_expert)]
+    store = lib.ExpertStore(blobs)
+    layout, _ = lib.layout(Q4_K, Q4_K, n_embd, n_ff)
+    logits = dev((rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32))
+    x = dev(rng.standard_normal((n_tokens, n_embd)).astype(np.float32))
+    chunk = pf.PrefillLayer(layout, n_expert, k, n_tokens, out_dtype=torch.float32).forward(store.table, logits, x, limit=5.0).clone()
+    dec = lib.MoeLayer(Q4_K, Q4_K, n_embd, n_ff, n_expert, k, max_tokens=8)
+    for t0 in range(0, n_tokens, 8):
+        got = dec.forward(store.table, logits[t0:t0 + 8].contiguous(), x[t0:t0 + 8].contiguous(), limit=5.0)
+        torch.cuda.synchronize()
+        for i in range(got.shape[0]):
+            assert rel_l2(chunk[t0 + i].cpu().numpy(), got[i].cpu().numpy()) <= 1e-4, t0 + i
+
+
 def test_unsupported_and_bad_arguments(pf):
     from maya_amd import lib
     assert pf.load().maya_moe_prefill_supported(Q4_K) == 1 and pf.load().maya_moe_prefill_supported(22) == 0
