@@ -29,8 +29,11 @@
  *   combine .......................... closed form
  *   EXL3 states / codebook ........... the reference's own golden vectors data/exl3-exllamav3 (13 .bin files made by exllamav3)
  *   EXL3 mat-vec ..................... reference build: exl3_ref.cpp bit-exact; H.H = I
- *   prefill grouped product .......... double product of dequantized weights x dequantized int8 activations
- *                                       (tests/hip/prefill_fused_parity.cpp:150-175)
+ *   prompt-chunk rows ................ the pieces above, row by row (the Q8_K quantizer, the Q4_K row dots, SwiGLU, combine):
+ *                                       a chunk's row is the CPU path's expert on that row's token
+ *   mo_grouped_ref / mo_quant_i8x32 .. helpers of the tests (a double product of dequantized weights x dequantized int8 rows,
+ *                                       tests/hip/prefill_fused_parity.cpp:150-175; the per-32 rounding of
+ *                                       src/prefill/moe_fused_rdna4.cu:87-109): an independent float64 numpy product; invariants
  */
 #ifndef MAYA_ORACLE_H
 #define MAYA_ORACLE_H
