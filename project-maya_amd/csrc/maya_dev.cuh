@@ -64,13 +64,15 @@ __device__ __forceinline__ uint32_t neg_bytes(uint32_t g, uint32_t c) {
 // Fmt<TYPE>: kBytes / kValues of a block; kUnit values a lane takes a step; decode(blk, u, cb) fills codes and scales.
 
 struct Unit32 {
-    int q[8];    // 32 int8 codes in value order
+    int q[8];    // 32 int8 codes in value order (the IQ1 types: codes + 9 - delta, see Fmt<kIQ1_S>)
     int s0, s1;  // integer scales of values 0..15 / 16..31
+    int dm[4];   // the IQ1 types: delta - 9 of each group of 8 values
 };
 
 template <int TYPE> struct Fmt;
 
 template <> struct Fmt<kIQ2_S> {
+    static constexpr bool kBiased = false;
     static constexpr int kBytes = 82, kValues = 256, kUnit = 32, kLdsWords = 2048;  // codebook: 1024 x u64
     static constexpr bool kMin = false;
     __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
@@ -118,19 +120,26 @@ __device__ __forceinline__ uint32_t iq1_codes(uint32_t g, uint32_t delta_byte) {
     return lo ^ ((v ^ delta_byte) & 0x80808080u);
 }
 
+// The IQ1 types: a value is d (2 s + 1) (g + delta / 8) with g in {-1, 0, +1} from the grid and delta = +-1 a group (IQ1_M)
+// or a sub-block (IQ1_S), i.e. the int8 code 8 g + delta.  In LDS the grid is kept as t = 8 g + 9 (bytes 1 / 9 / 17:
+// stage_codebook), so a looked-up word IS the operand of the dot products and no per-byte arithmetic is needed:
+//   sum (8 g + delta) y = sum t y + (delta - 9) sum y,
+// the second term from the activations' sums (the Q8_K bsums, and two dot products a group where delta changes inside
+// 16 values).
 template <> struct Fmt<kIQ1_S> {
     static constexpr int kBytes = 50, kValues = 256, kUnit = 32, kLdsWords = 4096;  // codebook: 2048 x u64
-    static constexpr bool kMin = false;
+    static constexpr bool kMin = false, kBiased = true;
     __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
     // third_party/ggml/ggml-common.h:425-430; decode: src/kernels/cuda/iq_kernels.cu:825-837
     __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
         const uint32_t q4 = ld32_a2(blk + 2 + 4 * ib), qh = ld16(blk + 34 + 2 * ib);
-        const uint32_t delta = (qh & 0x8000u) ? 0xffffffffu : 0x01010101u;
+        const int dm = (qh & 0x8000u) ? -10 : -8;
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
             const uint2 g = grid[((q4 >> (8 * l)) & 255u) | (((qh >> (3 * l)) & 7u) << 8)];
-            u.q[2 * l] = (int) iq1_codes(g.x, delta);
-            u.q[2 * l + 1] = (int) iq1_codes(g.y, delta);
+            u.q[2 * l] = (int) g.x;
+            u.q[2 * l + 1] = (int) g.y;
+            u.dm[l] = dm;
         }
         u.s0 = u.s1 = 2 * (int) ((qh >> 12) & 7u) + 1;
     }
@@ -138,7 +147,7 @@ template <> struct Fmt<kIQ1_S> {
 
 template <> struct Fmt<kIQ1_M> {
     static constexpr int kBytes = 56, kValues = 256, kUnit = 32, kLdsWords = 4096;
-    static constexpr bool kMin = false;
+    static constexpr bool kMin = false, kBiased = true;
     // the FP16 super-scale sits in the top nibbles of the four u16 scale words (src/kernels/cpu/iq_avx2.cpp:471-475)
     __device__ static __forceinline__ float scale(const uint8_t* blk) {
         const uint32_t s0 = ld16(blk + 48), s1 = ld16(blk + 50), s2 = ld16(blk + 52), s3 = ld16(blk + 54);
@@ -151,10 +160,10 @@ template <> struct Fmt<kIQ1_M> {
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
             const uint32_t nib = (qh >> (4 * l)) & 15u;
-            const uint32_t delta = (nib & 8u) ? 0xffffffffu : 0x01010101u;
             const uint2 g = grid[((q4 >> (8 * l)) & 255u) | ((nib & 7u) << 8)];
-            u.q[2 * l] = (int) iq1_codes(g.x, delta);
-            u.q[2 * l + 1] = (int) iq1_codes(g.y, delta);
+            u.q[2 * l] = (int) g.x;
+            u.q[2 * l + 1] = (int) g.y;
+            u.dm[l] = (nib & 8u) ? -10 : -8;
         }
         u.s0 = 2 * (int) (sc & 7u) + 1;
         u.s1 = 2 * (int) ((sc >> 3) & 7u) + 1;
@@ -162,6 +171,7 @@ template <> struct Fmt<kIQ1_M> {
 };
 
 template <> struct Fmt<kQ8_0> {
+    static constexpr bool kBiased = false;
     static constexpr int kBytes = 34, kValues = 32, kUnit = 32, kLdsWords = 0;
     static constexpr bool kMin = false;
     __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)); }
@@ -189,6 +199,7 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t* s, int j, int& sc, 
     }
 }
 template <> struct Fmt<kQ4_K> {
+    static constexpr bool kBiased = false;
     static constexpr int kBytes = 144, kValues = 256, kUnit = 64, kLdsWords = 0;
     static constexpr bool kMin = true;
     __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)); }

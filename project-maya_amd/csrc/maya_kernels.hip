@@ -798,6 +798,20 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
                     lo = dot4(u.q[i], y[i], lo);
                     hi = dot4(u.q[4 + i], y[4 + i], hi);
                 }
+                if constexpr (Fmt<TYPE>::kBiased) {
+                    // the table holds codes + 9 - delta: + (delta - 9) x (the activations' sums), 16 values a half
+                    const int bs = a.bs2[t * a.kd + un];
+                    const int s_lo = (int) (short) (bs & 0xffff), s_hi = bs >> 16;
+                    if constexpr (TYPE == kIQ1_S) {   // one delta a sub-block
+                        lo += u.dm[0] * s_lo;
+                        hi += u.dm[0] * s_hi;
+                    } else {                          // one a group of 8: the first group's sum, the second's by difference
+                        const int a0 = dot4(0x01010101, y[0], dot4(0x01010101, y[1], 0));
+                        const int a1 = dot4(0x01010101, y[4], dot4(0x01010101, y[5], 0));
+                        lo += u.dm[0] * a0 + u.dm[1] * (s_lo - a0);
+                        hi += u.dm[2] * a1 + u.dm[3] * (s_hi - a1);
+                    }
+                }
                 acc[t] = fmaf(__fmul_rn(D, a.d[t * a.kd + un]), (float) (u.s0 * lo + u.s1 * hi), acc[t]);
             }
         }
@@ -808,6 +822,23 @@ template <int TYPE> __device__ __forceinline__ const uint64_t* codebook_of(const
     if constexpr (TYPE == kIQ2_S) return cb.iq2s;
     else if constexpr (TYPE == kIQ1_S || TYPE == kIQ1_M) return cb.iq1s;
     else return nullptr;
+}
+
+// a type's codebook into LDS; the IQ1 grid (bytes -1 / 0 / +1) as 8 g + 9 (see Fmt<kIQ1_S>)
+template <int TYPE>
+__device__ __forceinline__ void stage_codebook(int* lds, const Codebooks& cb, int nthreads) {
+    constexpr int n = Fmt<TYPE>::kLdsWords;
+    if constexpr (n > 0) {
+        const uint32_t* src = (const uint32_t*) codebook_of<TYPE>(cb);
+        for (int i = threadIdx.x; i < n; i += nthreads) {
+            uint32_t g = src[i];
+            if constexpr (Fmt<TYPE>::kBiased) {
+                const uint32_t neg = (g >> 1) & 0x01010101u, pos = g & ~(g >> 1) & 0x01010101u;
+                g = 0x09090909u + (pos << 3) - (neg << 3);
+            }
+            lds[i] = (int) g;
+        }
+    }
 }
 
 // stage the codebook (once) and NT activation rows into LDS; rows[t] = the activation row of staged slot t (-1: none)
@@ -882,14 +913,8 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
     // the codebooks of the gate and of the up type (one copy when they share it)
     constexpr int cbg = Fmt<TG>::kLdsWords, cbu = Fmt<TG>::kLdsWords == Fmt<TU>::kLdsWords ? 0 : Fmt<TU>::kLdsWords;
     constexpr int cbw = cbg + cbu;
-    if constexpr (cbg > 0) {
-        const int* src = (const int*) codebook_of<TG>(cb);
-        for (int i = threadIdx.x; i < cbg; i += kGuThreads) lds[i] = src[i];
-    }
-    if constexpr (cbu > 0) {
-        const int* src = (const int*) codebook_of<TU>(cb);
-        for (int i = threadIdx.x; i < cbu; i += kGuThreads) lds[cbg + i] = src[i];
-    }
+    stage_codebook<TG>(lds, cb, kGuThreads);
+    if constexpr (cbu > 0) stage_codebook<TU>(lds + cbg, cb, kGuThreads);
     const uint2* grid_g = (const uint2*) lds;
     const uint2* grid_u = (const uint2*) (lds + (cbu > 0 ? cbg : 0));
     int* lds_act = lds + cbw;
@@ -908,7 +933,7 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
             rows[t] = ents[t] >= 0 ? ents[t] / a.k : -1;
         }
         __syncthreads();
-        stage_act<TG, NT>(lds_act, k, a.x, rows, Fmt<TG>::kMin || Fmt<TU>::kMin);
+        stage_act<TG, NT>(lds_act, k, a.x, rows, Fmt<TG>::kMin || Fmt<TU>::kMin || Fmt<TG>::kBiased || Fmt<TU>::kBiased);
         __syncthreads();
         for (int r = blockIdx.x * wg_rows + wave; r < min(n_ff, (int) (blockIdx.x + 1) * wg_rows); r += kGuThreads / 64) {
             float acc[NT];
@@ -946,10 +971,7 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
     if (!group_of(a, blockIdx.y, gr)) return;
     const int k = a.layout.n_ff, n_embd = a.layout.n_embd;
     constexpr int cbw = Fmt<TD>::kLdsWords;
-    if constexpr (cbw > 0) {
-        const int* src = (const int*) codebook_of<TD>(cb);
-        for (int i = threadIdx.x; i < cbw; i += kDnThreads) lds[i] = src[i];
-    }
+    stage_codebook<TD>(lds, cb, kDnThreads);
     const uint2* grid = (const uint2*) lds;
     int* lds_act = lds + cbw;
     const int kq = k >> 2, kd = k >> 5;
@@ -964,7 +986,7 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
 #pragma unroll
         for (int t = 0; t < NT; ++t) ents[t] = c0 + t < gr.ne ? entry_of(a, gr, c0 + t) : -1;
         __syncthreads();
-        stage_act<TD, NT>(lds_act, k, a.hq, ents, Fmt<TD>::kMin);
+        stage_act<TD, NT>(lds_act, k, a.hq, ents, Fmt<TD>::kMin || Fmt<TD>::kBiased);
         __syncthreads();
         const int r_end = min(n_embd, (int) (blockIdx.x + 1) * wg_rows);
         for (int r = blockIdx.x * wg_rows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
@@ -1022,10 +1044,7 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
     const int k = j.n_in, n_out = j.n_out;
     if ((int) blockIdx.x * wg_rows >= n_out) return;
     constexpr int cbw = Fmt<T>::kLdsWords;
-    if constexpr (cbw > 0) {
-        const int* src = (const int*) codebook_of<T>(cb);
-        for (int i = threadIdx.x; i < cbw; i += kDnThreads) lds[i] = src[i];
-    }
+    stage_codebook<T>(lds, cb, kDnThreads);
     const uint2* grid = (const uint2*) lds;
     int* lds_act = lds + cbw;
     const int kq = k >> 2, kd = k >> 5;
@@ -1039,7 +1058,7 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
 #pragma unroll
         for (int t = 0; t < NT; ++t) cols[t] = c0 + t < j.ncol ? c0 + t : -1;
         __syncthreads();
-        stage_act<T, NT>(lds_act, k, j.x, cols, Fmt<T>::kMin);
+        stage_act<T, NT>(lds_act, k, j.x, cols, Fmt<T>::kMin || Fmt<T>::kBiased);
         __syncthreads();
         const int r_end = min(n_out, (int) (blockIdx.x + 1) * wg_rows);
         for (int r = blockIdx.x * wg_rows + wave * 2 + rsub; r < r_end; r += (kDnThreads / 64) * 2) {
