@@ -143,6 +143,22 @@ template <> struct Fmt<kIQ1_S> {
         }
         u.s0 = u.s1 = 2 * (int) ((qh >> 12) & 7u) + 1;
     }
+    // the same from a quad of the stream order: the sub-blocks' index words, then their qh words, then the block scales
+    __device__ static __forceinline__ void decode_stream(const uint8_t* quad, int nu, int rq, int un, const uint2* grid,
+                                                         Unit32& u, float& d) {
+        const uint32_t q4 = ((const uint32_t*) quad)[un * 4 + rq];
+        const uint32_t qh = ((const uint16_t*) (quad + 16 * (size_t) nu))[un * 4 + rq];
+        d = f16_bits_to_f32(((const uint16_t*) (quad + 24 * (size_t) nu))[(un >> 3) * 4 + rq]) * 0.125f;
+        const int dm = (qh & 0x8000u) ? -10 : -8;
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint2 g = grid[((q4 >> (8 * l)) & 255u) | (((qh >> (3 * l)) & 7u) << 8)];
+            u.q[2 * l] = (int) g.x;
+            u.q[2 * l + 1] = (int) g.y;
+            u.dm[l] = dm;
+        }
+        u.s0 = u.s1 = 2 * (int) ((qh >> 12) & 7u) + 1;
+    }
 };
 
 template <> struct Fmt<kIQ1_M> {

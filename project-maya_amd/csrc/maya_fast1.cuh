@@ -1,0 +1,229 @@
+// maya_fast1.cuh - position-mapped decode kernels for IQ1_S rows in the stream packing: the skeleton of the IQ2_S ones
+// (maya_fast.cuh) with a cheaper unit.  A value is d (2 s + 1) (g + delta / 8), g in {-1, 0, +1} from the 2048-entry
+// grid, delta = +-1 a sub-block (third_party/ggml/ggml-common.h:425-430, src/kernels/cuda/iq_kernels.cu:825-837), i.e.
+// the int8 code 8 g + delta.  The grid sits in LDS as t = 8 g + 9 (bytes 1 / 9 / 17), so a looked-up word is the operand
+// of the dot products as it is, and
+//   sum (8 g + delta) y = sum t y + (delta - 9) SY,   SY = the sum of the lane's 32 activation codes (fixed for the kernel):
+// four lookups, eight dot products and a multiply-add a sub-block, no sign table and no per-byte arithmetic.
+//
+// Stream packing of IQ1_S (rows in quads; nu = k / 32 sub-blocks a row; a quad keeps its 4 x row_bytes = 25 nu bytes):
+//   the 4 index bytes of sub-block u of row r at 4 (4 u + r); its 16-bit qh word at 16 nu + 2 (4 u + r);
+//   block b's FP16 scale at 24 nu + 2 (4 b + r).
+#pragma once
+
+namespace maya {
+
+__device__ __forceinline__ void stage_iq1s_table(int* lds, const Codebooks& cb, int nthreads) {
+    const uint32_t* src = (const uint32_t*) cb.iq1s;
+    for (int i = threadIdx.x; i < 4096; i += nthreads) {
+        const uint32_t g = src[i];
+        const uint32_t neg = (g >> 1) & 0x01010101u, pos = g & ~(g >> 1) & 0x01010101u;
+        lds[i] = (int) (0x09090909u + (pos << 3) - (neg << 3));
+    }
+}
+constexpr int kFast1LdsWords = 4096;
+
+// A lane's share of one quad of rows (4 rows x its sub-block): 8 registers
+struct QuadIQ1S {
+    u32x4 i4;      // the four index bytes of rows 0..3
+    u32x2 qh, d;   // four qh halfwords, four FP16 block scales
+};
+struct QuadOffs1 {
+    uint32_t i4, qh, d;
+};
+template <int NU>
+__device__ __forceinline__ QuadOffs1 quad_offs1(uint32_t mat_off, int u) {
+    return QuadOffs1{mat_off + 16u * u, mat_off + 16u * NU + 8u * u, mat_off + 24u * NU + 8u * (u >> 3)};
+}
+__device__ __forceinline__ QuadIQ1S load_quad1(__amdgpu_buffer_rsrc_t rs, const QuadOffs1& o, uint32_t quad_off) {
+    QuadIQ1S q;
+    q.i4 = __builtin_amdgcn_raw_buffer_load_b128(rs, o.i4, quad_off, 0);
+    q.qh = __builtin_amdgcn_raw_buffer_load_b64(rs, o.qh, quad_off, 0);
+    q.d = __builtin_amdgcn_raw_buffer_load_b64(rs, o.d, quad_off, 0);
+    return q;
+}
+// row R of the quad against the lane's activation codes: sy9 = -9 SY and sy = SY are fixed for the lane
+template <int R>
+__device__ __forceinline__ float unit1_value(const QuadIQ1S& q, const uint2* grid, const int (&y)[8], int sy, float dy8) {
+    const uint32_t i4 = q.i4[R];
+    const uint32_t hw = R < 2 ? q.qh.x : q.qh.y, dw = R < 2 ? q.d.x : q.d.y;
+    const uint32_t qh = (R & 1) ? (hw >> 16) : (hw & 0xffffu), d = (R & 1) ? (dw >> 16) : (dw & 0xffffu);
+    int t = 0;
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        const uint2 g = grid[((i4 >> (8 * l)) & 255u) | (((qh >> (3 * l)) & 7u) << 8)];
+        t = dot4((int) g.x, y[2 * l], t);
+        t = dot4((int) g.y, y[2 * l + 1], t);
+    }
+    t += ((qh & 0x8000u) ? -10 : -8) * sy;
+    const int isum = __mul24(2 * (int) ((qh >> 12) & 7u) + 1, t);
+    return __fmul_rn(__fmul_rn(f16_bits_to_f32(d), dy8), (float) isum);
+}
+template <int B>
+__device__ __forceinline__ void quad1_values(const QuadIQ1S& q, const uint2* grid, const int (&y)[8], int sy, float dy8, float (&acc)[8]) {
+#define MAYA_ROW(R)                                              \
+    acc[B + R] = unit1_value<R>(q, grid, y, sy, dy8);            \
+    asm volatile("" : "+v"(acc[B + R]));                         \
+    __builtin_amdgcn_sched_barrier(0);
+    MAYA_ROW(0) MAYA_ROW(1) MAYA_ROW(2) MAYA_ROW(3)
+#undef MAYA_ROW
+}
+__device__ __forceinline__ int sum32_codes(const int (&y)[8]) {
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s = dot4(0x01010101, y[i], s);
+    return s;
+}
+
+// ---- gate/up, n_embd = 1024 NW: a workgroup of NW waves = the 2 * 32 NW sub-block positions of a (gate row, up row) pair;
+// grid (n_ff / ROWS, entries); entry e = token e / k, slot e % k.  Rows in batches of 8 (two quads), a quad ahead.
+template <int NW, int ROWS, int MINW>
+__global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
+    static_assert(ROWS % 8 == 0, "a batch is two quads");
+    constexpr int NU = 32 * NW;
+    __shared__ int lds[kFast1LdsWords];
+    __shared__ float part[2][2 * NW][8];
+    if (a.skip && *a.skip) return;
+    const int e = blockIdx.y;
+    const uint64_t blob = a.plan_ptr[e];
+    if (blob == 0ull) return;
+    stage_iq1s_table(lds, cb, 64 * NW);
+    const uint2* grid = (const uint2*) lds;
+    const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
+    const bool is_up = t >= NU;
+    const int u = is_up ? t - NU : t;
+    const int tok = e / a.k;
+    int y[8];
+    {
+        const int4* q = (const int4*) (a.x.q + (size_t) tok * (32 * NU));
+        const int4 ya = q[2 * u], yb = q[2 * u + 1];
+        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+    }
+    const int sy = sum32_codes(y);
+    const float dy8 = a.x.d[(size_t) tok * NU + u] * 0.125f;
+    constexpr uint32_t qb = NU / 8 * 50 * 4;  // bytes of a quad of rows
+    const int n_ff = a.layout.n_ff, r0 = blockIdx.x * ROWS;
+    const __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob + a.layout.gate_off, (uint32_t) (a.layout.down_off - a.layout.gate_off));
+    const QuadOffs1 qo = quad_offs1<NU>(is_up ? (uint32_t) (a.layout.up_off - a.layout.gate_off) : 0u, u);
+    const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+    constexpr int NQ = ROWS / 4;
+    QuadIQ1S nxt = load_quad1(rs, qo, quad0);
+    __syncthreads();
+    float acc[8];
+#pragma unroll 1
+    for (int r = 0; r < ROWS; r += 8) {
+        const int q = r >> 2;
+        {
+            const QuadIQ1S cur = nxt;
+            nxt = load_quad1(rs, qo, quad0 + (uint32_t) (q + 1) * qb);
+            quad1_values<0>(cur, grid, y, sy, dy8, acc);
+        }
+        {
+            const QuadIQ1S cur = nxt;
+            if (q + 2 < NQ) nxt = load_quad1(rs, qo, quad0 + (uint32_t) (q + 2) * qb);
+            quad1_values<4>(cur, grid, y, sy, dy8, acc);
+        }
+        const float v = reduce8_half(acc, lane);
+        const int buf = (r >> 3) & 1;
+        if ((lane & 3) == 0) part[buf][hw][(lane >> 2) & 7] = v;
+        __syncthreads();
+        if (t < 8) {
+            float g = part[buf][0][t], up = part[buf][NW][t];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                g += part[buf][w][t];
+                up += part[buf][NW + w][t];
+            }
+            if (r0 + r + t < n_ff) a.h[(size_t) e * n_ff + r0 + r + t] = swiglu(g, up, a.limit);
+        }
+    }
+}
+
+// ---- down + combine, n_ff = 2048 (64 sub-blocks a row = one wave): wave w = slot w of token blockIdx.y, rows in batches
+// of 8; grid (n_embd / ROWS, tokens).  Without a rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.  The
+// slots' rows meet in LDS and are summed in slot order.
+template <int ROWS, int MINW>
+__global__ __launch_bounds__(512, MINW) void down_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
+    static_assert(ROWS % 8 == 0, "a batch is two quads");
+    constexpr int NU = 64;
+    __shared__ int lds[kFast1LdsWords];
+    __shared__ float part[8][ROWS];
+    if (a.skip && *a.skip) return;
+    stage_iq1s_table(lds, cb, 512);
+    const uint2* grid = (const uint2*) lds;
+    const int n_embd = a.layout.n_embd;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r0 = blockIdx.x * ROWS;
+    const int e0 = blockIdx.y * a.k, ent = e0 + wave;
+    const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
+    __syncthreads();
+    if (blob != 0ull) {
+        constexpr uint32_t qb = NU / 8 * 50 * 4;
+        const uint64_t mat = blob + a.layout.down_off;
+        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
+        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
+        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
+        const QuadOffs1 qo = quad_offs1<NU>(0u, lane);
+        const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+        constexpr int NQ = ROWS / 4;
+        QuadIQ1S nxt = load_quad1(rs, qo, quad0);
+        int y[8];
+        float dy8;
+        if (a.hq.q) {
+            const int4* q = (const int4*) (a.hq.q + (size_t) ent * 2048);
+            const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+            y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+            dy8 = a.hq.d[(size_t) ent * 64 + lane] * 0.125f;
+        } else {
+            const float4* hv = (const float4*) (a.h + (size_t) ent * 2048 + 32 * lane);
+            float v[32];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float4 t = hv[i];
+                v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+            }
+            float d;
+            q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
+            dy8 = d * 0.125f;
+        }
+        const int sy = sum32_codes(y);
+        float acc[8];
+#pragma unroll 1
+        for (int r = 0; r < ROWS; r += 8) {
+            const int q = r >> 2;
+            {
+                const QuadIQ1S cur = nxt;
+                nxt = load_quad1(rs, qo, quad0 + (uint32_t) (q + 1) * qb);
+                quad1_values<0>(cur, grid, y, sy, dy8, acc);
+            }
+            {
+                const QuadIQ1S cur = nxt;
+                if (q + 2 < NQ) nxt = load_quad1(rs, qo, quad0 + (uint32_t) (q + 2) * qb);
+                quad1_values<4>(cur, grid, y, sy, dy8, acc);
+            }
+            float v = reduce8_half(acc, lane);
+            v += __shfl_xor(v, 32, kWave);
+            if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < ROWS) {
+        const int c = threadIdx.x;
+        float sum = 0.0f;
+        bool first = true;
+        for (int i = 0; i < a.k; ++i) {
+            if (a.plan_ptr[e0 + i] == 0ull) continue;
+            const float p = __fmul_rn(part[i][c], a.plan_w[e0 + i]);
+            sum = first ? p : __fadd_rn(sum, p);
+            first = false;
+        }
+        const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
+        if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
+        a.out[o] = sum;
+        if (a.part)
+            for (int i = 0; i < a.k; ++i)
+                if (a.plan_ptr[e0 + i] != 0ull) a.part[(size_t) (e0 + i) * n_embd + r0 + c] = part[i][c];
+    }
+}
+
+}  // namespace maya

@@ -138,11 +138,22 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         const float mag = __fmul_rn(dl, (float) (uint32_t) ((g >> (8 * j)) & 255u));
         r = (sg >> j) & 1 ? -mag : mag;
     } else if constexpr (TYPE == kIQ1_S) {
-        const uint8_t* blk = rp + (size_t) (v >> 8) * 50;
         const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
-        const uint32_t qh = ld16(blk + 34 + 2 * ib);
-        const uint64_t g = cb.iq1s[blk[2 + 4 * ib + il] | (((qh >> (3 * il)) & 7u) << 8)];
-        const float dl = __fmul_rn(f16_bits_to_f32(ld16(blk)), (float) (2 * (int) ((qh >> 12) & 7u) + 1));
+        uint32_t qs, qh, dbits;
+        if (packing == MAYA_PACK_STREAM) {
+            const int64_t nu = k >> 5, un = v >> 5, rq = row & 3;
+            const uint8_t* quad = w + (size_t) (row >> 2) * 4 * row_stride;
+            qs = quad[4 * (un * 4 + rq) + il];
+            qh = ld16(quad + 16 * nu + 2 * (un * 4 + rq));
+            dbits = ld16(quad + 24 * nu + 2 * ((un >> 3) * 4 + rq));
+        } else {
+            const uint8_t* blk = rp + (size_t) (v >> 8) * 50;
+            qs = blk[2 + 4 * ib + il];
+            qh = ld16(blk + 34 + 2 * ib);
+            dbits = ld16(blk);
+        }
+        const uint64_t g = cb.iq1s[qs | (((qh >> (3 * il)) & 7u) << 8)];
+        const float dl = __fmul_rn(f16_bits_to_f32(dbits), (float) (2 * (int) ((qh >> 12) & 7u) + 1));
         const float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
         r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
     } else {  // IQ1_M
@@ -195,6 +206,32 @@ __global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restr
             gd[0] = qs[o_d];
             gd[1] = qs[o_d + 1];
         }
+    }
+}
+
+// IQ1_S rows between the GGUF block sequence and the stream order (rows in quads: the sub-blocks' index words, then their
+// qh words, then the block scales); one thread a sub-block, grid (k/32 sub-blocks / 256, rows).  DIR as above.
+template <int DIR>
+__global__ __launch_bounds__(256) void repack_iq1s_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                          int64_t k, int64_t n_rows) {
+    const int64_t nu = k >> 5, rb = (k >> 8) * 50;
+    const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (un >= nu) return;
+    const int64_t b = un >> 3, rq = row & 3;
+    const int ib = (int) (un & 7);
+    const uint8_t* g = (DIR == 0 ? src : dst) + row * rb + b * 50;          // the GGUF block
+    const uint8_t* q = (DIR == 0 ? dst : src) + (row >> 2) * 4 * rb;        // the quad
+    const int64_t o_i = 4 * (un * 4 + rq), o_h = 16 * nu + 2 * (un * 4 + rq), o_d = 24 * nu + 2 * (b * 4 + rq);
+    uint8_t* gw = (uint8_t*) g;
+    uint8_t* qw = (uint8_t*) q;
+    if (DIR == 0) {
+        for (int i = 0; i < 4; ++i) qw[o_i + i] = g[2 + 4 * ib + i];
+        qw[o_h] = g[34 + 2 * ib], qw[o_h + 1] = g[35 + 2 * ib];
+        if (ib == 0) qw[o_d] = g[0], qw[o_d + 1] = g[1];
+    } else {
+        for (int i = 0; i < 4; ++i) gw[2 + 4 * ib + i] = q[o_i + i];
+        gw[34 + 2 * ib] = q[o_h], gw[35 + 2 * ib] = q[o_h + 1];
+        if (ib == 0) gw[0] = q[o_d], gw[1] = q[o_d + 1];
     }
 }
 
@@ -726,6 +763,9 @@ __global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__
 
 // ------------------------------------------------------------------------------------------------ expert rows
 
+// the types whose stream packing groups rows in quads
+__host__ __device__ constexpr bool quad_packed(int t) { return t == kIQ2_S || t == kIQ1_S; }
+
 // LDS view of up to NT staged activation rows of k values
 struct ActLds {
     const int* q;          // [NT][k/4]
@@ -777,8 +817,8 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
             }
             Unit32 u;
             float D;
-            if (TYPE == kIQ2_S && stream_packed) {
-                if constexpr (TYPE == kIQ2_S) Fmt<kIQ2_S>::decode_stream(row, nu, rq, un, grid, u, D);
+            if ((TYPE == kIQ2_S || TYPE == kIQ1_S) && stream_packed) {
+                if constexpr (TYPE == kIQ2_S || TYPE == kIQ1_S) Fmt<TYPE>::decode_stream(row, nu, rq, un, grid, u, D);
             } else if (TYPE == kQ8_0 && stream_packed) {   // the row's codes, then its scales
                 const int* c = (const int*) (row + 32 * (size_t) un);
 #pragma unroll
@@ -942,8 +982,8 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
             // (stream packing: the row's quad and its place in it; the GGUF packing: the row itself)
             // (only IQ2_S rows have a stream order; the other types' rows stay where GGUF puts them)
             // (IQ2_S rows are packed in quads, Q8_0 rows one by one)
-            const bool qg = packed && TG == kIQ2_S, qu = packed && TU == kIQ2_S;
-            const bool pg = packed && (TG == kIQ2_S || TG == kQ8_0), pu = packed && (TU == kIQ2_S || TU == kQ8_0);
+            const bool qg = packed && quad_packed(TG), qu = packed && quad_packed(TU);
+            const bool pg = packed && (quad_packed(TG) || TG == kQ8_0), pu = packed && (quad_packed(TU) || TU == kQ8_0);
             const int rq = r & 3;
             if constexpr (TG == TU) {
                 const uint8_t* row = blob + (is_up ? a.layout.up_off : a.layout.gate_off) + (size_t) (qg ? (r & ~3) : r) * grow;
@@ -979,8 +1019,8 @@ __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codeb
     const uint8_t* base = (const uint8_t*) gr.blob + a.layout.down_off;
     const size_t drow = (size_t) (k / Fmt<TD>::kValues) * Fmt<TD>::kBytes;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
-    const bool quads = a.layout.packing == MAYA_PACK_STREAM && TD == kIQ2_S;
-    const bool packed = a.layout.packing == MAYA_PACK_STREAM && (TD == kIQ2_S || TD == kQ8_0);
+    const bool quads = a.layout.packing == MAYA_PACK_STREAM && quad_packed(TD);
+    const bool packed = a.layout.packing == MAYA_PACK_STREAM && (quad_packed(TD) || TD == kQ8_0);
     for (int c0 = 0; c0 < gr.ne; c0 += NT) {
         int ents[NT];
 #pragma unroll
@@ -1051,8 +1091,8 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
     ActLds al{lds_act, (const float*) (lds_act + NT * kq), lds_act + NT * kq + NT * kd, kq, kd};
     const size_t drow = (size_t) (k / Fmt<T>::kValues) * Fmt<T>::kBytes;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 31, rsub = lane >> 5;
-    const bool quads = j.packing == MAYA_PACK_STREAM && T == kIQ2_S;
-    const bool packed = j.packing == MAYA_PACK_STREAM && (T == kIQ2_S || T == kQ8_0);
+    const bool quads = j.packing == MAYA_PACK_STREAM && quad_packed(T);
+    const bool packed = j.packing == MAYA_PACK_STREAM && (quad_packed(T) || T == kQ8_0);
     for (int c0 = 0; c0 < j.ncol; c0 += NT) {
         int cols[NT];
 #pragma unroll
@@ -1082,6 +1122,7 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
 }  // namespace maya
 
 #include "maya_fast.cuh"
+#include "maya_fast1.cuh"
 #include "maya_fastk.cuh"
 #include "maya_fastq.cuh"
 
@@ -1226,9 +1267,41 @@ bool gate_up_fuses_hq(const maya_moe_args& a) {
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
 }
+// ---- IQ1_S in the stream packing: the position-mapped kernels
+bool gate_up_iq1s_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (!(l.gate_type == kIQ1_S && l.up_type == kIQ1_S && l.packing == MAYA_PACK_STREAM)) return false;
+    if (l.n_embd % 1024 != 0 || l.n_ff % 16 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
+    const int nw = l.n_embd / 1024;
+    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+}
+bool down_iq1s_pos_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    return l.down_type == kIQ1_S && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 &&
+           (l.down_off & 15) == 0;
+}
+int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    const dim3 grid((unsigned) (a.layout.n_ff / 16), (unsigned) (a.n_tokens * a.k));
+    switch (a.layout.n_embd / 1024) {
+        case 4: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
+        case 6: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
+        case 7: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<7, 16, 8>), grid, dim3(448), 0, s, a, st.cb); break;
+        default: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<8, 16, 8>), grid, dim3(512), 0, s, a, st.cb); break;
+    }
+    MAYA_LAUNCHED("gate_up_iq1s_pos_kernel");
+    return MAYA_OK;
+}
+int launch_down_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    const dim3 grid((unsigned) (a.layout.n_embd / 16), (unsigned) a.n_tokens);
+    hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
+    MAYA_LAUNCHED("down_iq1s_pos_kernel");
+    return MAYA_OK;
+}
+
 // whether try_down_iq2s_1tok would take the position-mapped kernel, which can round h to Q8_K itself (hq.q == NULL)
 bool down_rounds_h(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
+    if (down_iq1s_pos_ok(a)) return true;
     if (l.down_type == kQ4_K) return l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
     return l.down_type == kIQ2_S && a.k <= 8 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 && l.n_embd % 16 == 0;
 }
@@ -1343,7 +1416,7 @@ int launch_down_q80_pos(const maya_moe_args& a, hipStream_t s) {
 // whether the gate/up (down) call is served entry by entry (no use for the groups of a window)
 bool gate_up_by_entries(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    if (gate_up_q4k_pos_ok(a)) return true;
+    if (gate_up_q4k_pos_ok(a) || gate_up_iq1s_pos_ok(a)) return true;
     if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM) || l.n_ff % 16 != 0 || l.n_embd % 1024 != 0) return false;
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
@@ -1433,6 +1506,10 @@ static int repack_impl(const maya_moe_layout* l, const void* src, void* dst, voi
             const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
             if (dir == 0) hipLaunchKernelGGL(repack_iq2s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
             else hipLaunchKernelGGL(repack_iq2s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+        } else if (r.type == kIQ1_S) {
+            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
+            if (dir == 0) hipLaunchKernelGGL(repack_iq1s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+            else hipLaunchKernelGGL(repack_iq1s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
         } else if (r.type == kQ8_0) {
             const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
             if (dir == 0) hipLaunchKernelGGL(repack_q80_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
@@ -1570,6 +1647,7 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
         if (try_gate_up_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
     if (gate_up_q4k_pos_ok(*a)) return launch_gate_up_q4k_pos(*a, s);
+    if (gate_up_iq1s_pos_ok(*a)) return launch_gate_up_iq1s_pos(*a, *st, s);
     if (gate_up_q80_pos_ok(*a)) return launch_gate_up_q80_pos(*a, s);
 #define MAYA_GU(TG, TU) if (tg == TG && tu == TU) return launch_gate_up_t<TG, TU>(*a, *st, s);
     MAYA_GU(kIQ2_S, kIQ2_S)
@@ -1596,6 +1674,7 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     if (!a->hq.q && !a->hq.d && !a->hq.bsums && a->h && a->out && down_rounds_h(*a)) {
         int rc = 0;   // the kernel rounds h itself
         if (a->layout.down_type == kQ4_K) return launch_down_q4k_pos(*a, as_stream(stream));
+        if (a->layout.down_type == kIQ1_S) return launch_down_iq1s_pos(*a, *st, as_stream(stream));
         if (try_down_iq2s_1tok(*a, *st, as_stream(stream), &rc)) return rc;
     }
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
@@ -1605,6 +1684,7 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
         if (try_down_iq2s_1tok(*a, *st, s, &rc)) return rc;
     }
     if (down_q4k_pos_ok(*a)) return launch_down_q4k_pos(*a, s);
+    if (down_iq1s_pos_ok(*a)) return launch_down_iq1s_pos(*a, *st, s);
     if (down_q80_pos_ok(*a)) {
         if (const int rc = launch_down_q80_pos(*a, s)) return rc;
         const dim3 cgrid((unsigned) ((a->layout.n_embd + 255) / 256), (unsigned) a->n_tokens);
@@ -1640,8 +1720,8 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
         if (j.n_in < 256 || j.n_in % 256 || j.n_in > 16384 || j.n_out < 1)
             return fail(MAYA_E_SHAPE, "mv: job %d: n_in %d (a multiple of 256 up to 16384) / n_out %d", i, j.n_in, j.n_out);
         if (j.ncol < 1 || j.ncol > MAYA_MAX_TOKENS) return fail(MAYA_E_SHAPE, "mv: job %d: ncol %d outside 1..%d", i, j.ncol, MAYA_MAX_TOKENS);
-        if (j.packing == MAYA_PACK_STREAM && j.type == kIQ2_S && j.n_out % 4)
-            return fail(MAYA_E_SHAPE, "mv: job %d: stream-packed IQ2_S rows come in quads, n_out %d", i, j.n_out);
+        if (j.packing == MAYA_PACK_STREAM && quad_packed(j.type) && j.n_out % 4)
+            return fail(MAYA_E_SHAPE, "mv: job %d: stream-packed IQ2_S / IQ1_S rows come in quads, n_out %d", i, j.n_out);
         if (j.packing == MAYA_PACK_STREAM && ((uintptr_t) j.w & 15)) return fail(MAYA_E_ARG, "mv: job %d: stream-packed weights must be 16-byte aligned", i);
         if (!j.w || !j.x.q || !j.x.d || (q8k_act(j.type) && !j.x.bsums) || !j.y) return fail(MAYA_E_ARG, "mv: job %d: null pointer", i);
         if (j.y_stride < j.n_out && j.ncol > 1) return fail(MAYA_E_ARG, "mv: job %d: y_stride %lld below n_out %d", i, (long long) j.y_stride, j.n_out);

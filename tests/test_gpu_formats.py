@@ -103,7 +103,7 @@ def test_i8x32_quant_byte_exact(lib, oracle):
         assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
 
 
-@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8)))
+@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8), (19, 19), (19, 22)))
 def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
     """maya_moe_repack regroups bytes only: unpack(repack(blob)) == blob, and the packed rows dequantize to the same bits."""
     n_embd, n_ff = 1024, 512
@@ -129,6 +129,16 @@ def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
             g = src[off:off + rb * rows].view(rows, k // 32, 34).cpu().numpy()
             p = packed[off:off + rb * rows].view(rows, rb).cpu().numpy()
             assert np.array_equal(p[:, :k], g[:, :, 2:].reshape(rows, k)) and np.array_equal(p[:, k:], g[:, :, :2].reshape(rows, -1))
+        elif t == 19:
+            # IQ1_S: per quad the sub-blocks' index words [u][row], then their qh words, then the block scales [block][row]
+            nu = k // 32
+            g = src[off:off + rb * rows].view(rows // 4, 4, nu // 8, 50).cpu().numpy()
+            p = packed[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
+            want_i = g[:, :, :, 2:34].reshape(rows // 4, 4, nu, 4).transpose(0, 2, 1, 3).reshape(rows // 4, -1)
+            want_h = g[:, :, :, 34:50].reshape(rows // 4, 4, nu, 2).transpose(0, 2, 1, 3).reshape(rows // 4, -1)
+            want_d = g[:, :, :, 0:2].transpose(0, 2, 1, 3).reshape(rows // 4, -1)
+            assert np.array_equal(p[:, :16 * nu], want_i) and np.array_equal(p[:, 16 * nu:24 * nu], want_h)
+            assert np.array_equal(p[:, 24 * nu:], want_d)
         elif t != 22:
             assert np.array_equal(a, b)
         want = oracle.dequant_rows(t, blob[off:off + rb * 16], k, 16)
