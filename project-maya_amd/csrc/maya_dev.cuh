@@ -184,6 +184,26 @@ template <> struct Fmt<kIQ1_M> {
         u.s0 = 2 * (int) (sc & 7u) + 1;
         u.s1 = 2 * (int) ((sc >> 3) & 7u) + 1;
     }
+    // the same from a quad of the stream order: index words, qh words, then 8 bytes a (block, row): the block scale, then
+    // the sixteen 3-bit scales in order
+    __device__ static __forceinline__ void decode_stream(const uint8_t* quad, int nu, int rq, int un, const uint2* grid,
+                                                         Unit32& u, float& d) {
+        const uint32_t q4 = ((const uint32_t*) quad)[un * 4 + rq];
+        const uint32_t qh = ((const uint16_t*) (quad + 16 * (size_t) nu))[un * 4 + rq];
+        const uint2 rec = ((const uint2*) (quad + 24 * (size_t) nu))[(un >> 3) * 4 + rq];
+        d = f16_bits_to_f32(rec.x & 0xffffu) * 0.125f;
+        const uint32_t sc = (uint32_t) ((((uint64_t) rec.y << 32) | (uint64_t) rec.x) >> (16 + 6 * (un & 7)));
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint32_t nib = (qh >> (4 * l)) & 15u;
+            const uint2 g = grid[((q4 >> (8 * l)) & 255u) | ((nib & 7u) << 8)];
+            u.q[2 * l] = (int) g.x;
+            u.q[2 * l + 1] = (int) g.y;
+            u.dm[l] = (nib & 8u) ? -10 : -8;
+        }
+        u.s0 = 2 * (int) (sc & 7u) + 1;
+        u.s1 = 2 * (int) ((sc >> 3) & 7u) + 1;
+    }
 };
 
 template <> struct Fmt<kQ8_0> {

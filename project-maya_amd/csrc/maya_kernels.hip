@@ -157,13 +157,29 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         const float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
         r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
     } else {  // IQ1_M
-        const uint8_t* blk = rp + (size_t) (v >> 8) * 56;
         const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
-        const uint32_t nib = (blk[32 + 2 * ib + (il >> 1)] >> (4 * (il & 1))) & 15u;
         const int ib16 = 2 * ib + (il >> 1);
-        const int s = (ld16(blk + 48 + 2 * (ib16 >> 2)) >> (3 * (ib16 & 3))) & 7;
-        const uint64_t g = cb.iq1s[blk[4 * ib + il] | ((nib & 7u) << 8)];
-        const float d = Fmt<kIQ1_M>::scale(blk) * 8.0f;  // scale() carries the 1/8 of the integer-code form
+        uint32_t qs, nib;
+        int s;
+        float d;
+        if (packing == MAYA_PACK_STREAM) {
+            const int64_t nu = k >> 5, un = v >> 5, rq = row & 3;
+            const uint8_t* quad = w + (size_t) (row >> 2) * 4 * row_stride;
+            qs = quad[4 * (un * 4 + rq) + il];
+            nib = (quad[16 * nu + 2 * (un * 4 + rq) + (il >> 1)] >> (4 * (il & 1))) & 15u;
+            const uint8_t* rec = quad + 24 * nu + 8 * ((un >> 3) * 4 + rq);
+            uint64_t r8 = 0;
+            for (int b = 0; b < 8; ++b) r8 |= (uint64_t) rec[b] << (8 * b);
+            s = (int) ((r8 >> (16 + 3 * ib16)) & 7u);
+            d = f16_bits_to_f32((uint32_t) (r8 & 0xffffu));
+        } else {
+            const uint8_t* blk = rp + (size_t) (v >> 8) * 56;
+            qs = blk[4 * ib + il];
+            nib = (blk[32 + 2 * ib + (il >> 1)] >> (4 * (il & 1))) & 15u;
+            s = (ld16(blk + 48 + 2 * (ib16 >> 2)) >> (3 * (ib16 & 3))) & 7;
+            d = Fmt<kIQ1_M>::scale(blk) * 8.0f;  // scale() carries the 1/8 of the integer-code form
+        }
+        const uint64_t g = cb.iq1s[qs | ((nib & 7u) << 8)];
         const float dl = __fmul_rn(d, (float) (2 * s + 1));
         const float delta = (nib & 8u) ? -0.125f : 0.125f;
         r = __fmul_rn(dl, __fadd_rn((float) (int8_t) ((g >> (8 * j)) & 255u), delta));
@@ -232,6 +248,46 @@ __global__ __launch_bounds__(256) void repack_iq1s_kernel(const uint8_t* __restr
         for (int i = 0; i < 4; ++i) gw[2 + 4 * ib + i] = q[o_i + i];
         gw[34 + 2 * ib] = q[o_h], gw[35 + 2 * ib] = q[o_h + 1];
         if (ib == 0) gw[0] = q[o_d], gw[1] = q[o_d + 1];
+    }
+}
+
+// IQ1_M rows likewise (quads: index words, qh words, then 8 bytes a (block, row): the block scale gathered from the top
+// nibbles of the four scale words, and their 4 x 12 bits of 3-bit scales in order); one thread a sub-block.
+template <int DIR>
+__global__ __launch_bounds__(256) void repack_iq1m_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                          int64_t k, int64_t n_rows) {
+    const int64_t nu = k >> 5, rb = (k >> 8) * 56;
+    const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (un >= nu) return;
+    const int64_t b = un >> 3, rq = row & 3;
+    const int ib = (int) (un & 7);
+    const uint8_t* g = (DIR == 0 ? src : dst) + row * rb + b * 56;          // the GGUF block
+    const uint8_t* q = (DIR == 0 ? dst : src) + (row >> 2) * 4 * rb;        // the quad
+    const int64_t o_i = 4 * (un * 4 + rq), o_h = 16 * nu + 2 * (un * 4 + rq), o_s = 24 * nu + 8 * (b * 4 + rq);
+    uint8_t* gw = (uint8_t*) g;
+    uint8_t* qw = (uint8_t*) q;
+    if (DIR == 0) {
+        for (int i = 0; i < 4; ++i) qw[o_i + i] = g[4 * ib + i];
+        qw[o_h] = g[32 + 2 * ib], qw[o_h + 1] = g[33 + 2 * ib];
+        if (ib == 0) {
+            uint64_t w[4];
+            for (int i = 0; i < 4; ++i) w[i] = (uint64_t) ld16(g + 48 + 2 * i);
+            const uint64_t d = (w[0] >> 12) | ((w[1] >> 8) & 0xf0u) | ((w[2] >> 4) & 0xf00u) | (w[3] & 0xf000u);
+            const uint64_t rec = d | ((w[0] & 0xfffu) << 16) | ((w[1] & 0xfffu) << 28) | ((w[2] & 0xfffu) << 40) | ((w[3] & 0xfffu) << 52);
+            for (int i = 0; i < 8; ++i) qw[o_s + i] = (uint8_t) (rec >> (8 * i));
+        }
+    } else {
+        for (int i = 0; i < 4; ++i) gw[4 * ib + i] = q[o_i + i];
+        gw[32 + 2 * ib] = q[o_h], gw[33 + 2 * ib] = q[o_h + 1];
+        if (ib == 0) {
+            uint64_t rec = 0;
+            for (int i = 0; i < 8; ++i) rec |= (uint64_t) q[o_s + i] << (8 * i);
+            const uint32_t d = (uint32_t) (rec & 0xffffu);
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = (uint32_t) ((rec >> (16 + 12 * i)) & 0xfffu) | (((d >> (4 * i)) & 0xfu) << 12);
+                gw[48 + 2 * i] = (uint8_t) w, gw[49 + 2 * i] = (uint8_t) (w >> 8);
+            }
+        }
     }
 }
 
@@ -764,7 +820,7 @@ __global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__
 // ------------------------------------------------------------------------------------------------ expert rows
 
 // the types whose stream packing groups rows in quads
-__host__ __device__ constexpr bool quad_packed(int t) { return t == kIQ2_S || t == kIQ1_S; }
+__host__ __device__ constexpr bool quad_packed(int t) { return t == kIQ2_S || t == kIQ1_S || t == kIQ1_M; }
 
 // LDS view of up to NT staged activation rows of k values
 struct ActLds {
@@ -817,8 +873,8 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
             }
             Unit32 u;
             float D;
-            if ((TYPE == kIQ2_S || TYPE == kIQ1_S) && stream_packed) {
-                if constexpr (TYPE == kIQ2_S || TYPE == kIQ1_S) Fmt<TYPE>::decode_stream(row, nu, rq, un, grid, u, D);
+            if (quad_packed(TYPE) && stream_packed) {
+                if constexpr (quad_packed(TYPE)) Fmt<TYPE>::decode_stream(row, nu, rq, un, grid, u, D);
             } else if (TYPE == kQ8_0 && stream_packed) {   // the row's codes, then its scales
                 const int* c = (const int*) (row + 32 * (size_t) un);
 #pragma unroll
@@ -1267,21 +1323,31 @@ bool gate_up_fuses_hq(const maya_moe_args& a) {
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
 }
-// ---- IQ1_S in the stream packing: the position-mapped kernels
+// ---- IQ1_S / IQ1_M in the stream packing: the position-mapped kernels
 bool gate_up_iq1s_pos_ok(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    if (!(l.gate_type == kIQ1_S && l.up_type == kIQ1_S && l.packing == MAYA_PACK_STREAM)) return false;
+    if (!((l.gate_type == kIQ1_S || l.gate_type == kIQ1_M) && l.up_type == l.gate_type && l.packing == MAYA_PACK_STREAM)) return false;
     if (l.n_embd % 1024 != 0 || l.n_ff % 16 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
     const int nw = l.n_embd / 1024;
     return nw == 4 || nw == 6 || nw == 7 || nw == 8;
 }
 bool down_iq1s_pos_ok(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    return l.down_type == kIQ1_S && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 &&
-           (l.down_off & 15) == 0;
+    return (l.down_type == kIQ1_S || l.down_type == kIQ1_M) && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 &&
+           l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
 }
 int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     const dim3 grid((unsigned) (a.layout.n_ff / 16), (unsigned) (a.n_tokens * a.k));
+    if (a.layout.gate_type == kIQ1_M) {
+        switch (a.layout.n_embd / 1024) {
+            case 4: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
+            case 6: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
+            case 7: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<7, 16, 8>), grid, dim3(448), 0, s, a, st.cb); break;
+            default: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<8, 16, 8>), grid, dim3(512), 0, s, a, st.cb); break;
+        }
+        MAYA_LAUNCHED("gate_up_iq1m_pos_kernel");
+        return MAYA_OK;
+    }
     switch (a.layout.n_embd / 1024) {
         case 4: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
         case 6: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
@@ -1293,7 +1359,8 @@ int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 }
 int launch_down_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     const dim3 grid((unsigned) (a.layout.n_embd / 16), (unsigned) a.n_tokens);
-    hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
+    if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
+    else hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
     MAYA_LAUNCHED("down_iq1s_pos_kernel");
     return MAYA_OK;
 }
@@ -1510,6 +1577,10 @@ static int repack_impl(const maya_moe_layout* l, const void* src, void* dst, voi
             const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
             if (dir == 0) hipLaunchKernelGGL(repack_iq1s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
             else hipLaunchKernelGGL(repack_iq1s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+        } else if (r.type == kIQ1_M) {
+            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
+            if (dir == 0) hipLaunchKernelGGL(repack_iq1m_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
+            else hipLaunchKernelGGL(repack_iq1m_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
         } else if (r.type == kQ8_0) {
             const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
             if (dir == 0) hipLaunchKernelGGL(repack_q80_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
@@ -1674,7 +1745,7 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     if (!a->hq.q && !a->hq.d && !a->hq.bsums && a->h && a->out && down_rounds_h(*a)) {
         int rc = 0;   // the kernel rounds h itself
         if (a->layout.down_type == kQ4_K) return launch_down_q4k_pos(*a, as_stream(stream));
-        if (a->layout.down_type == kIQ1_S) return launch_down_iq1s_pos(*a, *st, as_stream(stream));
+        if (a->layout.down_type == kIQ1_S || a->layout.down_type == kIQ1_M) return launch_down_iq1s_pos(*a, *st, as_stream(stream));
         if (try_down_iq2s_1tok(*a, *st, as_stream(stream), &rc)) return rc;
     }
     if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
@@ -1721,7 +1792,7 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
             return fail(MAYA_E_SHAPE, "mv: job %d: n_in %d (a multiple of 256 up to 16384) / n_out %d", i, j.n_in, j.n_out);
         if (j.ncol < 1 || j.ncol > MAYA_MAX_TOKENS) return fail(MAYA_E_SHAPE, "mv: job %d: ncol %d outside 1..%d", i, j.ncol, MAYA_MAX_TOKENS);
         if (j.packing == MAYA_PACK_STREAM && quad_packed(j.type) && j.n_out % 4)
-            return fail(MAYA_E_SHAPE, "mv: job %d: stream-packed IQ2_S / IQ1_S rows come in quads, n_out %d", i, j.n_out);
+            return fail(MAYA_E_SHAPE, "mv: job %d: stream-packed IQ2_S / IQ1_S / IQ1_M rows come in quads, n_out %d", i, j.n_out);
         if (j.packing == MAYA_PACK_STREAM && ((uintptr_t) j.w & 15)) return fail(MAYA_E_ARG, "mv: job %d: stream-packed weights must be 16-byte aligned", i);
         if (!j.w || !j.x.q || !j.x.d || (q8k_act(j.type) && !j.x.bsums) || !j.y) return fail(MAYA_E_ARG, "mv: job %d: null pointer", i);
         if (j.y_stride < j.n_out && j.ncol > 1) return fail(MAYA_E_ARG, "mv: job %d: y_stride %lld below n_out %d", i, (long long) j.y_stride, j.n_out);

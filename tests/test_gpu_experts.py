@@ -68,6 +68,11 @@ CASES = [
     (19, 19, 7168, 2048, 9, 8, 3),
     (19, 22, 6144, 2048, 4, 2, 2),
     (22, 19, 4096, 2048, 4, 3, 2),
+    # and IQ1_M
+    (29, 29, 4096, 2048, 6, 4, 1),
+    (29, 29, 7168, 2048, 9, 8, 3),
+    (29, 19, 6144, 2048, 4, 2, 2),
+    (12, 29, 8192, 2048, 4, 3, 2),
 ]
 
 
@@ -140,7 +145,7 @@ def test_zero_input_and_bf16_input(lib, oracle):
 
 
 @pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 12, 1024, 512, 10, 4, 6), (22, 22, 7168, 1024, 6, 4, 3), (22, 12, 4096, 2048, 7, 4, 4), (8, 8, 4096, 2048, 1, 1, 8),
-                                                     (19, 19, 4096, 2048, 5, 4, 4)))
+                                                     (19, 19, 4096, 2048, 5, 4, 4), (29, 29, 4096, 2048, 5, 4, 3)))
 def test_window_rows_equal_token_rows(lib, gt, dt, n_embd, n_ff, ne, k, nt):
     """A verify window's rows carry the bits its tokens give one at a time (the reference's window contract), in either
     row packing."""
@@ -172,9 +177,9 @@ def test_unsupported_and_bad_shapes_fail_cleanly(lib):
         lib.route_topk(torch.zeros((1, 4), device="cuda"), 8)
 
 
-@pytest.mark.parametrize("dt", (22, 12, 19))
+@pytest.mark.parametrize("dt", (22, 12, 19, 29))
 def test_down_rounds_h_itself_like_the_quantizer(lib, dt):
-    """The stream-packed IQ2_S / Q4_K / IQ1_S down kernels given no rounded h round it in their prologue: the same Q8_K codes as
+    """The stream-packed IQ2_S / Q4_K / IQ1_S / IQ1_M down kernels given no rounded h round it in their prologue: the same Q8_K codes as
     maya_quant_act (an all-zero block, equal magnitudes of both signs inside a lane's values, across lanes, and where
     the lower index sits in the higher lane), so the same output bits."""
     import ctypes as C

@@ -103,7 +103,7 @@ def test_i8x32_quant_byte_exact(lib, oracle):
         assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
 
 
-@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8), (19, 19), (19, 22)))
+@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8), (19, 19), (19, 22), (29, 29)))
 def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
     """maya_moe_repack regroups bytes only: unpack(repack(blob)) == blob, and the packed rows dequantize to the same bits."""
     n_embd, n_ff = 1024, 512
@@ -123,8 +123,23 @@ def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
         rb = lib.row_bytes(t, k)
         a = src[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
         b = packed[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
-        assert np.array_equal(np.sort(a, axis=1), np.sort(b, axis=1))
-        if t == 8:
+        if t != 29:   # (IQ1_M regroups bits, not bytes: the block scale's four nibbles are put together)
+            assert np.array_equal(np.sort(a, axis=1), np.sort(b, axis=1))
+        if t == 29:
+            # per quad the sub-blocks' index words [u][row], their qh words, then 8 bytes a (block, row): the FP16 block scale
+            # gathered from the top nibbles of the four scale words, then their 4 x 12 bits of 3-bit scales in order
+            nu = k // 32
+            g = src[off:off + rb * rows].view(rows // 4, 4, nu // 8, 56).cpu().numpy()
+            p = packed[off:off + rb * rows].view(rows // 4, 4 * rb).cpu().numpy()
+            want_i = g[:, :, :, 0:32].reshape(rows // 4, 4, nu, 4).transpose(0, 2, 1, 3).reshape(rows // 4, -1)
+            want_h = g[:, :, :, 32:48].reshape(rows // 4, 4, nu, 2).transpose(0, 2, 1, 3).reshape(rows // 4, -1)
+            w = g[:, :, :, 48:56].copy().view(np.uint16).astype(np.uint64)        # [quad][row][block][4]
+            d = (w[..., 0] >> 12) | ((w[..., 1] >> 8) & 0xf0) | ((w[..., 2] >> 4) & 0xf00) | (w[..., 3] & 0xf000)
+            rec = d | ((w[..., 0] & 0xfff) << 16) | ((w[..., 1] & 0xfff) << 28) | ((w[..., 2] & 0xfff) << 40) | ((w[..., 3] & 0xfff) << 52)
+            want_s = np.ascontiguousarray(rec.transpose(0, 2, 1)).view(np.uint8).reshape(rows // 4, -1)
+            assert np.array_equal(p[:, :16 * nu], want_i) and np.array_equal(p[:, 16 * nu:24 * nu], want_h)
+            assert np.array_equal(p[:, 24 * nu:], want_s)
+        elif t == 8:
             # Q8_0: a row's codes first, then its scales
             g = src[off:off + rb * rows].view(rows, k // 32, 34).cpu().numpy()
             p = packed[off:off + rb * rows].view(rows, rb).cpu().numpy()
