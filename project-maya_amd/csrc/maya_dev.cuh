@@ -63,6 +63,68 @@ __device__ __forceinline__ uint32_t neg_bytes(uint32_t g, uint32_t c) {
 //
 // Fmt<TYPE>: kBytes / kValues of a block; kUnit values a lane takes a step; decode(blk, u, cb) fills codes and scales.
 
+// A lane's value of lane ^ 1 (CTRL 0xB1, quad_perm [1,0,3,2]), lane ^ 2 (0x4E, quad_perm [2,3,0,1]) or of lane 7 - (lane & 7)
+// in its run of 8 (0x141, row_half_mirror): data-parallel-primitive moves, no LDS traffic.
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true); }
+
+// Q8_K rounding of a 256-value block held by 8 consecutive lanes, 32 values a lane: the arithmetic of the reference's quantize_q8_K_kernel (src/kernels/cuda/quantize_act.cu:161-207) and
+// codes, bit for bit, 4 codes a word in the order of v.  The block's scale comes from the signed value at the FIRST
+// largest magnitude.  Its magnitude is the largest magnitude; its sign depends on the order only when the largest
+// positive and the largest negative value share that magnitude.  So the common case needs two max3 chains over the raw
+// bits (as signed integers the largest is the largest positive value; as unsigned integers the largest is the negative
+// value of the largest magnitude) and three lane exchanges; only a wave that holds such a tie scans with indices
+// (index_of(i) = the index of v[i] inside the block, ascending in i).  A product never rounds beyond +-127
+// (|iscale * v| <= 127 (1 + 2^-23)), so the low byte of the magic-number sum is the code.
+template <typename IndexOf>
+__device__ __forceinline__ void q8k_round_lane32(const float (&v)[32], IndexOf index_of, int (&y)[8], float& d) {
+    int pb = __float_as_int(v[0]);
+    uint32_t nb = __float_as_uint(v[0]);
+#pragma unroll
+    for (int i = 1; i < 31; i += 2) {
+        pb = max(max(pb, __float_as_int(v[i])), __float_as_int(v[i + 1]));
+        nb = max(max(nb, __float_as_uint(v[i])), __float_as_uint(v[i + 1]));
+    }
+    pb = max(pb, __float_as_int(v[31]));
+    nb = max(nb, __float_as_uint(v[31]));
+    pb = max(pb, dpp_i<0xB1>(pb)), nb = max(nb, (uint32_t) dpp_i<0xB1>((int) nb));
+    pb = max(pb, dpp_i<0x4E>(pb)), nb = max(nb, (uint32_t) dpp_i<0x4E>((int) nb));
+    pb = max(pb, dpp_i<0x141>(pb)), nb = max(nb, (uint32_t) dpp_i<0x141>((int) nb));
+    const int pos = max(pb, 0);                                   // bits of the largest positive value, 0: none
+    const int neg = (nb >> 31) ? (int) (nb & 0x7fffffffu) : 0;    // bits of the largest magnitude among the negative ones
+    float sv = pos > neg ? __int_as_float(pos) : (neg > pos ? -__int_as_float(neg) : 0.0f);
+    if (__any(pos == neg && pos != 0)) {
+        float am = 0.0f;
+        int ix = 0;
+        sv = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {   // ascending index inside the lane: a strict > keeps the first
+            const float av = fabsf(v[i]);
+            if (av > am) am = av, sv = v[i], ix = index_of(i);
+        }
+#pragma unroll
+        for (int o = 1; o < 8; o <<= 1) {
+            const float oa = __shfl_xor(am, o, kWave), os = __shfl_xor(sv, o, kWave);
+            const int oi = __shfl_xor(ix, o, kWave);
+            if (oa > am || (oa == am && oi < ix)) am = oa, sv = os, ix = oi;
+        }
+    }
+    float iscale = 0.0f;
+    d = 0.0f;
+    if (sv != 0.0f) {
+        iscale = __fdiv_rn(-127.0f, sv);
+        d = __fdiv_rn(1.0f, iscale);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        uint32_t c[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) c[b] = __float_as_uint(__fadd_rn(__fmul_rn(iscale, v[4 * i + b]), 12582912.0f));
+        const uint32_t lo = __builtin_amdgcn_perm(c[1], c[0], 0x0c0c0400u), hi = __builtin_amdgcn_perm(c[3], c[2], 0x0c0c0400u);
+        y[i] = (int) __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+    }
+}
+
 struct Unit32 {
     int q[8];    // 32 int8 codes in value order (the IQ1 types: codes + 9 - delta, see Fmt<kIQ1_S>)
     int s0, s1;  // integer scales of values 0..15 / 16..31

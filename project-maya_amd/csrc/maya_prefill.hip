@@ -121,83 +121,102 @@ template <int DT> __device__ __forceinline__ float pf_load(const void* x, int64_
 }
 __device__ __forceinline__ int pf_rint(float f) { return (int) rintf(f); }
 
-// ggml's nearest_int: the magic-number round (ties to even) of a product already rounded to F32
-__device__ __forceinline__ int pf_nearest_int(float f) {
-    const float v = __fadd_rn(f, 12582912.0f);
-    return (__float_as_int(v) & 0x007fffff) - 0x00400000;
-}
-// One 256-value block by the 256 threads of a workgroup (thread = value), Q8_K - the activation format of the
-// reference's CPU expert path for the K-quants (src/kernels/cuda/quantize_act.cu:161-207): the block's signed maximum
-// is the value at the FIRST largest magnitude, iscale = -127 / max, c = min(127, nearest_int(iscale x)), d = 1 / iscale;
-// s = d * (the sum of each 32 codes), what the minimums of a Q4_K sub-block multiply.  sm: 256 + 8 words.
-struct PfCodes {
-    int c;
+// Q8_K rows - the activation format of the reference's CPU expert path for the K-quants
+// (src/kernels/cuda/quantize_act.cu:161-207) - rounded 32 values a lane, 8 lanes a 256-value block (q8k_round_lane32: no
+// LDS, no barrier): the block's signed maximum is the value at the FIRST largest magnitude, iscale = -127 / max,
+// c = min(127, nearest_int(iscale x)), d = 1 / iscale; s = d * (the sum of each 32 codes), what the minimums of a Q4_K
+// sub-block multiply.
+struct PfLane {
+    int y[8];      // 32 codes
     float d, ds;
 };
-__device__ __forceinline__ PfCodes pf_quant_block(float xv, int* sm) {
-    const int j = threadIdx.x;
-    float am = fabsf(xv);
-    int ix = j;
+template <int DT>
+__device__ __forceinline__ void pf_load32(const void* x, int64_t i0, bool on, float (&v)[32]) {
+    if (!on) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float oa = __shfl_xor(am, o, 64);
-        const int oi = __shfl_xor(ix, o, 64);
-        if (oa > am || (oa == am && oi < ix)) am = oa, ix = oi;
+        for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+        return;
     }
-    float* s_x = (float*) sm;
-    float* s_am = (float*) (sm + 256);
-    int* s_ix = sm + 260;
-    s_x[j] = xv;
-    if ((j & 63) == 0) s_am[j >> 6] = am, s_ix[j >> 6] = ix;
-    __syncthreads();
-    am = s_am[0], ix = s_ix[0];
+    if constexpr (DT == MAYA_DT_F32) {
+        const float* p = (const float*) x + i0;
+        if (((uintptr_t) p & 15) == 0) {
 #pragma unroll
-    for (int w = 1; w < 4; ++w)
-        if (s_am[w] > am) am = s_am[w], ix = s_ix[w];   // (a later wave holds later indices: a tie keeps the earlier)
-    PfCodes o;
-    o.c = 0, o.d = 0.0f;
-    if (am > 0.0f) {
-        const float iscale = __fdiv_rn(-127.0f, s_x[ix]);
-        o.c = min(127, pf_nearest_int(__fmul_rn(iscale, xv)));
-        o.d = __fdiv_rn(1.0f, iscale);
+            for (int i = 0; i < 8; ++i) {
+                const float4 t = ((const float4*) p)[i];
+                v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+            }
+            return;
+        }
+    } else {
+        const uint16_t* p = (const uint16_t*) x + i0;
+        if (((uintptr_t) p & 15) == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 t = ((const uint4*) p)[i];
+                const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if constexpr (DT == MAYA_DT_BF16) {
+                        v[8 * i + 2 * j] = __uint_as_float(w[j] << 16);
+                        v[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+                    } else {
+                        v[8 * i + 2 * j] = f16_bits_to_f32(w[j] & 0xffffu);
+                        v[8 * i + 2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+                    }
+                }
+            }
+            return;
+        }
     }
-    int sum = o.c;
 #pragma unroll
-    for (int s = 16; s > 0; s >>= 1) sum += __shfl_xor(sum, s, 64);
+    for (int i = 0; i < 32; ++i) v[i] = pf_load<DT>(x, i0 + i);
+}
+__device__ __forceinline__ PfLane pf_round_lane(const float (&v)[32], int lane) {
+    PfLane o;
+    q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, o.y, o.d);
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum = dot4(0x01010101, o.y[i], sum);
     o.ds = __fmul_rn(o.d, (float) sum);
-    __syncthreads();   // (sm is free for the next block)
     return o;
 }
-__device__ __forceinline__ void pf_store_codes(const maya_prefill_act& o, size_t row, int64_t k, int64_t v, const PfCodes& c) {
-    const size_t at = row * (size_t) k + (size_t) v;
-    o.q[at] = (int8_t) c.c;
-    if ((threadIdx.x & 31) == 0) o.s[at >> 5] = c.ds;
-    if (threadIdx.x == 0) o.d[at >> 8] = c.d;
+__device__ __forceinline__ void pf_store_lane(const maya_prefill_act& o, size_t row, int64_t k, int64_t v0, int lane, const PfLane& c) {
+    const size_t at = row * (size_t) k + (size_t) v0;
+    int4* q = (int4*) (o.q + at);
+    q[0] = make_int4(c.y[0], c.y[1], c.y[2], c.y[3]);
+    q[1] = make_int4(c.y[4], c.y[5], c.y[6], c.y[7]);
+    o.s[at >> 5] = c.ds;
+    if ((lane & 7) == 0) o.d[at >> 8] = c.d;
 }
 
-// grid (k / 256, tokens): a token's block is rounded once and written to the rows of all its entries in the plan
+// grid (k / 8192 rounded up, tokens): a token's values are rounded once and written to the rows of all its entries in the plan
 template <int DT>
 __global__ __launch_bounds__(256) void prefill_quant_kernel(const void* __restrict__ x, int64_t x_stride, maya_prefill_plan p,
                                                             int top_k, int64_t k, maya_prefill_act o) {
-    __shared__ int sm[264];
-    const int t = blockIdx.y;
-    const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;
-    const PfCodes c = pf_quant_block(pf_load<DT>(x, (int64_t) t * x_stride + v), sm);
+    const int t = blockIdx.y, lane = threadIdx.x & 63;
+    const int64_t v0 = ((int64_t) blockIdx.x * 256 + threadIdx.x) * 32;
+    const bool on = v0 < k;   // (k is a multiple of 256: the 8 lanes of a block are on or off together)
+    float v[32];
+    pf_load32<DT>(x, (int64_t) t * x_stride + v0, on, v);
+    const PfLane c = pf_round_lane(v, lane);
+    if (!on) return;
     for (int j = 0; j < top_k; ++j) {
         const int row = p.entry_row[t * top_k + j];
         if (row < 0) continue;   // an entry of an expert that is not resident
-        pf_store_codes(o, (size_t) row, k, v, c);
+        pf_store_lane(o, (size_t) row, k, v0, lane, c);
     }
 }
-// grid (k / 256, rows at most): the plan's row blockIdx.y of an F32 matrix (the SwiGLU outputs)
+// grid (k / 8192 rounded up, rows at most): the plan's row blockIdx.y of an F32 matrix (the SwiGLU outputs)
 __global__ __launch_bounds__(256) void prefill_quant_rows_kernel(const float* __restrict__ x, maya_prefill_plan p, int n_expert,
                                                                  int64_t k, maya_prefill_act o) {
-    __shared__ int sm[264];
-    const int row = blockIdx.y;
+    const int row = blockIdx.y, lane = threadIdx.x & 63;
     if (row >= p.bounds[n_expert]) return;
-    const int64_t v = (int64_t) blockIdx.x * 256 + threadIdx.x;
-    const PfCodes c = pf_quant_block(x[(size_t) row * k + v], sm);
-    pf_store_codes(o, (size_t) row, k, v, c);
+    const int64_t v0 = ((int64_t) blockIdx.x * 256 + threadIdx.x) * 32;
+    const bool on = v0 < k;
+    float v[32];
+    pf_load32<MAYA_DT_F32>(x, (int64_t) row * k + v0, on, v);
+    const PfLane c = pf_round_lane(v, lane);
+    if (on) pf_store_lane(o, (size_t) row, k, v0, lane, c);
 }
 
 // ---------------------------------------------------------------------------------------------------- the GEMM
@@ -603,7 +622,7 @@ int maya_moe_prefill_quant(const void* x, int x_dtype, int64_t x_stride, const m
         return fail(MAYA_E_SHAPE, "prefill_quant: entries %d k %d n_embd %lld", n_entries, k, (long long) n_embd);
     if (x_stride == 0) x_stride = n_embd;
     if (n_entries % k) return fail(MAYA_E_SHAPE, "prefill_quant: %d entries are not whole tokens of %d", n_entries, k);
-    const dim3 grid((unsigned) (n_embd / 256), (unsigned) (n_entries / k));
+    const dim3 grid((unsigned) ((n_embd + 8191) / 8192), (unsigned) (n_entries / k));
     hipStream_t s = as_stream(stream);
     switch (x_dtype) {
         case MAYA_DT_F32: hipLaunchKernelGGL(prefill_quant_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, x, x_stride, *plan, k, n_embd, xq); break;
@@ -646,7 +665,7 @@ int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_ta
     const dim3 grid((unsigned) (l->n_ff / 64), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
     if (const int rc = pf_launch<true>(a, grid, as_stream(stream))) return rc;
     MAYA_LAUNCHED("prefill_q4k_kernel<gate_up>");
-    const dim3 qgrid((unsigned) (l->n_ff / 256), (unsigned) n_entries);
+    const dim3 qgrid((unsigned) ((l->n_ff + 8191) / 8192), (unsigned) n_entries);
     hipLaunchKernelGGL(prefill_quant_rows_kernel, qgrid, dim3(256), 0, as_stream(stream), (const float*) h, *plan, n_expert, (int64_t) l->n_ff, hq);
     MAYA_LAUNCHED("prefill_quant_rows_kernel");
     return MAYA_OK;
