@@ -194,12 +194,13 @@ __device__ __forceinline__ h2 as_h2(uint32_t v) {
 }
 template <int K2>
 __device__ __forceinline__ void tile_values(uint32_t wa, uint32_t wb, int sh, h2& w01, h2& w23) {
-    const uint32_t c = (uint32_t) ((((uint64_t) wa << 32) | (uint64_t) wb) >> sh);
+    const uint32_t c = __builtin_amdgcn_alignbit(wa, wb, (uint32_t) sh);   // (wa : wb) >> sh, 0 <= sh < 32
     uint32_t hb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t st = __builtin_amdgcn_ubfe(c, Taps<K2>::below(i), 16);
-        hb[i] = __builtin_amdgcn_sad_u8(st * 0x83DCD12Du, 0u, 0x6400u);   // the bits of FP16(1024 + byte sum)
+        const uint32_t prod = st * 0x83DCD12Du;
+        hb[i] = __builtin_amdgcn_sad_u8(prod, 0u, 0x6400u);   // the bits of FP16(1024 + byte sum)
     }
     const h2 kinv = as_h2(0x1eee1eeeu), kbias = as_h2(0xc931c931u);
     w01 = __builtin_elementwise_fma(as_h2(hb[0] | (hb[1] << 16)), kinv, kbias);

@@ -19,7 +19,6 @@
 namespace maya {
 
 constexpr int kPfRows = 64;        // rows of a tile
-constexpr int kPfMt = kPfRows / 16;
 constexpr int kPlanThreads = 1024;
 constexpr int kPlanWaves = kPlanThreads / 64;
 
@@ -295,25 +294,18 @@ __device__ __forceinline__ float pf_swiglu(float g, float u, float limit) {
 }
 
 typedef unsigned short pf_u16x2 __attribute__((ext_vector_type(2)));
-// eight 4-bit codes (one a byte) times a factor <= 7: no byte overflows, so two packed 16-bit multiplies a word do it
-__device__ __forceinline__ long pf_scale_codes(uint64_t w, uint32_t f) {
+// four 4-bit codes (one a byte) times a factor <= 7: no byte overflows, so one packed 16-bit multiply does it
+__device__ __forceinline__ uint32_t pf_scale_codes(uint32_t w, uint32_t f) {
     const pf_u16x2 ff = {(unsigned short) f, (unsigned short) f};
-    const pf_u16x2 lo = __builtin_bit_cast(pf_u16x2, (uint32_t) w) * ff, hi = __builtin_bit_cast(pf_u16x2, (uint32_t) (w >> 32)) * ff;
-    return (long) (((uint64_t) __builtin_bit_cast(uint32_t, hi) << 32) | (uint64_t) __builtin_bit_cast(uint32_t, lo));
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(pf_u16x2, w) * ff);
 }
 
 // LDS reads of the GEMM loop are written out by hand.  The compiler cannot tell which LDS buffer a direct-to-LDS copy
 // fills, so before any LDS read of its own it waits for every copy in flight - here that would be the copy of the
 // super-block two ahead, issued moments earlier.  These reads it does not see; each group is followed by pf_lds_wait
 // on the registers it filled (the values pass through the wait, so nothing that uses them can move above it).
-typedef int pf_i2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pf_lds_addr(const void* p) {
     return (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) void*) p;
-}
-template <int OFF> __device__ __forceinline__ pf_i2 pf_lds_b64(uint32_t addr) {
-    pf_i2 v;
-    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
-    return v;
 }
 template <int OFF> __device__ __forceinline__ float pf_lds_f32(uint32_t addr) {
     float v;
@@ -322,6 +314,11 @@ template <int OFF> __device__ __forceinline__ float pf_lds_f32(uint32_t addr) {
 }
 template <int OFF> __device__ __forceinline__ v4f pf_lds_f32x4(uint32_t addr) {
     v4f v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> __device__ __forceinline__ v4i pf_lds_i32x4(uint32_t addr) {
+    v4i v;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
     return v;
 }
@@ -382,23 +379,25 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     dma.init(a, row0, nrows, wave, lane);
     dma.copy(b0, 0);
     if (nsb > 1) dma.copy(b1, 1);
-    // the weights of a super-block - the 16-byte header and the lane's four 8-byte slices of the codes of each of its two
-    // rows
-    uint64_t q[4][2], qn[4][2];     // [slice][row tile]
+    // the weights of a super-block - the 16-byte header of each of the lane's two rows and two 16-byte pieces of its
+    // codes: bytes 64 h + 16 g of the row's 128, h = 0, 1 (so the four lanes of a row read 64 bytes in a run)
+    typedef uint32_t w4 __attribute__((ext_vector_type(4)));
+    w4 q[2][2], qn[2][2];           // [piece h][row tile]
     uint32_t hdr[2][4], hdrn[2][4];
-    auto load_block = [&](int sb, uint64_t (&dq)[4][2], uint32_t (&dh)[2][4]) {
+    auto load_block = [&](int sb, w4 (&dq)[2][2], uint32_t (&dh)[2][4]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             wptr blk = wrow[t] + (size_t) sb * 144;
-            typedef uint32_t w4 __attribute__((ext_vector_type(4)));
             const w4 h = *(const __attribute__((address_space(1))) w4*) blk;
             dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) dq[j][t] = *(const __attribute__((address_space(1))) uint64_t*) (blk + 16 + 32 * j + 8 * g);
+            for (int j = 0; j < 2; ++j) dq[j][t] = *(const __attribute__((address_space(1))) w4*) (blk + 16 + 64 * j + 16 * g);
         }
     };
     if (wave_on) load_block(0, q, hdr);
-    const int a_base = ln * 256 + 8 * (g & 1), a_swz = (ln ^ (g >> 1)) << 4;
+    // a lane's 16 codes of a matrix instruction: values 16 (g & 1) .. + 15 of sub-block 4 h + 2 (g >> 1) + n = the row's
+    // 16-byte chunk 8 h + 2 n + 4 (g >> 1) + (g & 1), which sits at that index ^ the row
+    const int a_base = ln * 256, a_swz = (ln ^ (4 * (g >> 1) + (g & 1))) << 4;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     auto step = [&](int sb, const uint8_t* buf, uint8_t* buf2) {   // super-block sb from buf; sb + 2 is copied into buf2
@@ -442,41 +441,45 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
                             acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[2 * m + half], nb[half][t], acc[t][m], 0, 0, 0);
             }
             // The two plane products of the block, int32: [t][m][0] = (q lo) . c, [1] = (q hi) . c.  One 64-deep matrix
-            // instruction takes the two sub-blocks of a 32-byte slice of the codes: a lane's first 8 operand bytes are the
-            // low nibbles (sub-block 2p, values 8 g .. 8 g + 7), its second 8 the high nibbles (sub-block 2p + 1, the same
-            // values), each times its own sub-block's factor; the activations' operand pairs the same two runs of 8 codes.
+            // instruction takes the low (n = 0) or the high (n = 1) nibbles of the four lanes' pieces h: two whole
+            // sub-blocks, 4 h + n and 4 h + 2 + n, a lane's 16 operand bytes = 16 values of one of them times that
+            // sub-block's factor; the activations' operand is the same 16 codes (one 16-byte LDS read).
             v4i dot[2][NMT][2];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                pf_i2 xr[2 * NMT];
-                {
-                    const uint32_t at0 = lbuf + a_base + (a_swz ^ (64 * p)), at1 = lbuf + a_base + (a_swz ^ (64 * p + 32));
-                    pf_for_m<0, NMT>([&](auto mc) {
-                        constexpr int m = decltype(mc)::value;
-                        xr[2 * m] = pf_lds_b64<m * 4096>(at0);
-                        xr[2 * m + 1] = pf_lds_b64<m * 4096>(at1);
-                    });
-                }
-                v4i wl[2], wh[2];
+            for (int h = 0; h < 2; ++h) {
+                uint32_t s2[2];
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    const uint64_t w0 = q[p][t] & 0x0f0f0f0f0f0f0f0full, w1 = (q[p][t] >> 4) & 0x0f0f0f0f0f0f0f0full;
-                    const uint32_t s2 = sc[t][p >> 1] >> (16 * (p & 1));
-                    const uint32_t sa = s2 & 0x3fu, sb6 = (s2 >> 8) & 0x3fu;
-                    const long l0 = pf_scale_codes(w0, sa & 7u), l1 = pf_scale_codes(w1, sb6 & 7u);
-                    const long h0 = pf_scale_codes(w0, sa >> 3), h1 = pf_scale_codes(w1, sb6 >> 3);
-                    wl[t] = v4i{(int) l0, (int) (l0 >> 32), (int) l1, (int) (l1 >> 32)};
-                    wh[t] = v4i{(int) h0, (int) (h0 >> 32), (int) h1, (int) (h1 >> 32)};
-                }
-                pf_lds_wait(xr);
+                for (int t = 0; t < 2; ++t) s2[t] = sc[t][h] >> (16 * (g >> 1));   // the scales of sub-blocks 4 h + 2 (g >> 1), + 1
 #pragma unroll
-                for (int m = 0; m < NMT; ++m) {
-                    const v4i xc = {xr[2 * m].x, xr[2 * m].y, xr[2 * m + 1].x, xr[2 * m + 1].y};
+                for (int n = 0; n < 2; ++n) {
+                    v4i xr[NMT];
+                    {
+                        const uint32_t at = lbuf + a_base + (a_swz ^ ((8 * h + 2 * n) << 4));
+                        pf_for_m<0, NMT>([&](auto mc) {
+                            constexpr int m = decltype(mc)::value;
+                            xr[m] = pf_lds_i32x4<m * 4096>(at);
+                        });
+                    }
+                    v4i wl[2], wh[2];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        const v4i z = {0, 0, 0, 0};
-                        dot[t][m][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xc, wl[t], p ? dot[t][m][0] : z, 0, 0, 0);
-                        dot[t][m][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xc, wh[t], p ? dot[t][m][1] : z, 0, 0, 0);
+                        const uint32_t f = (s2[t] >> (8 * n)) & 0x3fu, flo = f & 7u, fhi = f >> 3;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t w = (q[h][t][i] >> (4 * n)) & 0x0f0f0f0fu;
+                            wl[t][i] = (int) pf_scale_codes(w, flo);
+                            wh[t][i] = (int) pf_scale_codes(w, fhi);
+                        }
+                    }
+                    pf_lds_wait(xr);
+#pragma unroll
+                    for (int m = 0; m < NMT; ++m) {
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) {
+                            const v4i z = {0, 0, 0, 0};
+                            dot[t][m][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xr[m], wl[t], (h | n) ? dot[t][m][0] : z, 0, 0, 0);
+                            dot[t][m][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xr[m], wh[t], (h | n) ? dot[t][m][1] : z, 0, 0, 0);
+                        }
                     }
                 }
             }
@@ -501,7 +504,8 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i], q[i][t] = qn[i][t];
+                    for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i];
+                    q[0][t] = qn[0][t], q[1][t] = qn[1][t];
                 }
             }
         }
