@@ -125,6 +125,14 @@ size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int 
  * (include/strata/kernels/glm_fast.hpp:284-300); this is the hook that runs on that copy.  src and dst must not overlap. */
 int maya_moe_repack(const maya_moe_layout* l, const void* src, void* dst, void* stream);
 int maya_moe_unpack(const maya_moe_layout* l, const void* src, void* dst, void* stream);
+/* A layer's expert blobs from its three stacked GGUF tensors, on the device: blob e at dst + e * dst_stride receives
+ * [gate rows | up rows | down rows] of expert e - gate_exps / up_exps / down_exps are ffn_{gate,up,down}_exps.weight as the
+ * file stores them, [n_expert][rows][row bytes] - in GGUF order (packing MAYA_PACK_GGUF: the concatenation the
+ * reference's packer writes on the host, tools/iq_pack.py:510-514, read back as native_expert_layout's blob,
+ * src/kernels/cuda/iq_kernels.cu:1077-1101) or already regrouped for the streaming kernels (MAYA_PACK_STREAM: what
+ * maya_moe_repack makes of that blob).  `l` describes the GGUF blob (maya_moe_layout_init); dst_stride >= its size. */
+int maya_moe_pack_experts(const maya_moe_layout* l, const void* gate_exps, const void* up_exps, const void* down_exps,
+                          int n_expert, int packing, void* dst, size_t dst_stride, void* stream);
 
 const char* maya_last_error(void);
 /* Device and library identification: "gfx950 ..." (host string, valid until the next call on this thread). */

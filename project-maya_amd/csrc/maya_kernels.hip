@@ -193,7 +193,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 // sub-block, grid (k/32 sub-blocks / 256, rows).  DIR 0: GGUF -> stream, 1: stream -> GGUF.  Every byte is written once.
 template <int DIR>
 __global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                          int64_t k, int64_t n_rows) {
+                                                          int64_t k, int64_t n_rows, size_t src_stride, size_t dst_stride) {
+    src += blockIdx.z * src_stride, dst += blockIdx.z * dst_stride;   // blob blockIdx.z of a layer's experts
     const int64_t nu = k >> 5, rb = (k >> 8) * 82;
     const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
     if (un >= nu) return;
@@ -229,7 +230,8 @@ __global__ __launch_bounds__(256) void repack_iq2s_kernel(const uint8_t* __restr
 // qh words, then the block scales); one thread a sub-block, grid (k/32 sub-blocks / 256, rows).  DIR as above.
 template <int DIR>
 __global__ __launch_bounds__(256) void repack_iq1s_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                          int64_t k, int64_t n_rows) {
+                                                          int64_t k, int64_t n_rows, size_t src_stride, size_t dst_stride) {
+    src += blockIdx.z * src_stride, dst += blockIdx.z * dst_stride;   // blob blockIdx.z of a layer's experts
     const int64_t nu = k >> 5, rb = (k >> 8) * 50;
     const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
     if (un >= nu) return;
@@ -255,7 +257,8 @@ __global__ __launch_bounds__(256) void repack_iq1s_kernel(const uint8_t* __restr
 // nibbles of the four scale words, and their 4 x 12 bits of 3-bit scales in order); one thread a sub-block.
 template <int DIR>
 __global__ __launch_bounds__(256) void repack_iq1m_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                          int64_t k, int64_t n_rows) {
+                                                          int64_t k, int64_t n_rows, size_t src_stride, size_t dst_stride) {
+    src += blockIdx.z * src_stride, dst += blockIdx.z * dst_stride;   // blob blockIdx.z of a layer's experts
     const int64_t nu = k >> 5, rb = (k >> 8) * 56;
     const int64_t un = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
     if (un >= nu) return;
@@ -295,7 +298,8 @@ __global__ __launch_bounds__(256) void repack_iq1m_kernel(const uint8_t* __restr
 // scales); one thread a block, grid (k/32 blocks / 256, rows).  DIR 0: GGUF -> stream, 1: stream -> GGUF.
 template <int DIR>
 __global__ __launch_bounds__(256) void repack_q80_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int64_t k,
-                                                         int64_t n_rows) {
+                                                         int64_t n_rows, size_t src_stride, size_t dst_stride) {
+    src += blockIdx.z * src_stride, dst += blockIdx.z * dst_stride;
     const int64_t nb = k >> 5, rb = nb * 34;
     const int64_t b = (int64_t) blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
     if (b >= nb || row >= n_rows) return;
@@ -313,8 +317,18 @@ __global__ __launch_bounds__(256) void repack_q80_kernel(const uint8_t* __restri
     }
 }
 
-__global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n) {
-    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) gridDim.x * 256) dst[i] = src[i];
+// n bytes of blob blockIdx.z, 16 at a time where both sides are aligned
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n,
+                                                         size_t src_stride, size_t dst_stride) {
+    src += blockIdx.z * src_stride, dst += blockIdx.z * dst_stride;
+    const size_t i0 = (size_t) blockIdx.x * 256 + threadIdx.x, step = (size_t) gridDim.x * 256;
+    if ((((uintptr_t) src | (uintptr_t) dst) & 15) == 0) {
+        const size_t n16 = n >> 4;
+        for (size_t i = i0; i < n16; i += step) ((uint4*) dst)[i] = ((const uint4*) src)[i];
+        for (size_t i = (n16 << 4) + i0; i < n; i += step) dst[i] = src[i];
+    } else {
+        for (size_t i = i0; i < n; i += step) dst[i] = src[i];
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ activation quantizers
@@ -1493,46 +1507,76 @@ size_t maya_moe_layout_init(maya_moe_layout* l, int gate_type, int up_type, int 
     return l->down_off + maya_moe_row_bytes(down_type, n_ff) * (size_t) n_embd;
 }
 
-static int repack_impl(const maya_moe_layout* l, const void* src, void* dst, void* stream, int dir) {
-    DeviceState* st;
-    if (const int rc = current_state(&st)) return rc;
-    if (!l || !src || !dst) return fail(MAYA_E_ARG, "repack: null pointer");
-    if (const int rc = check_layout(*l)) return rc;
-    if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_ARG, "repack: the layout must describe the GGUF blob");
+// dir 0: the blobs' GGUF row arrays -> stream order, 1: back, 2: a plain copy.  role i of blob b is read at
+// src[i] + b * src_stride[i] and written at dst[i] + b * dst_stride.
+static int repack_impl(const maya_moe_layout* l, const uint8_t* const (&src)[3], const size_t (&src_stride)[3], uint8_t* const (&dst)[3],
+                       size_t dst_stride, int n_blobs, void* stream, int dir) {
     hipStream_t s = as_stream(stream);
-    const struct { int type; uint64_t off; int64_t k, rows; } roles[3] = {
-        {l->gate_type, l->gate_off, l->n_embd, l->n_ff},
-        {l->up_type, l->up_off, l->n_embd, l->n_ff},
-        {l->down_type, l->down_off, l->n_ff, l->n_embd}};
-    for (const auto& r : roles) {
-        const uint8_t* sp = (const uint8_t*) src + r.off;
-        uint8_t* dp = (uint8_t*) dst + r.off;
-        if (r.type == kIQ2_S) {
-            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
-            if (dir == 0) hipLaunchKernelGGL(repack_iq2s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-            else hipLaunchKernelGGL(repack_iq2s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-        } else if (r.type == kIQ1_S) {
-            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
-            if (dir == 0) hipLaunchKernelGGL(repack_iq1s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-            else hipLaunchKernelGGL(repack_iq1s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-        } else if (r.type == kIQ1_M) {
-            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
-            if (dir == 0) hipLaunchKernelGGL(repack_iq1m_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-            else hipLaunchKernelGGL(repack_iq1m_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-        } else if (r.type == kQ8_0) {
-            const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows);
-            if (dir == 0) hipLaunchKernelGGL(repack_q80_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-            else hipLaunchKernelGGL(repack_q80_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows);
-        } else {
+    const struct { int type; int64_t k, rows; } roles[3] = {
+        {l->gate_type, l->n_embd, l->n_ff}, {l->up_type, l->n_embd, l->n_ff}, {l->down_type, l->n_ff, l->n_embd}};
+    for (int i = 0; i < 3; ++i) {
+        const auto& r = roles[i];
+        const uint8_t* sp = src[i];
+        uint8_t* dp = dst[i];
+        const size_t ss = src_stride[i], ds = dst_stride;
+        const dim3 grid((unsigned) (((r.k >> 5) + 255) / 256), (unsigned) r.rows, (unsigned) n_blobs);
+        if (dir == 2 || !(quad_packed(r.type) || r.type == kQ8_0)) {
             const size_t n = maya_moe_row_bytes(r.type, r.k) * (size_t) r.rows;
-            hipLaunchKernelGGL(copy_bytes_kernel, dim3(1024), dim3(256), 0, s, sp, dp, n);
+            hipLaunchKernelGGL(copy_bytes_kernel, dim3(256, 1, (unsigned) n_blobs), dim3(256), 0, s, sp, dp, n, ss, ds);
+        } else if (r.type == kIQ2_S) {
+            if (dir == 0) hipLaunchKernelGGL(repack_iq2s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+            else hipLaunchKernelGGL(repack_iq2s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+        } else if (r.type == kIQ1_S) {
+            if (dir == 0) hipLaunchKernelGGL(repack_iq1s_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+            else hipLaunchKernelGGL(repack_iq1s_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+        } else if (r.type == kIQ1_M) {
+            if (dir == 0) hipLaunchKernelGGL(repack_iq1m_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+            else hipLaunchKernelGGL(repack_iq1m_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+        } else {
+            if (dir == 0) hipLaunchKernelGGL(repack_q80_kernel<0>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
+            else hipLaunchKernelGGL(repack_q80_kernel<1>, grid, dim3(256), 0, s, sp, dp, r.k, r.rows, ss, ds);
         }
         MAYA_LAUNCHED("repack kernel");
     }
     return MAYA_OK;
 }
-int maya_moe_repack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_impl(l, src, dst, stream, 0); }
-int maya_moe_unpack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_impl(l, src, dst, stream, 1); }
+static int repack_blob(const maya_moe_layout* l, const void* src, void* dst, void* stream, int dir) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l || !src || !dst) return fail(MAYA_E_ARG, "repack: null pointer");
+    if (const int rc = check_layout(*l)) return rc;
+    if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_ARG, "repack: the layout must describe the GGUF blob");
+    const uint8_t* sp = (const uint8_t*) src;
+    uint8_t* dp = (uint8_t*) dst;
+    const uint8_t* const srcs[3] = {sp + l->gate_off, sp + l->up_off, sp + l->down_off};
+    uint8_t* const dsts[3] = {dp + l->gate_off, dp + l->up_off, dp + l->down_off};
+    const size_t strides[3] = {0, 0, 0};
+    return repack_impl(l, srcs, strides, dsts, 0, 1, stream, dir);
+}
+int maya_moe_repack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_blob(l, src, dst, stream, 0); }
+int maya_moe_unpack(const maya_moe_layout* l, const void* src, void* dst, void* stream) { return repack_blob(l, src, dst, stream, 1); }
+
+int maya_moe_pack_experts(const maya_moe_layout* l, const void* gate_exps, const void* up_exps, const void* down_exps, int n_expert,
+                          int packing, void* dst, size_t dst_stride, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l || !gate_exps || !up_exps || !down_exps || !dst) return fail(MAYA_E_ARG, "pack_experts: null pointer");
+    if (const int rc = check_layout(*l)) return rc;
+    if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_ARG, "pack_experts: the layout must describe the GGUF blob");
+    if (packing != MAYA_PACK_GGUF && packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "pack_experts: packing %d", packing);
+    if (n_expert <= 0 || n_expert > 65535) return fail(MAYA_E_SHAPE, "pack_experts: %d experts", n_expert);
+    const size_t gb = maya_moe_row_bytes(l->gate_type, l->n_embd) * (size_t) l->n_ff, ub = maya_moe_row_bytes(l->up_type, l->n_embd) * (size_t) l->n_ff;
+    const size_t db = maya_moe_row_bytes(l->down_type, l->n_ff) * (size_t) l->n_embd;
+    if (dst_stride < l->down_off + db) return fail(MAYA_E_SHAPE, "pack_experts: blobs %zu bytes apart hold %zu", dst_stride, (size_t) (l->down_off + db));
+    if (packing == MAYA_PACK_STREAM && ((((uintptr_t) dst | dst_stride | l->gate_off | l->up_off | l->down_off) & 15) ||
+                                        ((l->n_ff | l->n_embd) & 3)))
+        return fail(MAYA_E_ARG, "pack_experts: stream packing wants 16-byte aligned blobs and row arrays, rows in fours");
+    uint8_t* dp = (uint8_t*) dst;
+    const uint8_t* const srcs[3] = {(const uint8_t*) gate_exps, (const uint8_t*) up_exps, (const uint8_t*) down_exps};
+    uint8_t* const dsts[3] = {dp + l->gate_off, dp + l->up_off, dp + l->down_off};
+    const size_t strides[3] = {gb, ub, db};
+    return repack_impl(l, srcs, strides, dsts, dst_stride, n_expert, stream, packing == MAYA_PACK_STREAM ? 0 : 2);
+}
 
 int maya_dequant_rows(int t, const void* w, size_t row_stride, int64_t k, int64_t n_rows, float* out, void* stream) {
     return maya_dequant_rows_packed(t, MAYA_PACK_GGUF, w, row_stride, k, n_rows, out, stream);

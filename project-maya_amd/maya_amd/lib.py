@@ -17,7 +17,7 @@ EXPORTS = [
     "maya_last_error", "maya_device_info", "maya_init", "maya_moe_supported", "maya_moe_block_bytes",
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
-    "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack",
+    "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
     "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
 
@@ -75,6 +75,7 @@ def load():
     L.maya_dequant_rows_packed.argtypes = [i32, i32, vp, sz, i64, i64, vp, vp]
     L.maya_moe_repack.argtypes = [C.POINTER(Layout), vp, vp, vp]
     L.maya_moe_unpack.argtypes = [C.POINTER(Layout), vp, vp, vp]
+    L.maya_moe_pack_experts.argtypes = [C.POINTER(Layout), vp, vp, vp, i32, i32, vp, sz, vp]
     L.maya_quant_act.argtypes = [i32, vp, i32, i64, i32, i64, Act, vp]
     L.maya_quant_i8x32.argtypes = [vp, i32, i64, vp, i32, i64, vp, vp, vp]
     L.maya_moe_route_topk.argtypes = [vp, i32, i32, i32, vp, vp, vp]
@@ -158,6 +159,12 @@ def repack(l, src, dst, stream=None):
 
 def unpack(l, src, dst, stream=None):
     check(load().maya_moe_unpack(C.byref(l), _p(src), _p(dst), _stream(stream)))
+
+
+def pack_experts(l, gate_exps, up_exps, down_exps, n_expert, packing, dst, dst_stride, stream=None):
+    """The layer's blobs (dst_stride bytes apart in dst) from its three stacked GGUF tensors, in `packing` order."""
+    check(load().maya_moe_pack_experts(C.byref(l), _p(gate_exps), _p(up_exps), _p(down_exps), n_expert, packing, _p(dst),
+                                       dst_stride, _stream(stream)))
 
 
 def quant_act(act_type, x, stream=None):

@@ -159,3 +159,51 @@ def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
         want = oracle.dequant_rows(t, blob[off:off + rb * 16], k, 16)
         got = lib.dequant_rows(t, packed[off:], k, 16, packing=1).cpu().numpy()
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("gt,dt,pad", ((22, 22, 0), (22, 12, 64), (12, 12, 0), (8, 8, 32), (19, 29, 0)))
+def test_pack_experts_from_stacked_tensors(lib, gt, dt, pad):
+    """A layer's blobs built on the device from ffn_{gate,up,down}_exps as the file stores them ([expert][rows][row bytes]):
+    GGUF order = the host concatenation gate | up | down of each expert; stream order = maya_moe_repack of that blob."""
+    n_embd, n_ff, ne = 512, 256, 5
+    rng = np.random.default_rng(gt * 7 + dt)
+    blobs = [synth.expert_blob(gt, dt, n_embd, n_ff, rng) for _ in range(ne)]
+    l, nbytes = lib.layout(gt, dt, n_embd, n_ff)
+    gate = np.stack([b[:l.up_off] for b in blobs])
+    up = np.stack([b[l.up_off:l.down_off] for b in blobs])
+    down = np.stack([b[l.down_off:] for b in blobs])
+    stride = nbytes + pad
+    g_d, u_d, d_d = (torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (gate, up, down))
+    for packing in (0, 1):
+        pool = torch.full((ne * stride,), 0xA5, dtype=torch.uint8, device="cuda")
+        lib.pack_experts(l, g_d, u_d, d_d, ne, packing, pool, stride)
+        torch.cuda.synchronize()
+        got = pool.view(ne, stride).cpu().numpy()
+        assert (got[:, nbytes:] == 0xA5).all()          # nothing written between the blobs
+        for e in range(ne):
+            if packing == 0:
+                want = blobs[e]
+            else:
+                w = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+                lib.repack(l, torch.from_numpy(blobs[e]).cuda(), w)
+                want = w.cpu().numpy()
+            assert np.array_equal(got[e, :nbytes], want), (packing, e)
+
+
+def test_pack_experts_refusals(lib):
+    L = lib.load()
+    l, nbytes = lib.layout(22, 22, 512, 256)
+    a = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    dst = torch.full((nbytes + 16,), 7, dtype=torch.uint8, device="cuda")
+    args = lambda **kw: [kw.get("l", l), a.data_ptr(), kw.get("up", a.data_ptr()), a.data_ptr(), kw.get("ne", 1), kw.get("packing", 1),
+                         kw.get("dst", dst.data_ptr()), kw.get("stride", nbytes), lib._stream()]
+    import ctypes as C
+    call = lambda **kw: L.maya_moe_pack_experts(C.byref(args(**kw)[0]), *args(**kw)[1:])
+    assert call(up=None) == 3                       # MAYA_E_ARG
+    assert call(ne=0) == 2                          # MAYA_E_SHAPE
+    assert call(stride=nbytes - 1) == 2
+    assert call(packing=2) == 1                     # MAYA_E_UNSUPPORTED
+    assert call(dst=dst.data_ptr() + 2) == 3        # a stream blob must be 16-byte aligned
+    torch.cuda.synchronize()
+    assert int(dst.min()) == 7 and int(dst.max()) == 7
+    assert call(dst=dst.data_ptr() + 2, packing=0) == 0   # GGUF order takes any alignment
