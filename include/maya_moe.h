@@ -167,6 +167,17 @@ int maya_quant_i8x32(const void* x, int x_dtype, int64_t x_stride, const int32_t
  * double, stable top-k (strict >, lower index on ties) on the float probabilities, renormalised by max(sum, 2^-14). */
 int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights,
                         void* stream);
+/* The sigmoid router of the GLM / DeepSeek-V3 family: strata::kernels::router_sigmoid
+ * (include/strata/kernels/router_sigmoid.hpp:8-31, src/kernels/cuda/router_sigmoid.cu:29-74) and the selection of
+ * glmf::moe_route (include/strata/kernels/glm_fast.hpp:420-433): p = sigmoid(logits) in float, ids = the stable top-k of
+ * p + bias (bias NULL or [n_expert]: it chooses, it does not weigh; ties to the lower index), weights = p / D * w_scale with
+ * D = max(sum of the k chosen p, 2^-14) (norm MAYA_ROUTER_NORM_CLAMP = kRouteNormClamp), sum + 1e-20 (MAYA_ROUTER_NORM_HF =
+ * kRouteNormHf) or 1 (MAYA_ROUTER_NORM_NONE: norm_topk_prob off). */
+#define MAYA_ROUTER_NORM_NONE 0
+#define MAYA_ROUTER_NORM_CLAMP 1
+#define MAYA_ROUTER_NORM_HF 2
+int maya_moe_route_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                           int32_t* ids, float* weights, void* stream);
 /* ids -> plan: plan_ptr[e] = expert_table[ids[e]] (0 stays 0: not resident), the plan part of moe_route_kernel
  * (src/kernels/cuda/glm_fast.cu:3998-4545) without its residency tiers. */
 int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,
@@ -226,6 +237,21 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
                           const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
                           int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes,
                           void* stream);
+/* The same layer with the router named: NULL or kind MAYA_ROUTER_SOFTMAX = maya_moe_route_topk's (router_top10),
+ * MAYA_ROUTER_SIGMOID = maya_moe_route_sigmoid's with this bias, w_scale and norm - the route of glmf::moe_route
+ * (include/strata/kernels/glm_fast.hpp:424-433) in the head's launch. */
+#define MAYA_ROUTER_SOFTMAX 0
+#define MAYA_ROUTER_SIGMOID 1
+typedef struct maya_router {
+    int32_t kind;
+    int32_t norm;        /* sigmoid: MAYA_ROUTER_NORM_* */
+    const float* bias;   /* sigmoid: NULL or [n_expert] */
+    float w_scale;       /* sigmoid: routed_scaling_factor */
+} maya_router;
+int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                                 const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
+                                 float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
+                                 size_t workspace_bytes, void* stream);
 
 /* ============================================================================================= prefill
  * A prompt chunk's routed experts as a grouped GEMM (the reference's expert_count_kernel / expert_scatter_kernel,

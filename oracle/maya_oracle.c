@@ -603,6 +603,58 @@ void mo_router_topk_f64(const float* logits, int n_tokens, int n_expert, int k, 
     router_impl(logits, n_tokens, n_expert, k, ids, weights, 1);
 }
 
+/* The sigmoid router of the GLM / DeepSeek-V3 family (noaux_tc): p = sigmoid(logit), the bias enters the SELECTION only,
+ * stable top-k (ties to the lower index), w = p / max(sum, 2^-14) * w_scale (norm 1; norm 2: / (sum + 1e-20); norm 0: no
+ * division).  f64 = 0: the device arithmetic of src/kernels/cuda/router_sigmoid.cu:44-73 and moe_route_kernel
+ * (src/kernels/cuda/glm_fast.cu:4050-4056, 4214, 4297): p and p + bias in float, rank = the experts that beat e (a larger
+ * score, or an equal one at a lower index), the selected p summed in rank order in double, inv a float,
+ * w = (float)((double) p * inv * w_scale).  f64 = 1: the host form of src/kernels/router_sigmoid_parity.cpp:36-86
+ * (double sigmoid and scores, stable sort). */
+static void router_sigmoid_impl(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                                int32_t* ids, float* weights, int f64) {
+    double* pd = (double*) malloc(sizeof(double) * (size_t) n_expert);
+    double* sd = (double*) malloc(sizeof(double) * (size_t) n_expert);
+    float* p = (float*) malloc(sizeof(float) * (size_t) n_expert);
+    float* sel = (float*) malloc(sizeof(float) * (size_t) n_expert);
+    for (int t = 0; t < n_tokens; ++t) {
+        const float* l = logits + (size_t) t * n_expert;
+        for (int e = 0; e < n_expert; ++e) {
+            p[e] = 1.0f / (1.0f + expf(-l[e]));
+            sel[e] = bias ? p[e] + bias[e] : p[e];
+            pd[e] = 1.0 / (1.0 + exp(-(double) l[e]));
+            sd[e] = bias ? pd[e] + (double) bias[e] : pd[e];
+        }
+        for (int e = 0; e < n_expert; ++e) {
+            int rank = 0;
+            for (int f = 0; f < n_expert; ++f) {
+                if (f64) rank += (sd[f] > sd[e]) || (f < e && sd[f] == sd[e]);
+                else rank += (sel[f] > sel[e]) || (f < e && sel[f] == sel[e]);
+            }
+            if (rank < k) ids[(size_t) t * k + rank] = e;
+        }
+        double sum = 0.0;
+        for (int i = 0; i < k; ++i) sum += f64 ? pd[ids[(size_t) t * k + i]] : (double) p[ids[(size_t) t * k + i]];
+        const double invd = norm == 0 ? 1.0 : norm == 2 ? 1.0 / (sum + 1e-20) : 1.0 / fmax(sum, 6.103515625e-05);
+        const float inv = (float) invd;
+        for (int i = 0; i < k; ++i) {
+            const int e = ids[(size_t) t * k + i];
+            weights[(size_t) t * k + i] = f64 ? (float) (pd[e] * invd * (double) w_scale) : (float) ((double) p[e] * inv * w_scale);
+        }
+    }
+    free(pd);
+    free(sd);
+    free(p);
+    free(sel);
+}
+void mo_router_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                       int32_t* ids, float* weights) {
+    router_sigmoid_impl(logits, bias, n_tokens, n_expert, k, w_scale, norm, ids, weights, 0);
+}
+void mo_router_sigmoid_f64(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                           int32_t* ids, float* weights) {
+    router_sigmoid_impl(logits, bias, n_tokens, n_expert, k, w_scale, norm, ids, weights, 1);
+}
+
 /* src/kernels/cuda/native_moe.cu:36-52: sum = parts[0]*w[0]; sum += parts[i]*w[i] ... (each product and add rounded) */
 void mo_combine(const float* parts, const float* w, int k, int64_t n, float* out) {
     for (int64_t c = 0; c < n; ++c) {

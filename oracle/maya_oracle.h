@@ -26,6 +26,10 @@
  *   IQ2_S expert in device arithmetic  reference build: strata::ds4::par::gate_up_ref / down_ref, bit-exact
  *   SwiGLU ........................... closed form; exp_portable (ds4_par_exp.h:60-85) bit-exact against the reference build
  *   router top-k ..................... closed forms (all-equal logits, ties), float-p vs double-p cross-check
+ *   sigmoid router ................... the reference's host form (router_sigmoid_parity.cpp:36-86, restated in double with a
+ *                                       stable sort) on its own four case shapes incl. exact ties, to its tolerance (ids
+ *                                       equal, weights 1e-5); closed forms (equal logits, a bias that selects but does not
+ *                                       weigh, sum of weights = w_scale); the wrong readings the reference names must differ
  *   combine .......................... closed form
  *   EXL3 states / codebook ........... the reference's own golden vectors data/exl3-exllamav3 (13 .bin files made by exllamav3)
  *   EXL3 mat-vec ..................... reference build: exl3_ref.cpp bit-exact; H.H = I
@@ -114,6 +118,12 @@ void mo_expert(int gu_type, int d_type, const uint8_t* gate, const uint8_t* up, 
 /* ---- router (src/kernels/cuda/router_top10.cu:95-186; host form src/kernels/router_top10_parity.cpp:36-60) */
 void mo_router_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights);
 void mo_router_topk_f64(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights);
+/* ---- the sigmoid router (src/kernels/cuda/router_sigmoid.cu:44-73, moe_route_kernel src/kernels/cuda/glm_fast.cu:4050-4297;
+ * host form src/kernels/router_sigmoid_parity.cpp:36-86).  norm: 0 none, 1 / max(sum, 2^-14), 2 / (sum + 1e-20) */
+void mo_router_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                       int32_t* ids, float* weights);
+void mo_router_sigmoid_f64(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                           int32_t* ids, float* weights);
 
 /* ---- combine (src/kernels/cuda/native_moe.cu:36-52): out[c] = sum_i w[i] * parts[i][c] in order i = 0..k-1 */
 void mo_combine(const float* parts, const float* w, int k, int64_t n, float* out);

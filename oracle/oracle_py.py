@@ -215,6 +215,19 @@ def router_topk(logits, k, f64=False):
     return ids, w
 
 
+def router_sigmoid(logits, bias, k, w_scale=1.0, norm=1, f64=False):
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    nt, ne = logits.shape
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    ids = np.zeros((nt, k), dtype=np.int32)
+    w = np.zeros((nt, k), dtype=np.float32)
+    f = lib().mo_router_sigmoid_f64 if f64 else lib().mo_router_sigmoid
+    f.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p, C.c_void_p]
+    f.restype = None
+    f(_ptr(logits), None if b is None else _ptr(b), nt, ne, k, w_scale, norm, _ptr(ids), _ptr(w))
+    return ids, w
+
+
 def combine(parts, w):
     parts = np.ascontiguousarray(parts, dtype=np.float32)
     w = np.ascontiguousarray(w, dtype=np.float32)

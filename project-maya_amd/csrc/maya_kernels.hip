@@ -539,6 +539,44 @@ __device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm)
     }
 }
 
+// The k largest of n_expert 64-bit keys (a value's ordered bits above the complemented index, so "beats" is one unsigned
+// compare and equal values rank by the lower index) into sm.id / sm.w (= sm.p of the expert), 256 threads.  Ranking every
+// expert against every other grows with the square.  The k-th largest of the threads' best keys is a lower bound of the
+// k-th largest key overall (those are k different experts), so only keys at or above it can be among the k largest, and
+// every key that beats one of them is at or above it too: the few candidates (at most k threads' experts) are ranked
+// among themselves.
+__device__ __forceinline__ void topk_by_keys(const unsigned long long* key, int n_expert, int k, RouterLds& sm) {
+    const int tid = threadIdx.x;
+    unsigned long long best = 0ull;
+    for (int e = tid; e < n_expert; e += 256) best = key[e] > best ? key[e] : best;
+    sm.lb[tid] = best;
+    if (tid == 0) sm.nc = 0;
+    __syncthreads();
+    int rank = 0;
+    for (int j = 0; j < 256; j += 2) {
+        const ulonglong2 kj = *(const ulonglong2*) (sm.lb + j);
+        rank += kj.x > best ? 1 : 0;
+        rank += kj.y > best ? 1 : 0;
+    }
+    if (rank == k - 1) sm.thr = best;
+    __syncthreads();
+    const unsigned long long thr = sm.thr;
+    for (int e = tid; e < n_expert; e += 256)
+        if (key[e] >= thr) sm.cand[atomicAdd(&sm.nc, 1)] = key[e];
+    __syncthreads();
+    const int nc = sm.nc;
+    if (tid < nc) {
+        const unsigned long long kc = sm.cand[tid];
+        int r = 0;
+        for (int j = 0; j < nc; ++j) r += sm.cand[j] > kc ? 1 : 0;
+        if (r < k) {
+            const int e = (int) (0xffffffffu - (unsigned) (kc & 0xffffffffull));
+            sm.id[r] = e;
+            sm.w[r] = sm.p[e];
+        }
+    }
+}
+
 // 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights
 __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
     const int tid = threadIdx.x;
@@ -604,40 +642,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     for (int e = tid; e < n_expert; e += 256)
         key[e] = ((unsigned long long) __float_as_uint(sm.p[e]) << 32) | (unsigned long long) (0xffffffffu - (unsigned) e);
     __syncthreads();
-    {
-        // Ranking every expert against every other grows with the square.  The k-th largest of the
-        // threads' best keys is a lower bound of the k-th largest key overall (those are k different experts), so only keys
-        // at or above it can be among the k largest, and every key that beats one of them is at or above it too: the few
-        // candidates (at most k threads' experts) are ranked among themselves.
-        unsigned long long best = 0ull;
-        for (int e = tid; e < n_expert; e += 256) best = key[e] > best ? key[e] : best;
-        sm.lb[tid] = best;
-        if (tid == 0) sm.nc = 0;
-        __syncthreads();
-        int rank = 0;
-        for (int j = 0; j < 256; j += 2) {
-            const ulonglong2 kj = *(const ulonglong2*) (sm.lb + j);
-            rank += kj.x > best ? 1 : 0;
-            rank += kj.y > best ? 1 : 0;
-        }
-        if (rank == k - 1) sm.thr = best;
-        __syncthreads();
-        const unsigned long long thr = sm.thr;
-        for (int e = tid; e < n_expert; e += 256)
-            if (key[e] >= thr) sm.cand[atomicAdd(&sm.nc, 1)] = key[e];
-        __syncthreads();
-        const int nc = sm.nc;
-        if (tid < nc) {
-            const unsigned long long kc = sm.cand[tid];
-            int r = 0;
-            for (int j = 0; j < nc; ++j) r += sm.cand[j] > kc ? 1 : 0;
-            if (r < k) {
-                const int e = (int) (0xffffffffu - (unsigned) (kc & 0xffffffffull));
-                sm.id[r] = e;
-                sm.w[r] = sm.p[e];
-            }
-        }
-    }
+    topk_by_keys(key, n_expert, k, sm);
     __syncthreads();
     if (tid < 64) {
         // renormalisation: the sum of the k weights in slot order in double, one division a lane
@@ -650,11 +655,92 @@ __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_e
     __syncthreads();
 }
 
-__global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k,
+// ---- the sigmoid router of the GLM / DeepSeek-V3 family (src/kernels/cuda/router_sigmoid.cu:44-73; moe_route_kernel,
+// src/kernels/cuda/glm_fast.cu:4050-4056, 4214, 4297): p = 1 / (1 + expf(-logit)) in float, the selection score p + bias
+// (the bias chooses, it does not weigh), stable top-k, the chosen p summed in rank order in double,
+// w = (float)((double) p * inv * w_scale) with inv a float: 1 / max(sum, 2^-14) (norm 1), 1 / (sum + 1e-20) (norm 2), 1.
+struct RouterSpec {
+    const float* bias;   // [n_expert] or null (sigmoid only)
+    float w_scale;
+    int kind;            // MAYA_ROUTER_SOFTMAX, MAYA_ROUTER_SIGMOID
+    int norm;
+};
+// a float's bits as a signed integer that orders like the float (no -0.0 arises: p > 0 and p + bias = 0 rounds to +0.0)
+__device__ __forceinline__ int float_order_key(float v) {
+    const int b = __float_as_int(v);
+    return b >= 0 ? b : b ^ 0x7fffffff;
+}
+// one wave, up to 256 experts, sm.p and the scores (sm.ex's storage, as floats) filled; on return lane i < k holds slot i
+__device__ __forceinline__ void sigmoid_narrow(int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
+    const int lane = threadIdx.x;
+    const float* sel = (const float*) sm.ex;
+    constexpr int kNone = (int) 0x80000000;   // below every key: a taken expert, or none at this index
+    int key[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) key[q] = 64 * q + lane < n_expert ? float_order_key(sel[64 * q + lane]) : kNone;
+    int my_id = 0;
+    for (int i = 0; i < k; ++i) {
+        const int top = wave_max_i32(max(max(key[0], key[1]), max(key[2], key[3])));
+        unsigned long long b = __ballot(key[0] == top);
+        int q = 0;
+        if (b == 0ull) b = __ballot(key[1] == top), q = 1;
+        if (b == 0ull) b = __ballot(key[2] == top), q = 2;
+        if (b == 0ull) b = __ballot(key[3] == top), q = 3;
+        const int at = __builtin_ctzll(b);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) key[j] = (j == q && lane == at) ? kNone : key[j];
+        if (lane == i) my_id = 64 * q + at;
+    }
+    if (lane < k) sm.id[lane] = my_id;
+}
+// 256 threads; on return sm.id / sm.w hold the token's k experts and weights
+__device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l, int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
+    const int tid = threadIdx.x;
+    float* sel = (float*) sm.ex;
+    for (int e = tid; e < n_expert; e += 256) {
+        const float p = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-l[e])));
+        sm.p[e] = p;
+        sel[e] = r.bias ? __fadd_rn(p, r.bias[e]) : p;
+    }
+    __syncthreads();
+    if (n_expert <= 256) {
+        if (tid < 64) sigmoid_narrow(n_expert, k, r, sm);
+    } else {
+        // (the scores' ordered bits, offset to unsigned, above the complemented index; the keys take the scores' place)
+        float v[MAYA_MAX_EXPERTS / 256];
+#pragma unroll
+        for (int i = 0; i < MAYA_MAX_EXPERTS / 256; ++i) v[i] = tid + 256 * i < n_expert ? sel[tid + 256 * i] : 0.0f;
+        __syncthreads();
+        unsigned long long* key = (unsigned long long*) sm.ex;
+#pragma unroll
+        for (int i = 0; i < MAYA_MAX_EXPERTS / 256; ++i) {
+            const int e = tid + 256 * i;
+            if (e < n_expert)
+                key[e] = ((unsigned long long) ((unsigned) float_order_key(v[i]) ^ 0x80000000u) << 32) | (unsigned long long) (0xffffffffu - (unsigned) e);
+        }
+        __syncthreads();
+        topk_by_keys(key, n_expert, k, sm);
+    }
+    __syncthreads();
+    if (tid < 64) {
+        const float p = tid < k ? sm.p[sm.id[tid]] : 0.0f;
+        double s = 0.0;
+        for (int i = 0; i < k; ++i) s += (double) __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
+        const float inv = (float) (r.norm == 0 ? 1.0 : r.norm == 2 ? 1.0 / (s + 1e-20) : 1.0 / fmax(s, 6.103515625e-05));
+        if (tid < k) sm.w[tid] = (float) ((double) p * (double) inv * (double) r.w_scale);
+    }
+    __syncthreads();
+}
+__device__ __forceinline__ void route_any(const float* __restrict__ l, int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
+    if (r.kind == MAYA_ROUTER_SIGMOID) route_token_sigmoid(l, n_expert, k, r, sm);
+    else route_token(l, n_expert, k, sm);
+}
+
+__global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec r,
                                                      int32_t* __restrict__ ids, float* __restrict__ weights) {
     __shared__ RouterLds sm;
     const int t = blockIdx.x;
-    route_token(logits + (size_t) t * n_expert, n_expert, k, sm);
+    route_any(logits + (size_t) t * n_expert, n_expert, k, r, sm);
     if (threadIdx.x < k) {
         ids[(size_t) t * k + threadIdx.x] = sm.id[threadIdx.x];
         weights[(size_t) t * k + threadIdx.x] = sm.w[threadIdx.x];
@@ -665,7 +751,7 @@ __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ l
 // plan slots (blob addresses from the residency table) and - for token 0 - clears the gate/up kernels' arrival
 // counters; the other workgroups round one 256-value block of the hidden state each to Q8_K.
 template <int DT>
-__global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict__ logits, int n_expert, int k,
+__global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec rs,
                                                          const uint64_t* __restrict__ table, int32_t* __restrict__ ids,
                                                          float* __restrict__ weights, uint64_t* __restrict__ plan,
                                                          const void* __restrict__ x, int64_t n_embd, maya_act xq,
@@ -685,7 +771,7 @@ __global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict
             const int e = threadIdx.x + 256 * i;
             tab[i] = e < n_expert ? table[e] : 0ull;
         }
-        route_token(logits + (size_t) t * n_expert, n_expert, k, sm);
+        route_any(logits + (size_t) t * n_expert, n_expert, k, rs, sm);
 #pragma unroll
         for (int i = 0; i < MAYA_MAX_EXPERTS / 256; ++i) s_table[threadIdx.x + 256 * i] = tab[i];
         __syncthreads();
@@ -1652,17 +1738,36 @@ int maya_quant_i8x32(const void* x, int x_dtype, int64_t x_stride, const int32_t
     return MAYA_OK;
 }
 
-int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights,
-                        void* stream) {
+static int route_impl(const char* what, const float* logits, int n_tokens, int n_expert, int k, const RouterSpec& r, int32_t* ids,
+                      float* weights, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (!logits || !ids || !weights) return fail(MAYA_E_ARG, "route_topk: null pointer");
+    if (!logits || !ids || !weights) return fail(MAYA_E_ARG, "%s: null pointer", what);
     if (n_tokens <= 0 || n_tokens > 65535 || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k <= 0 || k > MAYA_MAX_K || k > n_expert)
-        return fail(MAYA_E_SHAPE, "route_topk: tokens %d experts %d k %d (limits %d experts, k %d)", n_tokens, n_expert, k,
+        return fail(MAYA_E_SHAPE, "%s: tokens %d experts %d k %d (limits %d experts, k %d)", what, n_tokens, n_expert, k,
                     MAYA_MAX_EXPERTS, MAYA_MAX_K);
-    hipLaunchKernelGGL(router_kernel, dim3((unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, ids, weights);
+    hipLaunchKernelGGL(router_kernel, dim3((unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, r, ids, weights);
     MAYA_LAUNCHED("router_kernel");
     return MAYA_OK;
+}
+static bool router_spec(const maya_router* r, RouterSpec& s) {
+    s = RouterSpec{nullptr, 1.0f, MAYA_ROUTER_SOFTMAX, 1};
+    if (!r) return true;
+    if (r->kind != MAYA_ROUTER_SOFTMAX && r->kind != MAYA_ROUTER_SIGMOID) return false;
+    if (r->kind == MAYA_ROUTER_SIGMOID) {
+        if (r->norm < 0 || r->norm > 2) return false;
+        s = RouterSpec{r->bias, r->w_scale, MAYA_ROUTER_SIGMOID, r->norm};
+    }
+    return true;
+}
+int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights,
+                        void* stream) {
+    return route_impl("route_topk", logits, n_tokens, n_expert, k, RouterSpec{nullptr, 1.0f, MAYA_ROUTER_SOFTMAX, 1}, ids, weights, stream);
+}
+int maya_moe_route_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
+                           int32_t* ids, float* weights, void* stream) {
+    if (norm < 0 || norm > 2) return fail(MAYA_E_UNSUPPORTED, "route_sigmoid: normalisation %d", norm);
+    return route_impl("route_sigmoid", logits, n_tokens, n_expert, k, RouterSpec{bias, w_scale, MAYA_ROUTER_SIGMOID, norm}, ids, weights, stream);
 }
 
 int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,
@@ -1848,9 +1953,17 @@ size_t maya_moe_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k) {
 int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
                           const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
                           float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    return maya_moe_layer_decode_routed(l, expert_table, n_expert, k, nullptr, logits, x, x_dtype, n_tokens, limit, add, ids, weights,
+                                        out, workspace, workspace_bytes, stream);
+}
+int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                                 const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                                 int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (!l) return fail(MAYA_E_ARG, "layer_decode: null layout");
+    RouterSpec rs;
+    if (!router_spec(router, rs)) return fail(MAYA_E_UNSUPPORTED, "layer_decode: router kind %d / normalisation %d", router->kind, router->norm);
     if (const int rc = check_layout(*l)) return rc;
     if (!expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "layer_decode: null pointer");
     if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K)
@@ -1879,14 +1992,14 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
         hipStream_t s = as_stream(stream);
         if (k > n_expert) return fail(MAYA_E_SHAPE, "layer_decode: k %d > n_expert %d", k, n_expert);
         switch (x_dtype) {
-            case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
-            case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
-            default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
         }
         MAYA_LAUNCHED("layer_head_kernel");
         a.hq_sync = down_rounds_h(a) ? nullptr : w.hq_sync;   // (the down kernel's own rounding of h is the cheaper one)
     } else {
-        if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+        if ((rc = route_impl("layer_decode", logits, n_tokens, n_expert, k, rs, ids, weights, stream))) return rc;
         if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }

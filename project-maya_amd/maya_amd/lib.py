@@ -18,14 +18,23 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
+    "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed",
     "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
+
+
+ROUTER_SOFTMAX, ROUTER_SIGMOID = 0, 1
+NORM_NONE, NORM_CLAMP, NORM_HF = 0, 1, 2
 
 
 class MayaError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__("maya_moe status %d: %s" % (code, msg))
         self.code = code
+
+
+class Router(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("norm", C.c_int32), ("bias", C.c_void_p), ("w_scale", C.c_float)]
 
 
 class Layout(C.Structure):
@@ -90,6 +99,9 @@ def load():
     L.maya_moe_workspace_bytes.restype = sz
     L.maya_moe_workspace_bytes.argtypes = [C.POINTER(Layout), i32, i32]
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
+    L.maya_moe_layer_decode_routed.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32, vp, vp, vp,
+                                               vp, vp, sz, vp]
+    L.maya_moe_route_sigmoid.argtypes = [vp, vp, i32, i32, i32, f32, i32, vp, vp, vp]
     _lib = L
     return L
 
@@ -193,6 +205,15 @@ def route_topk(logits, k, stream=None):
     return ids, w
 
 
+def route_sigmoid(logits, bias, k, w_scale=1.0, norm=NORM_CLAMP, stream=None):
+    assert logits.is_contiguous() and logits.dtype == torch.float32 and logits.dim() == 2
+    nt, ne = logits.shape
+    ids = torch.empty((nt, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((nt, k), dtype=torch.float32, device=logits.device)
+    check(load().maya_moe_route_sigmoid(_p(logits), _p(bias), nt, ne, k, w_scale, norm, _p(ids), _p(w), _stream(stream)))
+    return ids, w
+
+
 def plan(ids, expert_table, stream=None):
     out = torch.empty(ids.numel(), dtype=torch.int64, device=ids.device)
     check(load().maya_moe_plan(_p(ids), ids.numel(), _p(expert_table), expert_table.numel(), _p(out), _stream(stream)))
@@ -261,9 +282,15 @@ class MoeLayer:
         self.weights = torch.empty((max_tokens, k), dtype=torch.float32, device=device)
         self.out = torch.empty((max_tokens, n_embd), dtype=torch.float32, device=device)
 
-    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None):
+    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None):
+        """router: None (the softmax router) or a Router (kind, norm, bias pointer, w_scale)."""
         nt = x.shape[0]
         assert nt <= self.max_tokens and x.is_contiguous() and logits.is_contiguous()
+        if router is not None:
+            check(load().maya_moe_layer_decode_routed(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, C.byref(router),
+                                                      _p(logits), _p(x), dtype_id(x), nt, limit, _p(add), _p(self.ids),
+                                                      _p(self.weights), _p(self.out), _p(self.ws), self.ws_bytes, _stream(stream)))
+            return self.out[:nt]
         check(load().maya_moe_layer_decode(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, _p(logits), _p(x),
                                            dtype_id(x), nt, limit, _p(add), _p(self.ids), _p(self.weights), _p(self.out),
                                            _p(self.ws), self.ws_bytes, _stream(stream)))

@@ -22,11 +22,11 @@ def make_experts(gate_type, down_type, n_embd, n_ff, n_expert, seed, up_type=Non
 
 
 def oracle_layer(oracle, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x, limit=float("inf"), up_type=None,
-                 skip=()):
+                 skip=(), route=None):
     """The reference CPU path on the host: router, each routed expert (ggml contract), weighted sum in slot order.
     `skip`: expert ids whose blob is not resident (their part is left out).  Returns ids, weights, out, h."""
     up_type = gate_type if up_type is None else up_type
-    ids, w = oracle.router_topk(logits, k)
+    ids, w = route(logits, k) if route else oracle.router_topk(logits, k)
     up_off, down_off, _ = synth.blob_offsets(gate_type, down_type, n_embd, n_ff, up_type)
     nt = x.shape[0]
     out = np.zeros((nt, n_embd), dtype=np.float32)

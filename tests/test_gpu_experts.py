@@ -19,7 +19,7 @@ def lib():
 
 
 def run_layer(lib, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x, limit=float("inf"), up_type=None,
-              misalign=0, add=None, resident=None, packing=0):
+              misalign=0, add=None, resident=None, packing=0, router=None):
     gguf_layout, _ = lib.layout(gate_type, down_type, n_embd, n_ff, up_type)
     store = lib.ExpertStore(blobs, misalign=misalign, pack_layout=gguf_layout if packing else None)
     table = store.table
@@ -31,7 +31,7 @@ def run_layer(lib, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x, limi
     layer = lib.MoeLayer(gate_type, down_type, n_embd, n_ff, len(blobs), k, max_tokens=x.shape[0], up_type=up_type,
                          packing=packing)
     out = layer.forward(table, dev(logits), x if torch.is_tensor(x) else dev(x), limit=limit,
-                        add=None if add is None else dev(add))
+                        add=None if add is None else dev(add), router=router)
     torch.cuda.synchronize()
     return layer.ids.cpu().numpy(), layer.weights.cpu().numpy(), out.cpu().numpy(), store
 
@@ -88,6 +88,29 @@ def test_layer_matches_cpu_path(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt, pa
     ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=packing)
     wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x)
     assert np.array_equal(ids, wi)
+    for t in range(nt):
+        assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
+
+
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt,packing,norm", (
+    (22, 22, 7168, 2048, 9, 8, 1, 1, 1), (22, 22, 1024, 512, 16, 4, 3, 0, 2), (12, 12, 4096, 2048, 6, 4, 2, 1, 1),
+    (8, 8, 512, 256, 8, 2, 1, 0, 0), (22, 12, 1024, 768, 300, 8, 2, 0, 1)))
+def test_layer_with_the_sigmoid_router(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt, packing, norm):
+    """The layer's head routes as router_sigmoid / moe_route do (a selection bias, a scaling factor): ids bit-exact, weights
+    1e-5, the layer against the CPU path's experts combined with those weights."""
+    seed = gt * 1000 + dt * 10 + nt + 7
+    blobs = make_experts(gt, dt, n_embd, n_ff, min(ne, 12), seed)
+    blobs = [blobs[i % len(blobs)] for i in range(ne)]   # (many experts: the same few blobs again)
+    rng = np.random.default_rng(seed + 1)
+    logits = (rng.standard_normal((nt, ne)) * 2).astype(np.float32)
+    bias = (rng.standard_normal(ne) * 0.1).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    bias_d = dev(bias)
+    router = lib.Router(lib.ROUTER_SIGMOID, norm, bias_d.data_ptr(), 2.5)
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=packing, router=router)
+    wi, ww, wout = oracle_layer(oracle, gt, dt, blobs, k, n_embd, n_ff, logits, x,
+                                route=lambda l, kk: oracle.router_sigmoid(l, bias, kk, 2.5, norm))
+    assert np.array_equal(ids, wi) and np.max(np.abs(w - ww)) < 1e-5
     for t in range(nt):
         assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
 

@@ -96,3 +96,52 @@ def test_plan_and_group(lib):
             assert list(ge[start:start + len(members[b])]) == members[b]
             start += len(members[b])
         assert gs[len(order)] == start
+
+
+# ---- the sigmoid router (router_sigmoid / moe_route's selection): ids bit-exact with the CPU checker, weights to the
+# reference's bar of 1e-5 (src/kernels/router_sigmoid_parity.cpp:137-143), on that test's case shapes and wider ones
+
+from test_oracle_formats import SIGMOID_CASES, sigmoid_case
+
+
+def _check_sigmoid(lib, oracle, logits, bias, k, w_scale, norm):
+    b = None if bias is None else torch.from_numpy(bias).cuda()
+    ids, w = lib.route_sigmoid(torch.from_numpy(logits).cuda(), b, k, w_scale, norm)
+    wi, ww = oracle.router_sigmoid(logits, bias, k, w_scale, norm)
+    assert np.array_equal(ids.cpu().numpy(), wi)
+    assert np.max(np.abs(w.cpu().numpy() - ww)) < 1e-5
+    return ids.cpu().numpy(), w.cpu().numpy()
+
+
+@pytest.mark.parametrize("nt,ne,k,w_scale,norm_w,with_bias,quantize,seed", SIGMOID_CASES + [
+    (8, 1024, 8, 2.5, True, True, False, 21), (5, 1000, 16, 1.0, True, True, True, 22), (64, 256, 8, 2.5, True, True, False, 23),
+    (3, 8, 8, 1.0, True, False, False, 24), (7, 160, 6, 1.5, True, True, True, 25)])
+def test_sigmoid_router(lib, oracle, nt, ne, k, w_scale, norm_w, with_bias, quantize, seed):
+    logits, bias = sigmoid_case(nt, ne, with_bias, quantize, seed)
+    _check_sigmoid(lib, oracle, logits, bias, k, w_scale, 1 if norm_w else 0)
+    _check_sigmoid(lib, oracle, logits, bias, k, w_scale, 2)
+
+
+def test_sigmoid_router_ties_bias_and_tiny_sums(lib, oracle):
+    ne, k = 256, 8
+    logits = np.full((2, ne), 0.3, dtype=np.float32)
+    ids, w = _check_sigmoid(lib, oracle, logits, None, k, 2.5, 1)
+    assert np.array_equal(ids, np.tile(np.arange(k, dtype=np.int32), (2, 1))) and np.allclose(w, 2.5 / k, rtol=1e-6)
+    # a negative selection score and a bias that selects an expert whose weight stays its small unbiased p
+    logits = np.linspace(-3.0, -1.0, ne, dtype=np.float32)[None, :].copy()
+    bias = np.full(ne, -0.5, dtype=np.float32)      # every score negative: the order must still be the floats' order
+    bias[17] = 5.0
+    ids, w = _check_sigmoid(lib, oracle, logits, bias, k, 1.0, 0)
+    assert ids[0, 0] == 17 and np.array_equal(ids[0, 1:], np.arange(ne - 1, ne - k, -1))
+    assert abs(w[0, 0] - 1.0 / (1.0 + np.exp(-float(logits[0, 17])))) < 1e-6
+    # all sigmoids tiny: the clamp and the HF form part
+    logits = np.full((1, ne), -30.0, dtype=np.float32)
+    _, w1 = _check_sigmoid(lib, oracle, logits, None, k, 1.0, 1)
+    _, w2 = _check_sigmoid(lib, oracle, logits, None, k, 1.0, 2)
+    assert np.allclose(w2, 1.0 / k, rtol=1e-5) and float(w1.max()) < 1e-8
+    L = lib.load()
+    assert L.maya_moe_route_sigmoid(0, 0, 1, 8, 8, 1.0, 1, 0, 0, 0) == 3       # MAYA_E_ARG
+    x = torch.zeros((1, 8), device="cuda")
+    o = torch.zeros((1, 8), device="cuda")
+    assert L.maya_moe_route_sigmoid(x.data_ptr(), 0, 1, 8, 8, 1.0, 3, o.data_ptr(), o.data_ptr(), 0) == 1   # MAYA_E_UNSUPPORTED
+    assert L.maya_moe_route_sigmoid(x.data_ptr(), 0, 1, 8, 9, 1.0, 1, o.data_ptr(), o.data_ptr(), 0) == 2   # k > experts

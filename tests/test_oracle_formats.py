@@ -226,3 +226,91 @@ def test_float_and_double_selection_agree(oracle):
     a, _ = oracle.router_topk(logits, 8)
     b, _ = oracle.router_topk(logits, 8, f64=True)
     assert np.array_equal(a, b)
+
+
+# ---- the sigmoid router: the device arithmetic against the reference's host form (router_sigmoid_parity.cpp:36-86) restated
+# here in double with a stable sort, on that test's own case shapes, to its bars (ids equal, weights 1e-5; :137-143)
+
+def _ref_router_sigmoid(logits, bias, k, w_scale, norm_w, softmax=False, biased_weights=False, no_renorm=False, no_scale=False):
+    nt, ne = logits.shape
+    ids = np.zeros((nt, k), dtype=np.int32)
+    w = np.zeros((nt, k), dtype=np.float32)
+    for t in range(nt):
+        x = logits[t].astype(np.float64)
+        if softmax:
+            p = np.exp(x - x.max())
+            p /= p.sum()
+        else:
+            p = 1.0 / (1.0 + np.exp(-x))
+        score = p + (bias.astype(np.float64) if bias is not None else 0.0)
+        order = np.argsort(-score, kind="stable")[:k]
+        ids[t] = order
+        wf = p[order].astype(np.float32)
+        s = p[order].sum()
+        for i in range(k):
+            v = float(wf[i]) + (float(bias[order[i]]) if (biased_weights and bias is not None) else 0.0)
+            if norm_w and not no_renorm:
+                v /= max(s, 6.103515625e-5)
+            if not no_scale:
+                v *= w_scale
+            w[t, i] = np.float32(v)
+    return ids, w
+
+
+SIGMOID_CASES = [(4, 32, 8, 2.5, True, True, False, 11), (1, 288, 8, 2.5, True, True, False, 12),
+                 (4, 32, 8, 2.5, True, True, True, 13), (4, 32, 8, 1.0, False, False, False, 14),
+                 (16, 256, 8, 2.5, True, True, False, 15), (3, 384, 6, 1.0, True, True, True, 16)]
+
+
+def sigmoid_case(nt, ne, with_bias, quantize, seed):
+    rng = np.random.default_rng(seed)
+    logits = (rng.standard_normal((nt, ne)) * 2.0).astype(np.float32)
+    bias = (rng.standard_normal(ne) * 0.1).astype(np.float32) if with_bias else None
+    if quantize:   # exact selection-score ties on purpose
+        logits = (np.round(logits * 4) / 4).astype(np.float32)
+        if bias is not None:
+            bias = (np.round(bias * 4) / 4).astype(np.float32)
+    return logits, bias
+
+
+@pytest.mark.parametrize("nt,ne,k,w_scale,norm_w,with_bias,quantize,seed", SIGMOID_CASES)
+def test_sigmoid_router_against_the_reference_host_form(oracle, nt, ne, k, w_scale, norm_w, with_bias, quantize, seed):
+    logits, bias = sigmoid_case(nt, ne, with_bias, quantize, seed)
+    ids, w = oracle.router_sigmoid(logits, bias, k, w_scale, 1 if norm_w else 0)
+    rid, rw = _ref_router_sigmoid(logits, bias, k, w_scale, norm_w)
+    assert np.array_equal(ids, rid)
+    assert np.max(np.abs(w - rw)) < 1e-5
+    i64, w64 = oracle.router_sigmoid(logits, bias, k, w_scale, 1 if norm_w else 0, f64=True)
+    assert np.array_equal(i64, rid) and np.max(np.abs(w64 - rw)) < 1e-6
+    # the wrong readings the reference names must differ materially (:147-160)
+    if with_bias and not quantize:
+        assert np.max(np.abs(w - _ref_router_sigmoid(logits, bias, k, w_scale, norm_w, biased_weights=True)[1])) > 1e-3
+    assert np.max(np.abs(w - _ref_router_sigmoid(logits, bias, k, w_scale, norm_w, softmax=True)[1])) > 1e-2
+    if norm_w:
+        assert np.max(np.abs(w - _ref_router_sigmoid(logits, bias, k, w_scale, norm_w, no_renorm=True)[1])) > 1e-2
+    if w_scale != 1.0:
+        assert np.max(np.abs(w - _ref_router_sigmoid(logits, bias, k, w_scale, norm_w, no_scale=True)[1])) > 1e-2
+
+
+def test_sigmoid_router_closed_forms(oracle):
+    ne, k = 64, 8
+    logits = np.full((2, ne), 0.3, dtype=np.float32)
+    ids, w = oracle.router_sigmoid(logits, None, k, 2.5, 1)
+    assert np.array_equal(ids, np.tile(np.arange(k, dtype=np.int32), (2, 1)))          # a pure tie: the lower indices
+    assert np.allclose(w, 2.5 / k, rtol=1e-6)
+    # the bias selects but does not weigh: expert 40 has the smallest p and a large bias
+    logits = np.linspace(1.0, 2.0, ne, dtype=np.float32)[None, :].copy()
+    logits[0, 40] = -6.0
+    bias = np.zeros(ne, dtype=np.float32)
+    bias[40] = 5.0
+    ids, w = oracle.router_sigmoid(logits, bias, k, 1.0, 0)
+    assert ids[0, 0] == 40 and abs(w[0, 0] - 1.0 / (1.0 + np.exp(6.0))) < 1e-7
+    assert np.array_equal(ids[0, 1:], np.arange(ne - 1, ne - k, -1))
+    ids, w = oracle.router_sigmoid(logits, bias, k, 2.5, 1)
+    assert abs(float(w.sum()) - 2.5) < 1e-5                                              # normalised, then scaled
+    # all sigmoids tiny: the two normalisations part (max(sum, 2^-14) against sum + 1e-20)
+    logits = np.full((1, ne), -30.0, dtype=np.float32)
+    _, w1 = oracle.router_sigmoid(logits, None, k, 1.0, 1)
+    _, w2 = oracle.router_sigmoid(logits, None, k, 1.0, 2)
+    p = 1.0 / (1.0 + np.exp(30.0))
+    assert np.allclose(w1, p / 6.103515625e-5, rtol=1e-5) and np.allclose(w2, 1.0 / k, rtol=1e-5)
