@@ -327,6 +327,7 @@ def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=
     gate / up row dots, the clamped SwiGLU, h rounded to Q8_K, the down row dots: src/kernels/cpu/native_expert.cpp:306-442)
     in the plan's row order (src/kernels/cuda/glm_batch.cu:2102-2133), and the weighted sum in slot order.  Returns a dict
     of every stage: xq / xd / xs = the rows' codes, block scales and d * (sum of every 32 codes); h = the SwiGLU values."""
+    tg, td = t if isinstance(t, tuple) else (t, t)   # (gate/up type, down type)
     ids, w = router_topk(logits, k)
     ne = len(blobs)
     bounds, row_entry, entry_row = prefill_plan(ids, ne, resident)
@@ -342,15 +343,15 @@ def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=
     for r in range(rows):
         tok, e = int(row_entry[r]) // k, int(ids.reshape(-1)[row_entry[r]])
         if tok not in acts:
-            a = quant_act(t, x[tok])
+            a = quant_act(tg, x[tok])
             d, q, bs = q8k_fields(a)
             acts[tok] = (a, q, d, (d[:, None] * (bs[:, 0::2] + bs[:, 1::2]).astype(np.float32)).reshape(-1))
         a, xq[r], xd[r], xs[r] = acts[tok]
         b = blobs[e]
-        g = rows_of(t, b, n_embd, n_ff, a)
-        u = rows_of(t, b[up_off:], n_embd, n_ff, a)
+        g = rows_of(tg, b, n_embd, n_ff, a)
+        u = rows_of(tg, b[up_off:], n_embd, n_ff, a)
         h[r] = [sw(float(gv), float(uv), lim) for gv, uv in zip(g, u)]
-        part[r] = rows_of(t, b[down_off:], n_ff, n_embd, quant_act(t, h[r]))
+        part[r] = rows_of(td, b[down_off:], n_ff, n_embd, quant_act(td, h[r]))
     out = np.zeros((x.shape[0], n_embd), dtype=np.float32)
     for tok in range(x.shape[0]):
         sel = [j for j in range(k) if entry_row[tok * k + j] >= 0]

@@ -240,13 +240,14 @@ struct PfGemm {
 constexpr int kPfPlane = kPfRows * 256;
 constexpr int kPfSOff = kPfPlane, kPfDOff = kPfSOff + kPfRows * 32;
 constexpr int kPfBufBytes = kPfDOff + kPfRows * 4;
+constexpr int kPfDOffNoS = kPfPlane, kPfBufBytesNoS = kPfDOffNoS + kPfRows * 4;   // (a buffer without s: types without minimums)
 
 typedef __attribute__((address_space(3))) void* pf_lptr;
 // The tile's activations go from global memory to LDS without passing registers (each lane's 16 bytes land at the
 // wave's base + 16 lane): buffer loads whose per-lane offsets are fixed for the tile - the super-block rides in the
 // scalar offset - so a copy costs no vector arithmetic.  Rows past the tile's end repeat its last row (their results
 // are never stored).
-template <int NMT>
+template <int NMT, bool WITH_S = true>
 struct PfDma {
     __amdgpu_buffer_rsrc_t rq, rs, rd;
     uint32_t oq[NMT], os, od;
@@ -270,9 +271,9 @@ struct PfDma {
 #pragma unroll
         for (int n = 0; n < NMT; ++n)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rq, (pf_lptr) (buf + (wave + 4 * n) * 1024), 16, oq[n], sb * 256, 0, 0);
-        if (wave < 2 && 32 * wave < 16 * NMT)   // s: 32 rows an instruction, 32 bytes a row
+        if (WITH_S && wave < 2 && 32 * wave < 16 * NMT)   // s: 32 rows an instruction, 32 bytes a row
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (pf_lptr) (buf + kPfSOff + wave * 1024), 16, os, sb * 32, 0, 0);
-        if (wave == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (pf_lptr) (buf + kPfDOff), 4, od, sb * 4, 0, 0);
+        if (wave == 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rd, (pf_lptr) (buf + (WITH_S ? kPfDOff : kPfDOffNoS)), 4, od, sb * 4, 0, 0);
     }
 };
 
@@ -306,6 +307,17 @@ __device__ __forceinline__ uint32_t pf_scale_codes(uint32_t w, uint32_t f) {
 // on the registers it filled (the values pass through the wait, so nothing that uses them can move above it).
 __device__ __forceinline__ uint32_t pf_lds_addr(const void* p) {
     return (uint32_t) (uintptr_t) (const __attribute__((address_space(3))) void*) p;
+}
+typedef int pf_i2 __attribute__((ext_vector_type(2)));
+template <int OFF> __device__ __forceinline__ pf_i2 pf_lds_b64(uint32_t addr) {
+    pf_i2 v;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> __device__ __forceinline__ uint32_t pf_lds_u16(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
 }
 template <int OFF> __device__ __forceinline__ float pf_lds_f32(uint32_t addr) {
     float v;
@@ -534,6 +546,8 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     }
 }
 
+#include "maya_prefill_iq2s.cuh"
+
 // grid (bands of weight rows, tiles at most)
 template <bool GU>
 __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
@@ -599,7 +613,7 @@ int maya_moe_prefill_max_tiles(int n_entries, int n_expert) {
     if (n_entries <= 0 || n_expert <= 0) return 0;
     return (n_entries + kPfRows - 1) / kPfRows + n_expert;
 }
-int maya_moe_prefill_supported(int type) { return type == kQ4_K ? 1 : 0; }
+int maya_moe_prefill_supported(int type) { return type == kQ4_K || type == kIQ2_S ? 1 : 0; }
 
 int maya_moe_prefill_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert,
                           const maya_prefill_plan* plan, void* stream) {
@@ -638,12 +652,17 @@ int maya_moe_prefill_quant(const void* x, int x_dtype, int64_t x_stride, const m
 }
 
 static int prefill_check(const char* what, const maya_moe_layout* l, const uint64_t* table, int n_expert, const maya_prefill_plan* plan,
-                         int n_entries, int type_a, int type_b) {
+                         int n_entries, int type_a, int type_b, int64_t k) {
     if (!l || !table || !plan_ok(plan)) return fail(MAYA_E_ARG, "%s: null pointer", what);
-    if (type_a != kQ4_K || type_b != kQ4_K) return fail(MAYA_E_UNSUPPORTED, "%s: weight types %d / %d (Q4_K only)", what, type_a, type_b);
-    if (l->packing != MAYA_PACK_GGUF) return fail(MAYA_E_UNSUPPORTED, "%s: GGUF packing only", what);
+    if (type_a != type_b || (type_a != kQ4_K && type_a != kIQ2_S))
+        return fail(MAYA_E_UNSUPPORTED, "%s: weight types %d / %d (Q4_K or IQ2_S, gate and up alike)", what, type_a, type_b);
+    if (l->packing != MAYA_PACK_GGUF && l->packing != MAYA_PACK_STREAM) return fail(MAYA_E_UNSUPPORTED, "%s: packing %d", what, l->packing);
+    if (type_a == kIQ2_S && l->packing != MAYA_PACK_STREAM)
+        return fail(MAYA_E_UNSUPPORTED, "%s: IQ2_S rows are taken in the stream packing (maya_moe_repack)", what);
     if (l->n_embd <= 0 || l->n_ff <= 0 || l->n_embd % 256 || l->n_ff % 256)
         return fail(MAYA_E_SHAPE, "%s: n_embd %d / n_ff %d: multiples of 256 wanted", what, l->n_embd, l->n_ff);
+    // (IQ2_S: the 16-byte copies of a quad's index words want quads of a multiple of 16 bytes: 328 bytes a block)
+    if (type_a == kIQ2_S && k % 512) return fail(MAYA_E_SHAPE, "%s: IQ2_S rows of %lld values: a multiple of 512 wanted", what, (long long) k);
     if ((l->gate_off | l->up_off | l->down_off) & 15) return fail(MAYA_E_ARG, "%s: matrix offsets not 16-byte aligned", what);
     if (n_entries <= 0 || n_entries > 65535 * kPfRows || n_expert <= 0) return fail(MAYA_E_SHAPE, "%s: entries %d experts %d", what, n_entries, n_expert);
     return MAYA_OK;
@@ -653,7 +672,7 @@ int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_ta
                              int n_entries, maya_prefill_act xq, float limit, float* h, maya_prefill_act hq, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (const int rc = prefill_check("prefill_gate_up", l, expert_table, n_expert, plan, n_entries, l ? l->gate_type : 0, l ? l->up_type : 0)) return rc;
+    if (const int rc = prefill_check("prefill_gate_up", l, expert_table, n_expert, plan, n_entries, l ? l->gate_type : 0, l ? l->up_type : 0, l ? l->n_embd : 0)) return rc;
     if (!act_ok(xq) || !act_ok(hq) || !h) return fail(MAYA_E_ARG, "prefill_gate_up: null or misaligned activations");
     PfGemm a{};
     a.table = expert_table;
@@ -667,8 +686,13 @@ int maya_moe_prefill_gate_up(const maya_moe_layout* l, const uint64_t* expert_ta
     a.out = h;
     a.limit = limit;
     const dim3 grid((unsigned) (l->n_ff / 64), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
-    if (const int rc = pf_launch<true>(a, grid, as_stream(stream))) return rc;
-    MAYA_LAUNCHED("prefill_q4k_kernel<gate_up>");
+    if (l->gate_type == kIQ2_S) {
+        hipLaunchKernelGGL(prefill_iq2s_kernel<true>, grid, dim3(256), 0, as_stream(stream), a, st->cb);
+        MAYA_LAUNCHED("prefill_iq2s_kernel<gate_up>");
+    } else {
+        if (const int rc = pf_launch<true>(a, grid, as_stream(stream))) return rc;
+        MAYA_LAUNCHED("prefill_q4k_kernel<gate_up>");
+    }
     const dim3 qgrid((unsigned) ((l->n_ff + 8191) / 8192), (unsigned) n_entries);
     hipLaunchKernelGGL(prefill_quant_rows_kernel, qgrid, dim3(256), 0, as_stream(stream), (const float*) h, *plan, n_expert, (int64_t) l->n_ff, hq);
     MAYA_LAUNCHED("prefill_quant_rows_kernel");
@@ -679,7 +703,7 @@ int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table
                           int n_entries, maya_prefill_act hq, float* part, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (const int rc = prefill_check("prefill_down", l, expert_table, n_expert, plan, n_entries, l ? l->down_type : 0, l ? l->down_type : 0)) return rc;
+    if (const int rc = prefill_check("prefill_down", l, expert_table, n_expert, plan, n_entries, l ? l->down_type : 0, l ? l->down_type : 0, l ? l->n_ff : 0)) return rc;
     if (!act_ok(hq) || !part) return fail(MAYA_E_ARG, "prefill_down: null or misaligned pointer");
     if (l->n_embd % 32) return fail(MAYA_E_SHAPE, "prefill_down: n_embd %d", l->n_embd);
     PfGemm a{};
@@ -692,8 +716,13 @@ int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table
     a.x = hq;
     a.out = part;
     const dim3 grid((unsigned) ((l->n_embd + 127) / 128), (unsigned) maya_moe_prefill_max_tiles(n_entries, n_expert));
-    if (const int rc = pf_launch<false>(a, grid, as_stream(stream))) return rc;
-    MAYA_LAUNCHED("prefill_q4k_kernel<down>");
+    if (l->down_type == kIQ2_S) {
+        hipLaunchKernelGGL(prefill_iq2s_kernel<false>, grid, dim3(256), 0, as_stream(stream), a, st->cb);
+        MAYA_LAUNCHED("prefill_iq2s_kernel<down>");
+    } else {
+        if (const int rc = pf_launch<false>(a, grid, as_stream(stream))) return rc;
+        MAYA_LAUNCHED("prefill_q4k_kernel<down>");
+    }
     return MAYA_OK;
 }
 

@@ -159,6 +159,56 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
     assert torch.equal(got2, out)
 
 
+IQ_CASES = [
+    # gate/up type, down type, n_embd, n_ff, n_expert, k, n_tokens, limit, experts that are not resident
+    (22, 22, 512, 512, 6, 2, 41, 0.0, ()),
+    (22, 22, 1024, 512, 12, 4, 130, 7.0, (3,)),
+    (22, 12, 1024, 768, 5, 2, 70, 0.0, ()),          # IQ2_S gate / up with Q4_K down (the mixed experts)
+    (12, 22, 768, 1024, 4, 3, 90, 0.0, ()),          # and the other way round: 90-row experts, two tiles each
+    (22, 22, 7168, 2048, 3, 2, 20, 0.0, ()),         # the full expert shape
+]
+
+
+@pytest.mark.parametrize("case", IQ_CASES, ids=[str(c[:7]) for c in IQ_CASES])
+def test_iq2s_chunk_matches_checker(pf, oracle, case):
+    """The IQ2_S GEMMs (stream packing) and their mix with Q4_K: h, the down rows and the layer against the CPU path."""
+    from maya_amd import lib, synth
+    gt, dt, n_embd, n_ff, n_expert, k, n_tokens, limit, absent = case
+    rng = np.random.default_rng(900 + n_embd + gt)
+    blobs = [synth.expert_blob(gt, dt, n_embd, n_ff, rng) for _ in range(n_expert)]
+    up_off, down_off, _ = synth.blob_offsets(gt, dt, n_embd, n_ff)
+    gguf, _ = lib.layout(gt, dt, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf)
+    layout = lib.copy_layout(gguf, lib.PACK_STREAM)
+    table = store.table.clone()
+    resident = np.ones(n_expert, dtype=bool)
+    for e in absent:
+        table[e] = 0
+        resident[e] = False
+    logits = (rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32)
+    x = rng.standard_normal((n_tokens, n_embd)).astype(np.float32)
+    want = oracle.prefill_layer((gt, dt), blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit, resident)
+    ids, w = lib.route_topk(dev(logits), k)
+    p = pf.plan(ids.reshape(-1), table)
+    xq = pf.quant(dev(x), p, k)
+    hq = pf.gate_up(layout, table, p, xq, limit)
+    part = pf.down(layout, table, p, hq)
+    out = pf.combine(p, w, part, n_tokens, k)
+    torch.cuda.synchronize()
+    rows = int(want["bounds"][-1])
+    assert np.array_equal(ids.cpu().numpy(), want["ids"])
+    h = hq.f32.cpu().numpy()[:rows]
+    assert rel_l2(h, want["h"]) <= 1e-5
+    flat_ids = want["ids"].reshape(-1)
+    for r in range(0, rows, max(1, rows // 12)):
+        e = int(flat_ids[want["row_entry"][r]])
+        want_part = oracle.rows(dt, blobs[e][down_off:], n_ff, n_embd, oracle.quant_act(dt, h[r]))
+        assert rel_l2(part.cpu().numpy()[r], want_part) <= 1e-5, r
+    got = out.cpu().numpy()
+    for t in range(n_tokens):
+        assert rel_l2(got[t], want["out"][t]) <= 1e-3, t
+
+
 def test_chunk_tokens_equal_the_decode_layer(pf):
     """Two independent GPU paths, one contract: a token's row of the prompt chunk (grouped int8-MFMA GEMMs) is what the
     decode layer (dot-product mat-vecs) gives for that token alone - the same Q8_K codes and integer sums, F32 sums in
@@ -182,14 +232,19 @@ def test_chunk_tokens_equal_the_decode_layer(pf):
 
 def test_unsupported_and_bad_arguments(pf):
     from maya_amd import lib
-    assert pf.load().maya_moe_prefill_supported(Q4_K) == 1 and pf.load().maya_moe_prefill_supported(22) == 0
+    L = pf.load()
+    assert L.maya_moe_prefill_supported(Q4_K) == 1 and L.maya_moe_prefill_supported(22) == 1 and L.maya_moe_prefill_supported(19) == 0
     table = torch.arange(1, 5, dtype=torch.int64, device="cuda") * 4096
     ids = torch.zeros(8, dtype=torch.int32, device="cuda")
     p = pf.plan(ids, table)
     xq = pf.ActRows(8, 512)
     iq, _ = lib.layout(22, 22, 512, 256)
     with pytest.raises(lib.MayaError):
-        pf.gate_up(iq, table, p, xq)
+        pf.gate_up(iq, table, p, xq)                                   # IQ2_S rows in the GGUF packing
+    with pytest.raises(lib.MayaError):
+        pf.gate_up(lib.copy_layout(lib.layout(22, 22, 768, 256)[0], lib.PACK_STREAM), table, p, pf.ActRows(8, 768))   # 768 % 512
+    with pytest.raises(lib.MayaError):
+        pf.gate_up(lib.copy_layout(lib.layout(19, 19, 512, 256)[0], lib.PACK_STREAM), table, p, xq)                   # IQ1_S
     bad, _ = lib.layout(Q4_K, Q4_K, 512, 256)
     bad.n_ff = 200
     with pytest.raises(lib.MayaError):
