@@ -5,7 +5,7 @@
 // (2 ls_j + 1) (w_j . c_j), w = the grid magnitudes with their signs: the integer sums of the CPU path's IQ2_S x Q8_K
 // row dot (src/kernels/cpu/iq_avx2.cpp:160-176, 225-250).  The scale belongs to 16 values and (2 ls + 1) x 43 does not fit
 // int8, so a 32-deep matrix instruction takes ONE group: a lane (row ln, k-group kg) decodes grid entry kg of a
-// sub-block - 8 signed bytes, its whole operand - and the two groups of a sub-block come from two instructions whose
+// sub-block - 8 signed bytes (the grid's magnitudes and a sign-mask table sit in LDS), its whole operand - and the two groups of a sub-block come from two instructions whose
 // operands are zero in the lanes of the other group (kg < 2: values 0..15, kg >= 2: 16..31).  The vector ALU then adds
 // (2 ls + 1) x the group's sums to the block's int32 sums: two multiply-adds an output a sub-block.
 //
@@ -127,22 +127,25 @@ __device__ __forceinline__ void pf_tile_iq2s(const PfGemm& a, uint8_t* b0, uint8
                     const uint32_t ga = grid_lds + ((idx | (hi2 << 8)) << 3);
                     gr[t] = pf_lds_b64<0>(ga);
                 }
-                // the signs: bit i of the entry's sign byte -> 0x01 in byte i, the marked bytes negated (none is 0)
-                uint32_t c[2][2], s0[2], s1[2];
+                // the signs: the entry's sign byte -> 0xff in the bytes of its set bits (a 256-entry table beside the grid)
+                pf_i2 sm[2];
+                int s0[2], s1[2];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     const uint32_t sbyte = __builtin_amdgcn_ubfe((uint32_t) iw[t].y, sh8, 8u);
-                    c[t][0] = spread4(sbyte & 15u);
-                    c[t][1] = spread4(sbyte >> 4);
+                    sm[t] = pf_lds_b64<8192>(grid_lds + (sbyte << 3));
                     const uint32_t sc = hs[t] >> 8;
-                    s0[t] = 2u * (sc & 15u) + 1u;
-                    s1[t] = 2u * (sc >> 4) + 1u;
+                    s0[t] = (int) (2u * (sc & 15u) + 1u);
+                    s1[t] = (int) (2u * (sc >> 4) + 1u);
                 }
                 pf_lds_wait(gr);
+                pf_lds_wait(sm);
                 pf_lds_wait(xr);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const uint32_t wa = neg_bytes((uint32_t) gr[t].x, c[t][0]), wb = neg_bytes((uint32_t) gr[t].y, c[t][1]);
+                    // the marked bytes negated: (g ^ 0xff) + 1 a byte, no carry (no magnitude is 0)
+                    const uint32_t ma = (uint32_t) sm[t].x, mb = (uint32_t) sm[t].y;
+                    const uint32_t wa = ((uint32_t) gr[t].x ^ ma) + (ma & 0x01010101u), wb = ((uint32_t) gr[t].y ^ mb) + (mb & 0x01010101u);
                     const long o0 = (long) (((uint64_t) (wb & m0) << 32) | (uint64_t) (wa & m0));
                     const long o1 = (long) (((uint64_t) (wb & m1) << 32) | (uint64_t) (wa & m1));
 #pragma unroll
@@ -153,7 +156,11 @@ __device__ __forceinline__ void pf_tile_iq2s(const PfGemm& a, uint8_t* b0, uint8
                         const v4i d1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(xa, o1, z, 0, 0, 0);
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            isum[t][m][i] += __mul24((int) s0[t], d0[i]) + __mul24((int) s1[t], d1[i]);
+                        {   // two 24-bit multiply-adds (kept apart: joined, the compiler makes two multiplies and a 3-way add)
+                            int v = __mul24(s0[t], d0[i]) + isum[t][m][i];
+                            asm("" : "+v"(v));
+                            isum[t][m][i] = __mul24(s1[t], d1[i]) + v;
+                        }
                     }
                 }
             }
@@ -215,10 +222,17 @@ template <bool GU>
 __global__ __launch_bounds__(256, 2) void prefill_iq2s_kernel(PfGemm a, Codebooks cb) {
     __shared__ __attribute__((aligned(16))) uint8_t b0[kPfBufBytesNoS], b1[kPfBufBytesNoS], b2[kPfBufBytesNoS];
     __shared__ __attribute__((aligned(16))) uint8_t w0[kIqBufBytes], w1[kIqBufBytes];
-    __shared__ __attribute__((aligned(16))) uint64_t grid[1024];
+    __shared__ __attribute__((aligned(16))) uint64_t grid[1024 + 256];   // the magnitudes, then the sign masks
     const int tile = blockIdx.y;
     if (tile >= *a.plan.n_tiles) return;
     for (int i = threadIdx.x; i < 1024; i += 256) grid[i] = cb.iq2s[i];
+    {
+        uint64_t m = 0ull;
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+            if (threadIdx.x & (1 << b)) m |= 0xffull << (8 * b);
+        grid[1024 + threadIdx.x] = m;
+    }
     const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
     const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
     const uint32_t gl = pf_lds_addr(grid);
