@@ -140,7 +140,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="decode_iq2s",
                     help="decode_iq2s (configs[1], the default and the headline metric), or one of the other BASELINE "
-                         "configurations: single_q4k, batch8_mixed, prefill_q4k, exl3_verify")
+                         "configurations: single_q4k, batch8_mixed, prefill_q4k, exl3_verify; the prefill chunk on other expert types: "
+                         "prefill_iq2s, prefill_mixed")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters by)")

@@ -284,7 +284,8 @@ typedef struct maya_prefill_act {
 
 int maya_moe_prefill_tile_rows(void);
 int maya_moe_prefill_max_tiles(int n_entries, int n_expert);
-/* 1 when the prefill GEMMs take this weight type (Q4_K) */
+/* 1 when the prefill GEMMs take this weight type: Q4_K (either packing; 16-byte aligned matrices) and IQ2_S (the stream
+ * packing, rows of a multiple of 512 values); gate and up of one type, down of either (the mixed experts) */
 int maya_moe_prefill_supported(int type);
 int maya_moe_prefill_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert,
                           const maya_prefill_plan* plan, void* stream);

@@ -154,11 +154,41 @@ def batch8_mixed(K, W):
             "roofline": hbm_roofline("layer (routed gate_up_iq2s_pos_kernel + down_q4k_pos_kernel over 64 entries, shared expert gate_up_q80_pos_kernel + down_q80_pos_kernel)", nbytes, sec)}
 
 
+BLOCK_FIELDS = {lib.Q4_K: (144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}), 22: (82, {0: (2e-3, 6e-3)})}
+
+
 def prefill_q4k(K, W):
     """configs[3]: 512 tokens, 256 Q4_K experts top-8, Zipf(1.1)-skewed routing, int8 (Q8_K) activations, bf16 out."""
+    return _prefill(K, W, lib.Q4_K, lib.Q4_K, "configs[3]", "Q4_K")
+
+
+def prefill_iq2s(K, W):
+    """configs[3]'s chunk on the north-star layer's IQ2_S experts (stream packing)."""
+    return _prefill(K, W, 22, 22, "configs[3]'s chunk on IQ2_S experts", "IQ2_S")
+
+
+def prefill_mixed(K, W):
+    """configs[3]'s chunk on configs[2]'s experts: IQ2_S gate / up, Q4_K down (stream packing)."""
+    return _prefill(K, W, 22, lib.Q4_K, "configs[3]'s chunk on IQ2_S gate/up + Q4_K down experts", "IQ2_S / Q4_K")
+
+
+def _prefill(K, W, gt, dt, what, types):
     E, FF, NE, TK, T = 7168, 2048, 256, 8, 512
-    layout, bb = lib.layout(lib.Q4_K, lib.Q4_K, E, FF)
-    pool = random_blocks(NE * bb, 144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}, 11)
+    gguf, bb = lib.layout(gt, dt, E, FF)
+    stream_packed = gt != lib.Q4_K or dt != lib.Q4_K
+    layout = lib.copy_layout(gguf, lib.PACK_STREAM) if stream_packed else gguf
+    if stream_packed:
+        # the three stacked tensors as a file holds them, then the blobs built on the device in the stream packing
+        mats = []
+        for i, (t, nbytes) in enumerate(((gt, gguf.up_off), (gt, gguf.down_off - gguf.up_off), (dt, bb - gguf.down_off))):
+            block, fields = BLOCK_FIELDS[t]
+            mats.append(random_blocks(NE * nbytes, block, fields, 11 + i))
+        pool = torch.empty(NE * bb, dtype=torch.uint8, device="cuda")
+        lib.pack_experts(gguf, mats[0], mats[1], mats[2], NE, lib.PACK_STREAM, pool, bb)
+        torch.cuda.synchronize()
+        del mats
+    else:
+        pool = random_blocks(NE * bb, 144, BLOCK_FIELDS[lib.Q4_K][1], 11)
     table = torch.tensor([pool.data_ptr() + e * bb for e in range(NE)], dtype=torch.int64, device="cuda")
     rng = np.random.default_rng(12)
     logits = torch.from_numpy((rng.standard_normal((T, NE)) + synth.zipf_bias(NE)).astype(np.float32)).cuda()
@@ -185,11 +215,12 @@ def prefill_q4k(K, W):
     tops_gu = ops_gu / sec_gu / 1e12
     return {"metric": "prefill_int8_tops_512tok", "value": round(ops / sec / 1e12, 2), "unit": "TOP/s", "ms_per_step": sec * 1e3,
             "dtype": "int8",
-            "config": {"workload": "configs[3]: prefill chunk of 512 tokens, 256 experts Q4_K top-8, logits N(0,1) - 1.1 ln(e+1), "
+            "config": {"workload": what + ": prefill chunk of 512 tokens, 256 experts " + types + " top-8, logits N(0,1) - 1.1 ln(e+1), "
                                    "int8 activations in the CPU path's Q8_K rounding, bf16 out", "experts_with_rows": used, "int8_ops_per_step": ops,
                        "algorithmic_bytes_per_step": int(nbytes), "weight_gbps": round(nbytes / sec / 1e9, 1),
                        "pct_of_hbm_peak": round(100 * nbytes / sec / HBM_PEAK, 2)},
-            "roofline": {"bound": "mfma", "kernel": "prefill_q4k_kernel<gate_up>", "achieved": round(tops_gu, 2), "peak": 5000.0,
+            "roofline": {"bound": "mfma", "kernel": ("prefill_q4k_kernel" if gt == lib.Q4_K else "prefill_iq2s_kernel") + "<gate_up>",
+                         "achieved": round(tops_gu, 2), "peak": 5000.0,
                          "unit": "TOP/s", "frac": round(tops_gu * 1e12 / INT8_PEAK, 4), "traffic": None,
                          "algorithmic_ops_per_launch": ops_gu, "avg_launch_us": round(sec_gu * 1e6, 1)}}
 
@@ -234,4 +265,5 @@ def exl3_verify(K, W):
             "roofline": hbm_roofline("layer (exl3_gu_split_kernel + exl3_swiglu_kernel + exl3_down_kernel + exl3_combine_kernel)", nbytes, sec)}
 
 
-WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify}
+WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify,
+             "prefill_iq2s": prefill_iq2s, "prefill_mixed": prefill_mixed}
