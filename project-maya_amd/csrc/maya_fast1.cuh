@@ -60,7 +60,7 @@ __device__ __forceinline__ float unit1_value(const QuadIQ1S& q, const uint2* gri
         t = dot4((int) g.x, y[2 * l], t);
         t = dot4((int) g.y, y[2 * l + 1], t);
     }
-    t += ((qh & 0x8000u) ? -10 : -8) * sy;
+    t += __mul24((qh & 0x8000u) ? -10 : -8, sy);   // (a 24-bit multiply-add: the 32-bit one runs at a quarter of the rate)
     const int isum = __mul24(2 * (int) ((qh >> 12) & 7u) + 1, t);
     return __fmul_rn(__fmul_rn(f16_bits_to_f32(d), dy8), (float) isum);
 }
@@ -271,7 +271,7 @@ __device__ __forceinline__ float unitm_value(const QuadIQ1M& q, const uint2* gri
         const uint2 g = grid[((i4 >> (8 * l)) & 255u) | ((nib & 7u) << 8)];
         t[l >> 1] = dot4((int) g.x, y[2 * l], t[l >> 1]);
         t[l >> 1] = dot4((int) g.y, y[2 * l + 1], t[l >> 1]);
-        t[l >> 1] += ((nib & 8u) ? -10 : -8) * sy8[l];
+        t[l >> 1] += __mul24((nib & 8u) ? -10 : -8, sy8[l]);
     }
     const int isum = __mul24(2 * (int) (sc & 7u) + 1, t[0]) + __mul24(2 * (int) ((sc >> 3) & 7u) + 1, t[1]);
     return __fmul_rn(__fmul_rn(f16_bits_to_f32(s_lo & 0xffffu), dy8), (float) isum);

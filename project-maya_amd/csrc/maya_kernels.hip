@@ -890,10 +890,12 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
                     hi = dot4(u.hi[i], y[8 + i], hi);
                 }
                 const int b0 = a.bs2[t * a.kd + 2 * p], b1 = a.bs2[t * a.kd + 2 * p + 1];
-                const int ms = u.m0 * ((int) (short) (b0 & 0xffff) + (b0 >> 16)) +
-                               u.m1 * ((int) (short) (b1 & 0xffff) + (b1 >> 16));
+                // (24-bit multiplies throughout: the operands are sums of at most 32 products of bytes, and the 32-bit
+                // integer multiply runs at a quarter of the rate)
+                const int ms = __mul24(u.m0, (int) (short) (b0 & 0xffff) + (b0 >> 16)) +
+                               __mul24(u.m1, (int) (short) (b1 & 0xffff) + (b1 >> 16));
                 const float dy = a.d[t * a.kd + 2 * p];
-                acc[t] = fmaf(__fmul_rn(dy, D), (float) (u.sc0 * lo + u.sc1 * hi), acc[t]);
+                acc[t] = fmaf(__fmul_rn(dy, D), (float) (__mul24(u.sc0, lo) + __mul24(u.sc1, hi)), acc[t]);
                 acc[t] = fmaf(-__fmul_rn(dy, Dm), (float) ms, acc[t]);
             }
         }
@@ -937,16 +939,16 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
                     const int bs = a.bs2[t * a.kd + un];
                     const int s_lo = (int) (short) (bs & 0xffff), s_hi = bs >> 16;
                     if constexpr (TYPE == kIQ1_S) {   // one delta a sub-block
-                        lo += u.dm[0] * s_lo;
-                        hi += u.dm[0] * s_hi;
+                        lo += __mul24(u.dm[0], s_lo);
+                        hi += __mul24(u.dm[0], s_hi);
                     } else {                          // one a group of 8: the first group's sum, the second's by difference
                         const int a0 = dot4(0x01010101, y[0], dot4(0x01010101, y[1], 0));
                         const int a1 = dot4(0x01010101, y[4], dot4(0x01010101, y[5], 0));
-                        lo += u.dm[0] * a0 + u.dm[1] * (s_lo - a0);
-                        hi += u.dm[2] * a1 + u.dm[3] * (s_hi - a1);
+                        lo += __mul24(u.dm[0], a0) + __mul24(u.dm[1], s_lo - a0);
+                        hi += __mul24(u.dm[2], a1) + __mul24(u.dm[3], s_hi - a1);
                     }
                 }
-                acc[t] = fmaf(__fmul_rn(D, a.d[t * a.kd + un]), (float) (u.s0 * lo + u.s1 * hi), acc[t]);
+                acc[t] = fmaf(__fmul_rn(D, a.d[t * a.kd + un]), (float) (__mul24(u.s0, lo) + __mul24(u.s1, hi)), acc[t]);
             }
         }
     }
