@@ -1221,6 +1221,7 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
 #include "maya_fast1.cuh"
 #include "maya_fastk.cuh"
 #include "maya_fastq.cuh"
+#include "maya_fastmv.cuh"
 
 namespace maya {
 
@@ -1867,6 +1868,55 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
     return MAYA_OK;
 }
 
+}  // extern "C"
+
+namespace maya {
+// rows of 1024 NW values (NW 2, 4, 6, 7, 8) in whole groups of 16 row pairs; Q8_0 in the stream packing, Q4_K 16-byte aligned
+static bool mv_pos_ok(const maya_mv_job& j) {
+    const int nw = j.n_in / 1024;
+    if (j.n_in % 1024 || !(nw == 2 || nw == 4 || nw == 6 || nw == 7 || nw == 8) || j.n_out % 32 || ((uintptr_t) j.w & 15)) return false;
+    if ((size_t) j.n_out * maya_moe_row_bytes(j.type, j.n_in) >= (1ull << 32)) return false;   // (32-bit buffer offsets)
+    if (j.type == kQ8_0) return j.packing == MAYA_PACK_STREAM;
+    return j.type == kQ4_K;
+}
+template <int NW>
+static void launch_mv_pos_nw(const maya_mv_job& j, hipStream_t s) {
+    const MvPos a{(const uint8_t*) j.w, j.x, j.bias, j.y, (long long) j.y_stride, j.alpha, j.n_out, j.ncol};
+    // 16 row pairs a workgroup when that still gives two workgroups a compute unit, else 8
+    const bool big = j.n_out / 32 >= 512;
+    if (j.type == kQ4_K) {
+        if (big) hipLaunchKernelGGL((mv_q4k_pos_kernel<NW, 16>), dim3((unsigned) (j.n_out / 32), (unsigned) j.ncol), dim3(64 * NW), 0, s, a);
+        else hipLaunchKernelGGL((mv_q4k_pos_kernel<NW, 8>), dim3((unsigned) (j.n_out / 16), (unsigned) j.ncol), dim3(64 * NW), 0, s, a);
+    } else {
+        const unsigned g16 = (unsigned) (j.n_out / 32), g8 = (unsigned) (j.n_out / 16);
+        if (j.ncol == 1) {
+            if (big) hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 1, 16>), dim3(g16), dim3(64 * NW), 0, s, a);
+            else hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 1, 8>), dim3(g8), dim3(64 * NW), 0, s, a);
+        } else if (j.ncol == 2) {
+            if (big) hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 2, 16>), dim3(g16), dim3(64 * NW), 0, s, a);
+            else hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 2, 8>), dim3(g8), dim3(64 * NW), 0, s, a);
+        } else if (j.ncol <= 4) {
+            if (big) hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 4, 16>), dim3(g16), dim3(64 * NW), 0, s, a);
+            else hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 4, 8>), dim3(g8), dim3(64 * NW), 0, s, a);
+        } else {
+            if (big) hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 8, 16>), dim3(g16), dim3(64 * NW), 0, s, a);
+            else hipLaunchKernelGGL((mv_q80_pos_kernel<NW, 8, 8>), dim3(g8), dim3(64 * NW), 0, s, a);
+        }
+    }
+}
+static void launch_mv_pos(const maya_mv_job& j, hipStream_t s) {
+    switch (j.n_in / 1024) {
+        case 2: launch_mv_pos_nw<2>(j, s); break;
+        case 4: launch_mv_pos_nw<4>(j, s); break;
+        case 6: launch_mv_pos_nw<6>(j, s); break;
+        case 7: launch_mv_pos_nw<7>(j, s); break;
+        default: launch_mv_pos_nw<8>(j, s); break;
+    }
+}
+}  // namespace maya
+
+extern "C" {
+
 int maya_mv_supported(int type) { return type_ok(type) ? 1 : 0; }
 
 int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
@@ -1886,13 +1936,19 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
         if (!j.w || !j.x.q || !j.x.d || (q8k_act(j.type) && !j.x.bsums) || !j.y) return fail(MAYA_E_ARG, "mv: job %d: null pointer", i);
         if (j.y_stride < j.n_out && j.ncol > 1) return fail(MAYA_E_ARG, "mv: job %d: y_stride %lld below n_out %d", i, (long long) j.y_stride, j.n_out);
     }
+    // the position-mapped kernels take the jobs whose shape they cover, a launch each; the others go by type
+    bool fast[MAYA_MV_MAX_JOBS];
+    for (int i = 0; i < n_jobs; ++i) {
+        fast[i] = mv_pos_ok(jobs[i]);
+        if (fast[i]) launch_mv_pos(jobs[i], as_stream(stream));
+    }
     static const int kTypes[] = {kQ8_0, kQ4_K, kIQ1_S, kIQ2_S, kIQ1_M};
     for (const int t : kTypes) {
         MvBatch b{};
         int n = 0, max_in = 0, max_out = 0, max_col = 0;
         for (int i = 0; i < n_jobs; ++i) {
             const maya_mv_job& j = jobs[i];
-            if (j.type != t) continue;
+            if (j.type != t || fast[i]) continue;
             b.job[n++] = MvJobDev{(const uint8_t*) j.w, j.x, j.bias, j.y, (long long) j.y_stride, j.alpha, j.n_in, j.n_out, j.ncol, j.packing};
             max_in = j.n_in > max_in ? j.n_in : max_in;
             max_out = j.n_out > max_out ? j.n_out : max_out;

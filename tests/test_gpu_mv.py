@@ -44,15 +44,31 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("t,n_in,n_out,ncol,alpha,with_bias", CASES)
-def test_mv_against_the_oracle_rows(lib, oracle, t, n_in, n_out, ncol, alpha, with_bias):
+def q80_stream_rows(w, n_out, n_in):
+    """Q8_0 rows from the GGUF block order (2-byte scale, 32 codes, ...) to the stream order (a row's codes, then its scales)."""
+    g = w.reshape(n_out, n_in // 32, 34)
+    return np.ascontiguousarray(np.concatenate([g[:, :, 2:].reshape(n_out, n_in), g[:, :, :2].reshape(n_out, -1)], axis=1)).reshape(-1)
+
+
+# shapes the position-mapped kernels take (rows of 1024 NW values, n_out a multiple of 32; Q8_0 in the stream packing, Q4_K
+# 16-byte aligned): type, n_in, n_out, columns, alpha, bias, packing
+POS_CASES = [
+    (8, 2048, 64, 1, 1.0, False, 1), (8, 7168, 96, 5, 0.5, True, 1), (8, 4096, 32, 8, 1.0, False, 1), (8, 6144, 64, 16, 1.0, True, 1),
+    (8, 8192, 32, 3, 2.0, False, 1), (8, 2048, 16384, 2, 1.0, True, 1),
+    (12, 7168, 64, 1, 1.0, True, 0), (12, 2048, 16384, 2, 0.25, False, 0), (12, 4096, 96, 4, 1.0, False, 1), (12, 8192, 32, 1, 1.0, True, 0),
+    (12, 6144, 160, 3, 1.0, False, 0),
+]
+
+
+@pytest.mark.parametrize("t,n_in,n_out,ncol,alpha,with_bias,packing", [c + (0,) for c in CASES] + POS_CASES)
+def test_mv_against_the_oracle_rows(lib, oracle, t, n_in, n_out, ncol, alpha, with_bias, packing):
     rng = np.random.default_rng(t * 1000 + n_out)
     w = synth.constructed_rows(t, n_out, n_in, rng)
     x = rng.standard_normal((ncol, n_in)).astype(np.float32)
     bias = rng.standard_normal(n_out).astype(np.float32) if with_bias else None
     want = want_of(oracle, t, w, n_in, n_out, x, alpha, bias)
-    w_d, x_d = dev(w), dev(x)
-    job = dict(w=w_d, type=t, x=x_d, n_out=n_out, alpha=alpha, bias=None if bias is None else dev(bias))
+    w_d, x_d = dev(q80_stream_rows(w, n_out, n_in) if (t == 8 and packing) else w), dev(x)
+    job = dict(w=w_d, type=t, x=x_d, n_out=n_out, alpha=alpha, bias=None if bias is None else dev(bias), packing=packing)
     (got,) = lib.mv([job])
     torch.cuda.synchronize()
     assert rel_l2(got.cpu().numpy(), want) <= TOL
