@@ -231,6 +231,8 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream);               /*
  * the host (the sequence of glm_fast_path.cu:2688-2691 and ds4_gguf.cu:1903-1971).
  *   expert_table: [n_expert] device array of blob addresses (0: not resident);
  *   x: [n_tokens][n_embd] of x_dtype; out: [n_tokens][n_embd] F32; ids / weights: [n_tokens][k] results of the router;
+ *   logits NULL (here, in maya_moe_prefill_layer and in maya_exl3_layer_decode): the tokens are already routed - ids and
+ *   weights are inputs (any router's: maya_moe_route_sigmoid, the engine's own) and the layer starts at the plan;
  *   workspace: maya_moe_workspace_bytes(layout, n_tokens, k) bytes, 256-byte aligned. */
 size_t maya_moe_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k);
 int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,

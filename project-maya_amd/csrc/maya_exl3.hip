@@ -688,13 +688,13 @@ size_t maya_exl3_workspace_bytes(const maya_exl3_layout* l, int n_tokens, int k)
 int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
                            const float* x, int n_tokens, float limit, const float* add, int32_t* ids, float* weights,
                            float* out, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!l || !expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "exl3 layer: null pointer");
+    if (!l || !expert_table || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "exl3 layer: null pointer");
     if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K) return fail(MAYA_E_SHAPE, "exl3 layer: n_tokens %d / k %d", n_tokens, k);
     if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "exl3 layer: workspace not 256-byte aligned");
     const Exl3Ws w = exl3_carve(*l, n_tokens, k, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "exl3 layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     int rc;
-    if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+    if (logits && (rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;   // (null: ids / weights are given)
     if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
     maya_exl3_args a{};
     a.layout = *l;

@@ -2023,7 +2023,7 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
     RouterSpec rs;
     if (!router_spec(router, rs)) return fail(MAYA_E_UNSUPPORTED, "layer_decode: router kind %d / normalisation %d", router->kind, router->norm);
     if (const int rc = check_layout(*l)) return rc;
-    if (!expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "layer_decode: null pointer");
+    if (!expert_table || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "layer_decode: null pointer");
     if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K)
         return fail(MAYA_E_SHAPE, "layer_decode: n_tokens %d / k %d", n_tokens, k);
     if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "layer_decode: workspace not 256-byte aligned");
@@ -2043,7 +2043,7 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
     a.part = w.part;
     a.add = add;
     a.out = out;
-    if (q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
+    if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
         // one launch: route, plan, Q8_K of x, cleared counters
         const int n_counters = n_tokens * k * (l->n_ff / 256);
         const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
@@ -2057,7 +2057,7 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
         MAYA_LAUNCHED("layer_head_kernel");
         a.hq_sync = down_rounds_h(a) ? nullptr : w.hq_sync;   // (the down kernel's own rounding of h is the cheaper one)
     } else {
-        if ((rc = route_impl("layer_decode", logits, n_tokens, n_expert, k, rs, ids, weights, stream))) return rc;
+        if (logits && (rc = route_impl("layer_decode", logits, n_tokens, n_expert, k, rs, ids, weights, stream))) return rc;   // (null: ids / weights are given)
         if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }

@@ -786,14 +786,14 @@ size_t maya_moe_prefill_workspace_bytes(const maya_moe_layout* l, int n_tokens, 
 int maya_moe_prefill_layer(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
                            const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
                            float* weights, void* out, int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!l || !expert_table || !logits || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "prefill_layer: null pointer");
+    if (!l || !expert_table || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "prefill_layer: null pointer");
     if (n_tokens <= 0 || n_tokens > 8192 || k <= 0 || k > MAYA_MAX_K) return fail(MAYA_E_SHAPE, "prefill_layer: tokens %d k %d", n_tokens, k);
     if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "prefill_layer: workspace not 256-byte aligned");
     const PrefillWs w = prefill_carve(*l, n_tokens, k, n_expert, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "prefill_layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     const int ne = n_tokens * k;
     int rc;
-    if ((rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;
+    if (logits && (rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;   // (null: ids / weights are given)
     if ((rc = maya_moe_prefill_plan(ids, ne, expert_table, n_expert, &w.plan, stream))) return rc;
     if ((rc = maya_moe_prefill_quant(x, x_dtype, 0, &w.plan, ne, n_expert, k, l->n_embd, w.x, stream))) return rc;
     if ((rc = maya_moe_prefill_gate_up(l, expert_table, n_expert, &w.plan, ne, w.x, limit, w.hf, w.h, stream))) return rc;

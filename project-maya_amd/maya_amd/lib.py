@@ -282,10 +282,17 @@ class MoeLayer:
         self.weights = torch.empty((max_tokens, k), dtype=torch.float32, device=device)
         self.out = torch.empty((max_tokens, n_embd), dtype=torch.float32, device=device)
 
-    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None):
-        """router: None (the softmax router) or a Router (kind, norm, bias pointer, w_scale)."""
+    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None, routed=None):
+        """router: None (the softmax router) or a Router (kind, norm, bias pointer, w_scale); routed = (ids, weights)
+        [nt, k] tensors: the tokens are already routed (logits is then ignored)."""
         nt = x.shape[0]
-        assert nt <= self.max_tokens and x.is_contiguous() and logits.is_contiguous()
+        assert nt <= self.max_tokens and x.is_contiguous()
+        if routed is not None:
+            self.ids[:nt].copy_(routed[0])
+            self.weights[:nt].copy_(routed[1])
+            logits = None
+        else:
+            assert logits.is_contiguous()
         if router is not None:
             check(load().maya_moe_layer_decode_routed(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, C.byref(router),
                                                       _p(logits), _p(x), dtype_id(x), nt, limit, _p(add), _p(self.ids),

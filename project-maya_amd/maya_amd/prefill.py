@@ -121,9 +121,16 @@ class PrefillLayer:
         self.weights = torch.empty((max_tokens, k), dtype=torch.float32, device=device)
         self.out = torch.empty((max_tokens, layout.n_embd), dtype=out_dtype, device=device)
 
-    def forward(self, expert_table, logits, x, limit=0.0, add=None, stream=None):
+    def forward(self, expert_table, logits, x, limit=0.0, add=None, stream=None, routed=None):
+        """routed = (ids, weights) [nt, k] tensors: the tokens are already routed (logits is then ignored)."""
         nt = x.shape[0]
-        assert nt <= self.max_tokens and x.is_contiguous() and logits.is_contiguous()
+        assert nt <= self.max_tokens and x.is_contiguous()
+        if routed is not None:
+            self.ids[:nt].copy_(routed[0])
+            self.weights[:nt].copy_(routed[1])
+            logits = None
+        else:
+            assert logits.is_contiguous()
         L.check(load().maya_moe_prefill_layer(C.byref(self.layout), L._p(expert_table), self.n_expert, self.k, L._p(logits),
                                               L._p(x), L.dtype_id(x), nt, limit, L._p(add), L._p(self.ids), L._p(self.weights),
                                               L._p(self.out), L.dtype_id(self.out), L._p(self.ws), self.ws_bytes,

@@ -247,3 +247,30 @@ def test_down_rounds_h_itself_like_the_quantizer(lib, dt):
         outs.append(out.cpu().numpy())
     assert np.array_equal(outs[0], outs[1])
     assert np.abs(outs[0]).max() > 0
+
+
+def test_layers_take_tokens_that_are_already_routed(lib, oracle):
+    """logits NULL: ids / weights are inputs.  The sigmoid router's ids and weights through the decode layer, the prompt-chunk
+    layer and (in test_gpu_exl3) the EXL3 layer give what the routed layer gives."""
+    from maya_amd import prefill
+    gt, n_embd, n_ff, ne, k, nt = 12, 1024, 512, 10, 3, 6
+    blobs = make_experts(gt, gt, n_embd, n_ff, ne, 321)
+    rng = np.random.default_rng(322)
+    logits = (rng.standard_normal((nt, ne)) * 2).astype(np.float32)
+    bias = (rng.standard_normal(ne) * 0.1).astype(np.float32)
+    x = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    bias_d = dev(bias)
+    ids, w = lib.route_sigmoid(dev(logits), bias_d, k, 2.5, 1)
+    store = lib.ExpertStore(blobs)
+    layer = lib.MoeLayer(gt, gt, n_embd, n_ff, ne, k, max_tokens=nt)
+    a = layer.forward(store.table, dev(logits), x, router=lib.Router(lib.ROUTER_SIGMOID, 1, bias_d.data_ptr(), 2.5)).clone()
+    b = layer.forward(store.table, None, x, routed=(ids, w)).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(layer.ids, ids) and rel_l2(b.cpu().numpy(), a.cpu().numpy()) <= 1e-6 and float(a.abs().max()) > 0
+    # the prompt-chunk layer on the same routing: the same tokens' outputs (another summation order)
+    layout, _ = lib.layout(gt, gt, n_embd, n_ff)
+    pl = prefill.PrefillLayer(layout, ne, k, nt, out_dtype=torch.float32)
+    c = pl.forward(store.table, None, x, limit=0.0, routed=(ids, w))
+    torch.cuda.synchronize()
+    for t in range(nt):
+        assert rel_l2(c[t].cpu().numpy(), a[t].cpu().numpy()) <= 1e-4, t
