@@ -425,6 +425,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
                 __hip_atomic_store(a.h + (size_t) e * n_ff + r0 + r + t, swiglu(g, up, a.limit), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
+    if constexpr (NW < 4) return;   // (the block rounding below wants 256 threads; narrower rows leave it to the down kernel)
     if (a.hq_sync == nullptr) return;
     // The Q8_K rounding of h for the down rows: the last of the 256 / ROWS workgroups that share a 256-value block
     // of h rounds it.  The rows of h are written and read back with device-coherent accesses, so no cache-wide
@@ -440,7 +441,6 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     }
     __syncthreads();
     if (!s_last) return;
-    static_assert(NW >= 4, "the block rounding wants 256 threads");
     const bool active = t < 256;
     const float hv = active ? __hip_atomic_load(a.h + (size_t) e * n_ff + (size_t) blk * 256 + t, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT)
@@ -448,12 +448,13 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     quant_q8k_block(hv, t, active, lds, a.hq, (size_t) e * n_ff + (size_t) blk * 256);
 }
 
-// ---- down + combine, one token, n_ff = 2048 (64 sub-blocks a row = one wave): wave w = plan slot w, rows in batches
-// of 8; grid (n_embd / ROWS).  The slots' rows meet in LDS and are summed in slot order.
-template <int ROWS, int DEPTH, int MINW>
+// ---- down + combine, one token, n_ff = 32 NU <= 2048 (NU sub-blocks a row on the first NU lanes of one wave; NU a
+// multiple of 8, the lanes past it idle): wave w = plan slot w, rows in batches of 8; grid (n_embd / ROWS).  The slots' rows
+// meet in LDS and are summed in slot order.
+template <int ROWS, int DEPTH, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads; the ring holds one or two");
-    constexpr int NU = 64;
+    static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ int lds[kFastLdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
@@ -476,7 +477,10 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
         const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
         const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        const QuadOffs qo = quad_offs<NU>(0u, lane);
+        // (an idle lane reads the last position's weights again and meets them with zero activations)
+        const bool on = NU == 64 || lane < NU;
+        const int pos = on ? lane : NU - 1;
+        const QuadOffs qo = quad_offs<NU>(0u, pos);
         const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
         constexpr int NQ = ROWS / 4;
         QuadIQ2S ring[DEPTH];
@@ -484,25 +488,36 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
         int y[8];
         float dy8;
+        if (!on) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = 0;
+            dy8 = 0.0f;
+        }
         if (a.hq.q) {
-            const int4* q = (const int4*) (a.hq.q + (size_t) ent * 2048);
-            const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
-            y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
-            dy8 = a.hq.d[(size_t) ent * 64 + lane] * 0.125f;
+            if (on) {
+                const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
+                const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+                y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+                dy8 = a.hq.d[(size_t) ent * NU + lane] * 0.125f;
+            }
         } else {
             // no rounded h given: the wave rounds its slot's h to Q8_K itself (quant_q8k_block's arithmetic): a lane holds
             // sub-block `lane`, a 256-value block is 8 lanes; the block's signed maximum is the value at the FIRST largest
             // magnitude - inside a lane the scan keeps the first, between lanes the lower lane wins a tie
-            const float4* hv = (const float4*) (a.h + (size_t) ent * 2048 + 32 * lane);
+            const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
             float v[32];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float4 t = hv[i];
                 v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
             }
+            if (!on) {
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+            }
             float d;
             q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
-            dy8 = d * 0.125f;
+            dy8 = on ? d * 0.125f : 0.0f;
         }
         int yn[8];
 #pragma unroll

@@ -111,12 +111,13 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe
     }
 }
 
-// ---- down + combine, n_ff = 2048 (64 positions a row = one wave): wave w = slot w of token blockIdx.y, rows in batches of 8;
-// grid (n_embd / ROWS, tokens).  Without a rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.
-template <int ROWS, int MINW>
+// ---- down + combine, n_ff = 32 NU <= 2048 (NU positions a row on the first NU lanes of one wave; NU a multiple of 8, the
+// lanes past it idle): wave w = slot w of token blockIdx.y, rows in batches of 8; grid (n_embd / ROWS, tokens).  Without a
+// rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.
+template <int ROWS, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a) {
     static_assert(ROWS % 8 == 0, "rows come in batches of 8");
-    constexpr int NU = 64;
+    static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
     const int n_embd = a.layout.n_embd;
@@ -125,8 +126,11 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
     const int e0 = blockIdx.y * a.k, ent = e0 + wave;
     const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
     if (blob != 0ull) {
+        // (an idle lane reads the last position's weights again and meets them with zero activations)
+        const bool on = NU == 64 || lane < NU;
+        const int pos = on ? lane : NU - 1;
         PosQ4K p;
-        pos_q4k_init(p, lane, 0u);
+        pos_q4k_init(p, pos, 0u);
         // the first row's weights are requested before h is rounded: their latency hides behind that arithmetic
         constexpr uint32_t rb = NU / 8 * 144;
         const uint64_t mat = blob + a.layout.down_off;
@@ -136,19 +140,23 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
         u32x4 hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) r0 * rb, 0);
         u32x4 qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) r0 * rb, 0);
         if (a.hq.q) {
-            pos_q4k_codes(p, lane, a.hq.q + (size_t) ent * 2048, a.hq.d + (size_t) ent * NU, a.hq.bsums + (size_t) ent * (2 * NU));
+            pos_q4k_codes(p, pos, a.hq.q + (size_t) ent * (32 * NU), a.hq.d + (size_t) ent * NU, a.hq.bsums + (size_t) ent * (2 * NU));
         } else {
             // Q8_K of h in registers (quant_q8k_block's arithmetic): the lane's 32 values are two runs of 16, a block is
             // 8 lanes; the block's signed maximum is the value at the FIRST largest magnitude, so candidates carry their index
-            const int piece = lane & 7, j = piece >> 1, half = piece & 1;
-            const int v0 = 256 * (lane >> 3) + 64 * j + 16 * half;
-            const float* hrow = a.h + (size_t) ent * 2048;
+            const int piece = pos & 7, j = piece >> 1, half = piece & 1;
+            const int v0 = 256 * (pos >> 3) + 64 * j + 16 * half;
+            const float* hrow = a.h + (size_t) ent * (32 * NU);
             float v[32];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float4 lo = *(const float4*) (hrow + v0 + 4 * i), hi = *(const float4*) (hrow + v0 + 32 + 4 * i);
                 v[4 * i] = lo.x, v[4 * i + 1] = lo.y, v[4 * i + 2] = lo.z, v[4 * i + 3] = lo.w;
                 v[16 + 4 * i] = hi.x, v[16 + 4 * i + 1] = hi.y, v[16 + 4 * i + 2] = hi.z, v[16 + 4 * i + 3] = hi.w;
+            }
+            if (!on) {
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[i] = 0.0f;
             }
             int y[8];
             float d;
@@ -158,6 +166,12 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
             p.dx = d;
             p.slo = dot4(0x01010101, p.ylo[0], dot4(0x01010101, p.ylo[1], dot4(0x01010101, p.ylo[2], dot4(0x01010101, p.ylo[3], 0))));
             p.shi = dot4(0x01010101, p.yhi[0], dot4(0x01010101, p.yhi[1], dot4(0x01010101, p.yhi[2], dot4(0x01010101, p.yhi[3], 0))));
+        }
+        if (!on) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p.ylo[i] = p.yhi[i] = 0;
+            p.slo = p.shi = 0;
+            p.dx = 0.0f;
         }
         float acc[8];
 #pragma unroll 1

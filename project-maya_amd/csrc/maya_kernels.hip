@@ -1317,10 +1317,14 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
 }
+// the rows the position-mapped down kernels take on one wave: n_ff = 1024, 1536 or 2048
+static bool down_pos_nff_ok(int n_ff) { return n_ff == 1024 || n_ff == 1536 || n_ff == 2048; }
 int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
     const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
-    hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);
+    if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7, 32>), grid, dim3(512), 0, s, a, st.cb);
+    else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7, 48>), grid, dim3(512), 0, s, a, st.cb);
+    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
     return MAYA_OK;
 }
@@ -1345,7 +1349,10 @@ int try_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStre
     if (l.packing == MAYA_PACK_STREAM) {
         if (l.n_ff % 16 != 0) return 0;
         switch (l.n_embd / 1024 * (l.n_embd % 1024 == 0)) {
+            case 2: *rc = launch_gate_up_iq2s_pos<2>(a, st, s); return 1;
+            case 3: *rc = launch_gate_up_iq2s_pos<3>(a, st, s); return 1;
             case 4: *rc = launch_gate_up_iq2s_pos<4>(a, st, s); return 1;
+            case 5: *rc = launch_gate_up_iq2s_pos<5>(a, st, s); return 1;
             case 6: *rc = launch_gate_up_iq2s_pos<6>(a, st, s); return 1;
             case 7: *rc = launch_gate_up_iq2s_pos<7>(a, st, s); return 1;
             case 8: *rc = launch_gate_up_iq2s_pos<8>(a, st, s); return 1;
@@ -1410,15 +1417,15 @@ int launch_down_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStrea
 bool down_rounds_h(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
     if (down_iq1s_pos_ok(a)) return true;
-    if (l.down_type == kQ4_K) return l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
-    return l.down_type == kIQ2_S && a.k <= 8 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 && l.n_embd % 16 == 0;
+    if (l.down_type == kQ4_K) return l.packing == MAYA_PACK_STREAM && a.k <= 8 && down_pos_nff_ok(l.n_ff) && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
+    return l.down_type == kIQ2_S && a.k <= 8 && l.packing == MAYA_PACK_STREAM && down_pos_nff_ok(l.n_ff) && l.n_embd % 16 == 0;
 }
 int try_down_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStream_t s, int* rc) {
     const maya_moe_layout& l = a.layout;
     if (a.k > 8) return 0;
     if (l.packing != MAYA_PACK_STREAM && !fast_1tok(a)) return 0;
     if (l.packing == MAYA_PACK_STREAM) {
-        if (l.n_ff != 2048 || l.n_embd % 16 != 0) return 0;
+        if (!down_pos_nff_ok(l.n_ff) || l.n_embd % 16 != 0) return 0;
         *rc = launch_down_iq2s_pos(a, st, s);
         return 1;
     }
@@ -1433,11 +1440,11 @@ bool gate_up_q4k_pos_ok(const maya_moe_args& a) {
     if (!(l.gate_type == kQ4_K && l.up_type == kQ4_K && l.packing == MAYA_PACK_STREAM)) return false;
     if (l.n_embd % 1024 != 0 || l.n_ff % 16 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
     const int nw = l.n_embd / 1024;
-    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+    return nw >= 2 && nw <= 8;
 }
 bool down_q4k_pos_ok(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    return l.down_type == kQ4_K && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 && l.n_embd % 16 == 0 &&
+    return l.down_type == kQ4_K && l.packing == MAYA_PACK_STREAM && a.k <= 8 && down_pos_nff_ok(l.n_ff) && l.n_embd % 16 == 0 &&
            (l.down_off & 15) == 0;
 }
 int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
@@ -1449,7 +1456,10 @@ int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
     if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 8>), grid, dim3(64 * NWV), 0, s, a);          \
     else hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a);
     switch (a.layout.n_embd / 1024) {
+        case 2: MAYA_Q4(2) break;
+        case 3: MAYA_Q4(3) break;
         case 4: MAYA_Q4(4) break;
+        case 5: MAYA_Q4(5) break;
         case 6: MAYA_Q4(6) break;
         case 7: MAYA_Q4(7) break;
         default: MAYA_Q4(8) break;
@@ -1461,7 +1471,9 @@ int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
 int launch_down_q4k_pos(const maya_moe_args& a, hipStream_t s) {
     constexpr int kRows = 16;
     const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
-    hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8>), grid, dim3(512), 0, s, a);
+    if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8, 32>), grid, dim3(512), 0, s, a);
+    else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8, 48>), grid, dim3(512), 0, s, a);
+    else hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8>), grid, dim3(512), 0, s, a);
     MAYA_LAUNCHED("down_q4k_pos_kernel");
     return MAYA_OK;
 }

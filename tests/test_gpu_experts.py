@@ -73,6 +73,13 @@ CASES = [
     (29, 29, 7168, 2048, 9, 8, 3),
     (29, 19, 6144, 2048, 4, 2, 2),
     (12, 29, 8192, 2048, 4, 3, 2),
+    # other expert shapes on the position-mapped kernels: rows of 2048 / 3072 / 5120 values, n_ff 1024 / 1536 (the down
+    # rows then leave lanes of their wave idle)
+    (22, 22, 5120, 1536, 6, 4, 1),
+    (22, 22, 2048, 1024, 6, 4, 3),
+    (12, 12, 3072, 1536, 5, 3, 2),
+    (22, 12, 5120, 1024, 5, 3, 1),
+    (12, 22, 2048, 1536, 4, 2, 2),
 ]
 
 
