@@ -1883,10 +1883,10 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
 }  // extern "C"
 
 namespace maya {
-// rows of 1024 NW values (NW 2, 4, 6, 7, 8) in whole groups of 16 row pairs; Q8_0 in the stream packing, Q4_K 16-byte aligned
+// rows of 1024 NW values (NW 2 .. 8) in whole groups of 16 row pairs; Q8_0 in the stream packing, Q4_K 16-byte aligned
 static bool mv_pos_ok(const maya_mv_job& j) {
     const int nw = j.n_in / 1024;
-    if (j.n_in % 1024 || !(nw == 2 || nw == 4 || nw == 6 || nw == 7 || nw == 8) || j.n_out % 32 || ((uintptr_t) j.w & 15)) return false;
+    if (j.n_in % 1024 || nw < 2 || nw > 8 || j.n_out % 32 || ((uintptr_t) j.w & 15)) return false;
     if ((size_t) j.n_out * maya_moe_row_bytes(j.type, j.n_in) >= (1ull << 32)) return false;   // (32-bit buffer offsets)
     if (j.type == kQ8_0) return j.packing == MAYA_PACK_STREAM;
     return j.type == kQ4_K;
@@ -1919,7 +1919,9 @@ static void launch_mv_pos_nw(const maya_mv_job& j, hipStream_t s) {
 static void launch_mv_pos(const maya_mv_job& j, hipStream_t s) {
     switch (j.n_in / 1024) {
         case 2: launch_mv_pos_nw<2>(j, s); break;
+        case 3: launch_mv_pos_nw<3>(j, s); break;
         case 4: launch_mv_pos_nw<4>(j, s); break;
+        case 5: launch_mv_pos_nw<5>(j, s); break;
         case 6: launch_mv_pos_nw<6>(j, s); break;
         case 7: launch_mv_pos_nw<7>(j, s); break;
         default: launch_mv_pos_nw<8>(j, s); break;

@@ -56,7 +56,7 @@ POS_CASES = [
     (8, 2048, 64, 1, 1.0, False, 1), (8, 7168, 96, 5, 0.5, True, 1), (8, 4096, 32, 8, 1.0, False, 1), (8, 6144, 64, 16, 1.0, True, 1),
     (8, 8192, 32, 3, 2.0, False, 1), (8, 2048, 16384, 2, 1.0, True, 1),
     (12, 7168, 64, 1, 1.0, True, 0), (12, 2048, 16384, 2, 0.25, False, 0), (12, 4096, 96, 4, 1.0, False, 1), (12, 8192, 32, 1, 1.0, True, 0),
-    (12, 6144, 160, 3, 1.0, False, 0),
+    (12, 6144, 160, 3, 1.0, False, 0), (12, 5120, 64, 2, 1.0, True, 0), (8, 3072, 96, 4, 1.0, False, 1),
 ]
 
 
