@@ -95,15 +95,20 @@ __global__ __launch_bounds__(64 * NW) void gate_up_q80_pos_kernel(maya_moe_args 
     }
 }
 
-// ---- down, n_ff = 2048 (64 block positions a row = one wave): every wave takes its own rows (wg_rows / 8 of them), a step
-// 8 / NT rows for NT entries of the group; writes part[entry][row]; grid (n_embd / wg_rows, groups)
-template <int NT>
+// ---- down, n_ff = 32 NU <= 2048 (NU block positions a row on the first NU lanes of one wave, the lanes past it idle):
+// every wave takes its own rows (wg_rows / 8 of them), a step 8 / NT rows for NT entries of the group; writes
+// part[entry][row]; grid (n_embd / wg_rows, groups)
+template <int NT, int NU = 64>
 __global__ __launch_bounds__(512) void down_q80_pos_kernel(maya_moe_args a, int wg_rows) {
-    constexpr int NU = 64, R = 8 / NT;
+    constexpr int R = 8 / NT;
+    static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "a row on one wave");
     GroupRef gr;
     if (!group_of(a, blockIdx.y, gr)) return;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n_embd = a.layout.n_embd, k = 2048;
+    const int wave = threadIdx.x >> 6, lane0 = threadIdx.x & 63;
+    // (an idle lane reads the last position's weights again and meets them with zero activations)
+    const bool on = NU == 64 || lane0 < NU;
+    const int lane = on ? lane0 : NU - 1;
+    const int n_embd = a.layout.n_embd, k = 32 * NU;
     const int per_wave = wg_rows >> 3, r0 = blockIdx.x * wg_rows + wave * per_wave;
     constexpr uint32_t rb = NU * 34;
     const uint64_t mat = gr.blob + a.layout.down_off;
@@ -113,6 +118,14 @@ __global__ __launch_bounds__(512) void down_q80_pos_kernel(maya_moe_args a, int 
         int ents[NT], y[NT][8];
         float dx[NT];
         q80_chunk<NT>(a, gr, c0, a.hq, false, k, lane, ents, y, dx);
+        if (!on) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) y[t][i] = 0;
+                dx[t] = 0.0f;
+            }
+        }
         for (int r = 0; r < per_wave; r += R) {
             float acc[8];
 #pragma unroll
@@ -124,10 +137,10 @@ __global__ __launch_bounds__(512) void down_q80_pos_kernel(maya_moe_args a, int 
                 const uint32_t db = __builtin_amdgcn_raw_buffer_load_b16(rs, od, ro, 0);
                 q80_values<NT>(qa, qb, db, y, dx, acc, rr * NT);
             }
-            float v = reduce8_half(acc, lane);
+            float v = reduce8_half(acc, lane0);
             v += __shfl_xor(v, 32, kWave);
-            if ((lane & 35) == 0) {
-                const int i = (lane >> 2) & 7, rr = i / NT, tk = i % NT;
+            if ((lane0 & 35) == 0) {
+                const int i = (lane0 >> 2) & 7, rr = i / NT, tk = i % NT;
                 if (ents[tk] >= 0 && r0 + r + rr < n_embd) a.part[(size_t) ents[tk] * n_embd + r0 + r + rr] = v;
             }
         }

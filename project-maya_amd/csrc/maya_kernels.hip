@@ -1483,11 +1483,11 @@ bool gate_up_q80_pos_ok(const maya_moe_args& a) {
     if (!(l.gate_type == kQ8_0 && l.up_type == kQ8_0 && l.packing == MAYA_PACK_STREAM)) return false;
     if (l.n_embd % 1024 != 0 || l.n_ff % 8 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
     const int nw = l.n_embd / 1024;
-    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+    return nw >= 2 && nw <= 8;
 }
 bool down_q80_pos_ok(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    return l.down_type == kQ8_0 && l.packing == MAYA_PACK_STREAM && l.n_ff == 2048 && l.n_embd % 64 == 0 && (l.down_off & 15) == 0;
+    return l.down_type == kQ8_0 && l.packing == MAYA_PACK_STREAM && down_pos_nff_ok(l.n_ff) && l.n_embd % 64 == 0 && (l.down_off & 15) == 0;
 }
 // tokens of a group served by one read of the weights: as many as the call can have in a group, rounded up to 1, 2, 4, 8
 inline int q80_group_tokens(const maya_moe_args& a) {
@@ -1505,7 +1505,10 @@ int launch_gate_up_q80_pos(const maya_moe_args& a, hipStream_t s) {
         default: hipLaunchKernelGGL((gate_up_q80_pos_kernel<NWV, 1, 8>), grid, dim3(64 * NWV), 0, s, a); break; \
     }
     switch (a.layout.n_embd / 1024) {
+        case 2: MAYA_Q8(2) break;
+        case 3: MAYA_Q8(3) break;
         case 4: MAYA_Q8(4) break;
+        case 5: MAYA_Q8(5) break;
         case 6: MAYA_Q8(6) break;
         case 7: MAYA_Q8(7) break;
         default: MAYA_Q8(8) break;
@@ -1523,12 +1526,15 @@ int launch_down_q80_pos(const maya_moe_args& a, hipStream_t s) {
     while (per_wave > step && (long long) (a.layout.n_embd / (per_wave * 8)) * a.n_tokens * a.k < 1024) per_wave >>= 1;
     const int wg_rows = per_wave * 8;
     const dim3 grid((unsigned) ((a.layout.n_embd + wg_rows - 1) / wg_rows), (unsigned) (a.n_tokens * a.k));
-    switch (nt) {
-        case 8: hipLaunchKernelGGL((down_q80_pos_kernel<8>), grid, dim3(512), 0, s, a, wg_rows); break;
-        case 4: hipLaunchKernelGGL((down_q80_pos_kernel<4>), grid, dim3(512), 0, s, a, wg_rows); break;
-        case 2: hipLaunchKernelGGL((down_q80_pos_kernel<2>), grid, dim3(512), 0, s, a, wg_rows); break;
-        default: hipLaunchKernelGGL((down_q80_pos_kernel<1>), grid, dim3(512), 0, s, a, wg_rows); break;
+#define MAYA_DQ(NUV)                                                                                                    \
+    switch (nt) {                                                                                                       \
+        case 8: hipLaunchKernelGGL((down_q80_pos_kernel<8, NUV>), grid, dim3(512), 0, s, a, wg_rows); break;        \
+        case 4: hipLaunchKernelGGL((down_q80_pos_kernel<4, NUV>), grid, dim3(512), 0, s, a, wg_rows); break;        \
+        case 2: hipLaunchKernelGGL((down_q80_pos_kernel<2, NUV>), grid, dim3(512), 0, s, a, wg_rows); break;        \
+        default: hipLaunchKernelGGL((down_q80_pos_kernel<1, NUV>), grid, dim3(512), 0, s, a, wg_rows); break;       \
     }
+    if (a.layout.n_ff == 1024) { MAYA_DQ(32) } else if (a.layout.n_ff == 1536) { MAYA_DQ(48) } else { MAYA_DQ(64) }
+#undef MAYA_DQ
     MAYA_LAUNCHED("down_q80_pos_kernel");
     return MAYA_OK;
 }

@@ -80,6 +80,9 @@ CASES = [
     (12, 12, 3072, 1536, 5, 3, 2),
     (22, 12, 5120, 1024, 5, 3, 1),
     (12, 22, 2048, 1536, 4, 2, 2),
+    (8, 8, 5120, 1536, 3, 2, 1),
+    (8, 8, 3072, 1024, 3, 1, 6),
+    (8, 22, 2048, 1536, 4, 2, 3),
 ]
 
 
