@@ -147,10 +147,10 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1s_pos_kernel(maya_mo
 // ---- down + combine, n_ff = 2048 (64 sub-blocks a row = one wave): wave w = slot w of token blockIdx.y, rows in batches
 // of 8; grid (n_embd / ROWS, tokens).  Without a rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.  The
 // slots' rows meet in LDS and are summed in slot order.
-template <int ROWS, int MINW>
+template <int ROWS, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
-    constexpr int NU = 64;
+    static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ int lds[kFast1LdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
@@ -168,28 +168,41 @@ __global__ __launch_bounds__(512, MINW) void down_iq1s_pos_kernel(maya_moe_args 
         const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
         const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
         const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        const QuadOffs1 qo = quad_offs1<NU>(0u, lane);
+        // (an idle lane - past the row's NU positions - reads the last position's weights again and meets them with zero
+        // activations)
+        const bool on = NU == 64 || lane < NU;
+        const int pos = on ? lane : NU - 1;
+        const QuadOffs1 qo = quad_offs1<NU>(0u, pos);
         const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
         constexpr int NQ = ROWS / 4;
         QuadIQ1S nxt = load_quad1(rs, qo, quad0);
         int y[8];
         float dy8;
         if (a.hq.q) {
-            const int4* q = (const int4*) (a.hq.q + (size_t) ent * 2048);
-            const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+            const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
+            const int4 ya = q[2 * pos], yb = q[2 * pos + 1];
             y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
-            dy8 = a.hq.d[(size_t) ent * 64 + lane] * 0.125f;
+            dy8 = a.hq.d[(size_t) ent * NU + pos] * 0.125f;
         } else {
-            const float4* hv = (const float4*) (a.h + (size_t) ent * 2048 + 32 * lane);
+            const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
             float v[32];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float4 t = hv[i];
                 v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
             }
+            if (!on) {
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+            }
             float d;
             q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
             dy8 = d * 0.125f;
+        }
+        if (!on) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = 0;
+            dy8 = 0.0f;
         }
         const int sy = sum32_codes(y);
         float acc[8];
@@ -360,10 +373,10 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1m_pos_kernel(maya_mo
 // ---- down + combine, n_ff = 2048 (64 sub-blocks a row = one wave): wave w = slot w of token blockIdx.y, rows in batches
 // of 8; grid (n_embd / ROWS, tokens).  Without a rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.  The
 // slots' rows meet in LDS and are summed in slot order.
-template <int ROWS, int MINW>
+template <int ROWS, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq1m_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
-    constexpr int NU = 64;
+    static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ int lds[kFast1LdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
@@ -381,28 +394,41 @@ __global__ __launch_bounds__(512, MINW) void down_iq1m_pos_kernel(maya_moe_args 
         const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
         const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
         const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        const QuadOffsM qo = quad_offsm<NU>(0u, lane);
+        // (an idle lane - past the row's NU positions - reads the last position's weights again and meets them with zero
+        // activations)
+        const bool on = NU == 64 || lane < NU;
+        const int pos = on ? lane : NU - 1;
+        const QuadOffsM qo = quad_offsm<NU>(0u, pos);
         const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
         constexpr int NQ = ROWS / 4;
         QuadIQ1M nxt = load_quadm(rs, qo, quad0);
         int y[8];
         float dy8;
         if (a.hq.q) {
-            const int4* q = (const int4*) (a.hq.q + (size_t) ent * 2048);
-            const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
+            const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
+            const int4 ya = q[2 * pos], yb = q[2 * pos + 1];
             y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
-            dy8 = a.hq.d[(size_t) ent * 64 + lane] * 0.125f;
+            dy8 = a.hq.d[(size_t) ent * NU + pos] * 0.125f;
         } else {
-            const float4* hv = (const float4*) (a.h + (size_t) ent * 2048 + 32 * lane);
+            const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
             float v[32];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float4 t = hv[i];
                 v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
             }
+            if (!on) {
+#pragma unroll
+                for (int i = 0; i < 32; ++i) v[i] = 0.0f;
+            }
             float d;
             q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
             dy8 = d * 0.125f;
+        }
+        if (!on) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = 0;
+            dy8 = 0.0f;
         }
         int sy8[4];
         sums8_codes(y, sy8);

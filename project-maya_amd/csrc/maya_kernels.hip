@@ -1377,17 +1377,20 @@ bool gate_up_iq1s_pos_ok(const maya_moe_args& a) {
     if (!((l.gate_type == kIQ1_S || l.gate_type == kIQ1_M) && l.up_type == l.gate_type && l.packing == MAYA_PACK_STREAM)) return false;
     if (l.n_embd % 1024 != 0 || l.n_ff % 16 != 0 || ((l.gate_off | l.up_off | l.down_off) & 15)) return false;
     const int nw = l.n_embd / 1024;
-    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
+    return nw >= 2 && nw <= 8;
 }
 bool down_iq1s_pos_ok(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
-    return (l.down_type == kIQ1_S || l.down_type == kIQ1_M) && l.packing == MAYA_PACK_STREAM && a.k <= 8 && l.n_ff == 2048 &&
-           l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
+    return (l.down_type == kIQ1_S || l.down_type == kIQ1_M) && l.packing == MAYA_PACK_STREAM && a.k <= 8 &&
+           (l.n_ff == 1024 || l.n_ff == 1536 || l.n_ff == 2048) && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
 }
 int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     const dim3 grid((unsigned) (a.layout.n_ff / 16), (unsigned) (a.n_tokens * a.k));
     if (a.layout.gate_type == kIQ1_M) {
         switch (a.layout.n_embd / 1024) {
+            case 2: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<2, 16, 8>), grid, dim3(128), 0, s, a, st.cb); break;
+            case 3: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<3, 16, 8>), grid, dim3(192), 0, s, a, st.cb); break;
+            case 5: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<5, 16, 8>), grid, dim3(320), 0, s, a, st.cb); break;
             case 4: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
             case 6: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
             case 7: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<7, 16, 8>), grid, dim3(448), 0, s, a, st.cb); break;
@@ -1397,6 +1400,9 @@ int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
         return MAYA_OK;
     }
     switch (a.layout.n_embd / 1024) {
+        case 2: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<2, 16, 8>), grid, dim3(128), 0, s, a, st.cb); break;
+        case 3: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<3, 16, 8>), grid, dim3(192), 0, s, a, st.cb); break;
+        case 5: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<5, 16, 8>), grid, dim3(320), 0, s, a, st.cb); break;
         case 4: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
         case 6: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
         case 7: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<7, 16, 8>), grid, dim3(448), 0, s, a, st.cb); break;
@@ -1407,8 +1413,11 @@ int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 }
 int launch_down_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     const dim3 grid((unsigned) (a.layout.n_embd / 16), (unsigned) a.n_tokens);
-    if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
-    else hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7>), grid, dim3(512), 0, s, a, st.cb);
+#define MAYA_D1(NUV)                                                                                                     \
+    if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<16, 7, NUV>), grid, dim3(512), 0, s, a, st.cb); \
+    else hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7, NUV>), grid, dim3(512), 0, s, a, st.cb);
+    if (a.layout.n_ff == 1024) { MAYA_D1(32) } else if (a.layout.n_ff == 1536) { MAYA_D1(48) } else { MAYA_D1(64) }
+#undef MAYA_D1
     MAYA_LAUNCHED("down_iq1s_pos_kernel");
     return MAYA_OK;
 }

@@ -83,6 +83,9 @@ CASES = [
     (8, 8, 5120, 1536, 3, 2, 1),
     (8, 8, 3072, 1024, 3, 1, 6),
     (8, 22, 2048, 1536, 4, 2, 3),
+    (19, 19, 5120, 1536, 4, 3, 1),
+    (29, 29, 3072, 1024, 4, 2, 2),
+    (19, 29, 2048, 1536, 3, 2, 3),
 ]
 
 
