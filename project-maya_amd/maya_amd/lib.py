@@ -304,6 +304,45 @@ class MoeLayer:
         return self.out[:nt]
 
 
+class DenseExpert:
+    """The expert every token takes (a shared expert, a dense FFN) through the stage entry points: its plan is static - all
+    n tokens on one blob, weight 1, one group - so it is made once here and a step is quantize x -> gate/up -> quantize h
+    -> down -> combine, with no routing, plan or grouping launch (the reference runs the shared expert's rows as extra
+    blocks of the routed experts' launches, include/strata/kernels/glm_fast.hpp:496-501)."""
+
+    def __init__(self, gate_type, down_type, n_embd, n_ff, n_tokens, blob_addr, packing=PACK_GGUF, device="cuda"):
+        self.gguf_layout, self.blob_bytes = layout(gate_type, down_type, n_embd, n_ff)
+        self.layout = copy_layout(self.gguf_layout, packing)
+        self.n, self.n_embd, self.n_ff = n_tokens, n_embd, n_ff
+        n = n_tokens
+        self.plan_ptr = torch.full((n,), blob_addr, dtype=torch.int64, device=device)
+        self.plan_w = torch.ones(n, dtype=torch.float32, device=device)
+        self.grp_ptr, self.grp_start, self.grp_ent, self.n_groups = group(self.plan_ptr)
+        self.xq, self.hq = ActBuf(n, n_embd, device), ActBuf(n, n_ff, device)
+        self.h = torch.empty((n, n_ff), dtype=torch.float32, device=device)
+        self.part = torch.empty((n, n_embd), dtype=torch.float32, device=device)
+        self.out = torch.empty((n, n_embd), dtype=torch.float32, device=device)
+        a = Args()
+        a.layout = self.layout
+        a.n_tokens, a.k = n, 1
+        a.plan_ptr, a.plan_w = self.plan_ptr.data_ptr(), self.plan_w.data_ptr()
+        a.grp_ptr, a.grp_start = self.grp_ptr.data_ptr(), self.grp_start.data_ptr()
+        a.grp_ent, a.n_groups = self.grp_ent.data_ptr(), self.n_groups.data_ptr()
+        a.x, a.h, a.hq = self.xq.c(), self.h.data_ptr(), self.hq.c()
+        a.part, a.out = self.part.data_ptr(), self.out.data_ptr()
+        self.args = a
+
+    def forward(self, x, limit=float("inf"), stream=None):
+        assert x.shape == (self.n, self.n_embd) and x.is_contiguous()
+        L, a, s = load(), self.args, _stream(stream)
+        a.limit = limit
+        check(L.maya_quant_act(self.layout.gate_type, _p(x), dtype_id(x), 0, self.n, self.n_embd, self.xq.c(), s))
+        check(L.maya_moe_gate_up(C.byref(a), s))
+        check(L.maya_quant_act(self.layout.down_type, _p(self.h), 0, 0, self.n, self.n_ff, self.hq.c(), s))
+        check(L.maya_moe_down(C.byref(a), s))
+        return self.out
+
+
 def mv(jobs, stream=None):
     """jobs: dicts with w (uint8 rows), type, x [ncol, n_in] float activations, n_out and optionally packing, alpha, bias,
     y; quantizes each x to the type's activation format and runs ONE maya_mv call.  Returns the outputs [ncol, n_out]."""

@@ -126,8 +126,9 @@ def batch8_mixed(K, W):
         staging.copy_(sh_pool[c * shared.blob_bytes:(c + 1) * shared.blob_bytes])
         lib.repack(shared.gguf_layout, staging, sh_pool[c * shared.blob_bytes:(c + 1) * shared.blob_bytes])
     torch.cuda.synchronize()
-    sh_tables = [torch.tensor([sh_pool.data_ptr() + c * shared.blob_bytes], dtype=torch.int64, device="cuda") for c in range(n_sh)]
-    sh_logits = torch.zeros((T, 1), device="cuda")
+    # (the shared expert's plan is static - every token, weight 1 - so it runs through the stage calls without routing)
+    dense = [lib.DenseExpert(lib.Q8_0, lib.Q8_0, E, FF, T, sh_pool.data_ptr() + c * shared.blob_bytes, packing=lib.PACK_STREAM)
+             for c in range(n_sh)]
     rng = np.random.default_rng(9)
     n_sets = 8
     logits = torch.from_numpy(rng.standard_normal((n_sets, T, NE)).astype(np.float32)).cuda()
@@ -139,7 +140,7 @@ def batch8_mixed(K, W):
     stream = torch.cuda.Stream()
 
     def step(i):
-        sh = shared.forward(sh_tables[i % n_sh], sh_logits, x)
+        sh = dense[i % n_sh].forward(x)
         layer.forward(table, logits[i % n_sets], x, add=sh)
 
     dt = timed_graph(step, K, W, stream)

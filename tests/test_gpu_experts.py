@@ -287,3 +287,22 @@ def test_layers_take_tokens_that_are_already_routed(lib, oracle):
     torch.cuda.synchronize()
     for t in range(nt):
         assert rel_l2(c[t].cpu().numpy(), a[t].cpu().numpy()) <= 1e-4, t
+
+
+def test_dense_expert_through_the_stage_calls(lib, oracle):
+    """The expert every token takes, with a static plan and no routing launch: the same rows as a k = 1 layer over one expert."""
+    t, n_embd, n_ff, nt = 8, 4096, 2048, 5
+    blobs = make_experts(t, t, n_embd, n_ff, 1, 77)
+    gguf, _ = lib.layout(t, t, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf)
+    rng = np.random.default_rng(78)
+    x = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    dense = lib.DenseExpert(t, t, n_embd, n_ff, nt, int(store.table[0].item()), packing=lib.PACK_STREAM)
+    a = dense.forward(x, limit=6.0).clone()
+    layer = lib.MoeLayer(t, t, n_embd, n_ff, 1, 1, max_tokens=nt, packing=lib.PACK_STREAM)
+    b = layer.forward(store.table, dev(np.zeros((nt, 1), dtype=np.float32)), x, limit=6.0)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and float(a.abs().max()) > 0
+    want = oracle.expert(t, t, blobs[0], blobs[0][gguf.up_off:], blobs[0][gguf.down_off:], n_embd, n_ff, x.cpu().numpy(), 6.0)
+    for i in range(nt):
+        assert rel_l2(a[i].cpu().numpy(), want[i]) <= TOL, i
