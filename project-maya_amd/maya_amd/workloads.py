@@ -226,11 +226,11 @@ def _prefill(K, W, gt, dt, what, types):
                          "algorithmic_ops_per_launch": ops_gu, "avg_launch_us": round(sec_gu * 1e6, 1)}}
 
 
-def exl3_verify(K, W):
+def exl3_verify(K, W, k2=6):
     """configs[4]: 160 EXL3 experts (3 bits a weight: k2 = 6, mul1 codebook), top-8, hidden 6144, intermediate 1536, a
-    4-token verify window; 8 logit sets rotate."""
+    4-token verify window; 8 logit sets rotate.  (k2 = 8, 10: the same layer at 4 and 5 bits a weight.)"""
     E, FF, NE, TK, T = 6144, 1536, 160, 8, 4
-    l, bb = exl3.make_layout(E, FF, 6, exl3.CB_MUL1)
+    l, bb = exl3.make_layout(E, FF, k2, exl3.CB_MUL1)
     stride = (bb + 255) & ~255
     pool = random_blocks(NE * stride, 256, {}, 13)
     view = pool.view(NE, stride)
@@ -260,11 +260,13 @@ def exl3_verify(K, W):
     sec = dt / K
     return {"metric": "exl3_moe_layer_hbm_gbps_4tok", "value": round(nbytes / sec / 1e9, 2), "unit": "GB/s", "ms_per_step": sec * 1e3,
             "dtype": "f16",
-            "config": {"workload": "configs[4]: EXL3 3-bit trellis experts (k2 6, mul1), 160 experts top-8, hidden 6144, "
+            "config": {"workload": ("configs[4]" if k2 == 6 else "configs[4] at another bit rate") +
+                                   ": EXL3 %g-bit trellis experts (k2 %d, mul1), 160 experts top-8, hidden 6144, " % (k2 / 2, k2) +
                                    "intermediate 1536, 4-token verify window; 8 logit sets rotate",
                        "distinct_experts_per_step": d_avg, "algorithmic_bytes_per_step": int(nbytes)},
             "roofline": hbm_roofline("layer (exl3_gu_split_kernel + exl3_swiglu_kernel + exl3_down_kernel + exl3_combine_kernel)", nbytes, sec)}
 
 
 WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify,
-             "prefill_iq2s": prefill_iq2s, "prefill_mixed": prefill_mixed}
+             "prefill_iq2s": prefill_iq2s, "prefill_mixed": prefill_mixed,
+             "exl3_verify_4bit": lambda K, W: exl3_verify(K, W, 8), "exl3_verify_5bit": lambda K, W: exl3_verify(K, W, 10)}
