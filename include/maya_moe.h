@@ -178,6 +178,12 @@ int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, 
 #define MAYA_ROUTER_NORM_HF 2
 int maya_moe_route_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
                            int32_t* ids, float* weights, void* stream);
+/* Route and plan in one launch (router NULL: the softmax router; else see maya_router below): ids, weights and
+ * plan_ptr[e] = expert_table[ids[e]] - the routing and look-up of glmf::moe_route (include/strata/kernels/glm_fast.hpp:424-433)
+ * without its residency tiers. */
+struct maya_router;
+int maya_moe_route_plan(const struct maya_router* router, const float* logits, int n_tokens, int n_expert, int k,
+                        const uint64_t* expert_table, int32_t* ids, float* weights, uint64_t* plan_ptr, void* stream);
 /* ids -> plan: plan_ptr[e] = expert_table[ids[e]] (0 stays 0: not resident), the plan part of moe_route_kernel
  * (src/kernels/cuda/glm_fast.cu:3998-4545) without its residency tiers. */
 int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,

@@ -694,8 +694,9 @@ int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_tab
     const Exl3Ws w = exl3_carve(*l, n_tokens, k, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "exl3 layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     int rc;
-    if (logits && (rc = maya_moe_route_topk(logits, n_tokens, n_expert, k, ids, weights, stream))) return rc;   // (null: ids / weights are given)
-    if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+    if (logits) {   // route and plan in one launch; null: ids / weights are given
+        if ((rc = maya_moe_route_plan(nullptr, logits, n_tokens, n_expert, k, expert_table, ids, weights, w.plan_ptr, stream))) return rc;
+    } else if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
     maya_exl3_args a{};
     a.layout = *l;
     a.n_tokens = n_tokens;

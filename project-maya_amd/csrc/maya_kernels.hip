@@ -1800,6 +1800,22 @@ int maya_moe_route_sigmoid(const float* logits, const float* bias, int n_tokens,
     return route_impl("route_sigmoid", logits, n_tokens, n_expert, k, RouterSpec{bias, w_scale, MAYA_ROUTER_SIGMOID, norm}, ids, weights, stream);
 }
 
+int maya_moe_route_plan(const maya_router* router, const float* logits, int n_tokens, int n_expert, int k, const uint64_t* expert_table,
+                        int32_t* ids, float* weights, uint64_t* plan_ptr, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    RouterSpec rs;
+    if (!router_spec(router, rs)) return fail(MAYA_E_UNSUPPORTED, "route_plan: router kind %d / normalisation %d", router->kind, router->norm);
+    if (!logits || !expert_table || !ids || !weights || !plan_ptr) return fail(MAYA_E_ARG, "route_plan: null pointer");
+    if (n_tokens <= 0 || n_tokens > 65535 || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k <= 0 || k > MAYA_MAX_K || k > n_expert)
+        return fail(MAYA_E_SHAPE, "route_plan: tokens %d experts %d k %d (limits %d experts, k %d)", n_tokens, n_expert, k, MAYA_MAX_EXPERTS, MAYA_MAX_K);
+    // (the layer head's routing workgroup alone: no activation blocks, no counters)
+    hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, dim3(1, (unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, rs,
+                       expert_table, ids, weights, plan_ptr, nullptr, (int64_t) 0, maya_act{nullptr, nullptr, nullptr}, nullptr, 0);
+    MAYA_LAUNCHED("layer_head_kernel");
+    return MAYA_OK;
+}
+
 int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,
                   void* stream) {
     DeviceState* st;
@@ -2086,8 +2102,12 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
         MAYA_LAUNCHED("layer_head_kernel");
         a.hq_sync = down_rounds_h(a) ? nullptr : w.hq_sync;   // (the down kernel's own rounding of h is the cheaper one)
     } else {
-        if (logits && (rc = route_impl("layer_decode", logits, n_tokens, n_expert, k, rs, ids, weights, stream))) return rc;   // (null: ids / weights are given)
-        if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+        if (logits && n_expert <= MAYA_MAX_EXPERTS) {
+            if ((rc = maya_moe_route_plan(router, logits, n_tokens, n_expert, k, expert_table, ids, weights, w.plan_ptr, stream))) return rc;
+        } else {
+            if (logits && (rc = route_impl("layer_decode", logits, n_tokens, n_expert, k, rs, ids, weights, stream))) return rc;   // (null: ids / weights are given)
+            if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
+        }
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }
     if (n_tokens > 1 && !(gate_up_by_entries(a) && down_by_entries(a))) {

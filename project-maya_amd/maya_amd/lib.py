@@ -18,7 +18,7 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
-    "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed",
+    "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan",
     "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
 
@@ -102,6 +102,7 @@ def load():
     L.maya_moe_layer_decode_routed.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32, vp, vp, vp,
                                                vp, vp, sz, vp]
     L.maya_moe_route_sigmoid.argtypes = [vp, vp, i32, i32, i32, f32, i32, vp, vp, vp]
+    L.maya_moe_route_plan.argtypes = [C.POINTER(Router), vp, i32, i32, i32, vp, vp, vp, vp, vp]
     _lib = L
     return L
 
@@ -212,6 +213,17 @@ def route_sigmoid(logits, bias, k, w_scale=1.0, norm=NORM_CLAMP, stream=None):
     w = torch.empty((nt, k), dtype=torch.float32, device=logits.device)
     check(load().maya_moe_route_sigmoid(_p(logits), _p(bias), nt, ne, k, w_scale, norm, _p(ids), _p(w), _stream(stream)))
     return ids, w
+
+
+def route_plan(logits, k, expert_table, router=None, stream=None):
+    """ids, weights and the plan (blob addresses) in one launch."""
+    nt, ne = logits.shape
+    ids = torch.empty((nt, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((nt, k), dtype=torch.float32, device=logits.device)
+    pl = torch.empty(nt * k, dtype=torch.int64, device=logits.device)
+    check(load().maya_moe_route_plan(None if router is None else C.byref(router), _p(logits), nt, ne, k, _p(expert_table), _p(ids),
+                                     _p(w), _p(pl), _stream(stream)))
+    return ids, w, pl
 
 
 def plan(ids, expert_table, stream=None):

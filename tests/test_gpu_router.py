@@ -145,3 +145,18 @@ def test_sigmoid_router_ties_bias_and_tiny_sums(lib, oracle):
     o = torch.zeros((1, 8), device="cuda")
     assert L.maya_moe_route_sigmoid(x.data_ptr(), 0, 1, 8, 8, 1.0, 3, o.data_ptr(), o.data_ptr(), 0) == 1   # MAYA_E_UNSUPPORTED
     assert L.maya_moe_route_sigmoid(x.data_ptr(), 0, 1, 8, 9, 1.0, 1, o.data_ptr(), o.data_ptr(), 0) == 2   # k > experts
+
+
+def test_route_plan_in_one_launch(lib):
+    rng = np.random.default_rng(31)
+    for ne, k, nt in ((256, 8, 5), (300, 6, 3), (8, 2, 1)):
+        logits = torch.from_numpy(rng.standard_normal((nt, ne)).astype(np.float32)).cuda()
+        table = (torch.arange(1, ne + 1, dtype=torch.int64, device="cuda") * 4096)
+        table[::7] = 0
+        bias = torch.from_numpy((rng.standard_normal(ne) * 0.1).astype(np.float32)).cuda()
+        for router in (None, lib.Router(lib.ROUTER_SIGMOID, 1, bias.data_ptr(), 2.5)):
+            ids, w, pl = lib.route_plan(logits, k, table, router)
+            wi, ww = lib.route_topk(logits, k) if router is None else lib.route_sigmoid(logits, bias, k, 2.5, 1)
+            torch.cuda.synchronize()
+            assert torch.equal(ids, wi) and torch.equal(w, ww)
+            assert torch.equal(pl, lib.plan(wi.reshape(-1), table))
