@@ -159,6 +159,12 @@ def main():
     lib.check(L.maya_init())
     info = L.maya_device_info().decode()
     torch.cuda.set_device(0)
+    if args.calib_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.workload != "decode_iq2s":
         from maya_amd import workloads
         if args.workload not in workloads.WORKLOADS:
@@ -189,13 +195,6 @@ def main():
     rng = np.random.default_rng(11)
     x = torch.from_numpy(rng.standard_normal((1, N_EMBD)).astype(np.float32)).to(torch.bfloat16).cuda()
     torch.cuda.synchronize()
-
-    if args.calib_copy:
-        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     stream = torch.cuda.Stream()
     K, W = args.steps, args.warmup

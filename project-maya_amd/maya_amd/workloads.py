@@ -69,10 +69,17 @@ def event_time(fn, reps, stream):
         return e0.elapsed_time(e1) * 1e-3 / reps
 
 
-def hbm_roofline(kernel, bytes_launch, seconds):
+# HBM bytes a step (a launch of the named kernel for the prefill chunks) read from rocprofv3's FETCH_SIZE and WRITE_SIZE
+# counters, scaled by a plain copy of known size (profiles/other_configs_hbm_traffic_pmc.txt); they belong to the
+# synthetic inputs these workloads make (fixed seeds), so they are constants here
+TRAFFIC_BYTES = {"single_q4k": 25286343, "batch8_mixed": 1185852494, "exl3_verify": 336937077,
+                 "prefill_q4k": 2122985062, "prefill_iq2s": 1253165670, "prefill_mixed": 1253165670}
+
+
+def hbm_roofline(kernel, bytes_launch, seconds, traffic=None):
     rate = bytes_launch / seconds / 1e9
     return {"bound": "hbm", "kernel": kernel, "achieved": round(rate, 2), "peak": 8000.0, "unit": "GB/s",
-            "frac": round(rate * 1e9 / HBM_PEAK, 4), "traffic": None, "algorithmic_bytes_per_launch": int(bytes_launch),
+            "frac": round(rate * 1e9 / HBM_PEAK, 4), "traffic": traffic, "algorithmic_bytes_per_launch": int(bytes_launch),
             "avg_launch_us": round(seconds * 1e6, 3)}
 
 
@@ -96,7 +103,7 @@ def single_q4k(K, W):
             "config": {"workload": "configs[0]: one expert GLU, gate/up [2048x7168] + down [7168x2048] Q4_K (constructed "
                                    "blocks), 1 token F32; 16 copies of the expert rotate over the steps",
                        "algorithmic_bytes_per_step": nbytes},
-            "roofline": hbm_roofline("layer (layer_head_kernel + gate_up_q4k_pos_kernel + down_q4k_pos_kernel)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (layer_head_kernel + gate_up_q4k_pos_kernel + down_q4k_pos_kernel)", nbytes, sec, TRAFFIC_BYTES["single_q4k"])}
 
 
 def batch8_mixed(K, W):
@@ -152,7 +159,7 @@ def batch8_mixed(K, W):
             "config": {"workload": "configs[2]: 8 tokens, 256 experts top-8 (gate/up IQ2_S, down Q4_K) + a Q8_0 shared expert; "
                                    "8 logit sets rotate", "distinct_experts_per_step": d_avg,
                        "algorithmic_bytes_per_step": int(nbytes)},
-            "roofline": hbm_roofline("layer (routed gate_up_iq2s_pos_kernel + down_q4k_pos_kernel over 64 entries, shared expert gate_up_q80_pos_kernel + down_q80_pos_kernel)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (routed gate_up_iq2s_pos_kernel + down_q4k_pos_kernel over 64 entries, shared expert gate_up_q80_pos_kernel + down_q80_pos_kernel)", nbytes, sec, TRAFFIC_BYTES["batch8_mixed"])}
 
 
 BLOCK_FIELDS = {lib.Q4_K: (144, {0: (2e-4, 6e-4), 2: (2e-4, 6e-4)}), 22: (82, {0: (2e-3, 6e-3)})}
@@ -222,7 +229,8 @@ def _prefill(K, W, gt, dt, what, types):
                        "pct_of_hbm_peak": round(100 * nbytes / sec / HBM_PEAK, 2)},
             "roofline": {"bound": "mfma", "kernel": ("prefill_q4k_kernel" if gt == lib.Q4_K else "prefill_iq2s_kernel") + "<gate_up>",
                          "achieved": round(tops_gu, 2), "peak": 5000.0,
-                         "unit": "TOP/s", "frac": round(tops_gu * 1e12 / INT8_PEAK, 4), "traffic": None,
+                         "unit": "TOP/s", "frac": round(tops_gu * 1e12 / INT8_PEAK, 4),
+                         "traffic": TRAFFIC_BYTES["prefill_q4k" if gt == lib.Q4_K else "prefill_iq2s"],
                          "algorithmic_ops_per_launch": ops_gu, "avg_launch_us": round(sec_gu * 1e6, 1)}}
 
 
@@ -264,7 +272,8 @@ def exl3_verify(K, W, k2=6):
                                    ": EXL3 %g-bit trellis experts (k2 %d, mul1), 160 experts top-8, hidden 6144, " % (k2 / 2, k2) +
                                    "intermediate 1536, 4-token verify window; 8 logit sets rotate",
                        "distinct_experts_per_step": d_avg, "algorithmic_bytes_per_step": int(nbytes)},
-            "roofline": hbm_roofline("layer (exl3_gu_split_kernel + exl3_swiglu_kernel + exl3_down_kernel + exl3_combine_kernel)", nbytes, sec)}
+            "roofline": hbm_roofline("layer (exl3_gu_split_kernel + exl3_swiglu_kernel + exl3_down_kernel + exl3_combine_kernel)", nbytes, sec,
+                                     TRAFFIC_BYTES["exl3_verify"] if k2 == 6 else None)}
 
 
 WORKLOADS = {"single_q4k": single_q4k, "batch8_mixed": batch8_mixed, "prefill_q4k": prefill_q4k, "exl3_verify": exl3_verify,
