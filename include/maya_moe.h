@@ -172,7 +172,10 @@ int maya_moe_route_topk(const float* logits, int n_tokens, int n_expert, int k, 
  * glmf::moe_route (include/strata/kernels/glm_fast.hpp:420-433): p = sigmoid(logits) in float, ids = the stable top-k of
  * p + bias (bias NULL or [n_expert]: it chooses, it does not weigh; ties to the lower index), weights = p / D * w_scale with
  * D = max(sum of the k chosen p, 2^-14) (norm MAYA_ROUTER_NORM_CLAMP = kRouteNormClamp), sum + 1e-20 (MAYA_ROUTER_NORM_HF =
- * kRouteNormHf) or 1 (MAYA_ROUTER_NORM_NONE: norm_topk_prob off). */
+ * kRouteNormHf) or 1 (MAYA_ROUTER_NORM_NONE: norm_topk_prob off).
+ * A token with a non-finite logit or score (NaN, +-Inf; a bias counts) is refused as the engine's routers refuse it
+ * (route_kernel, src/kernels/cuda/glm_batch.cu:2077-2092; moe_route_kernel, glm_fast.cu:4040, 4136-4141): ids -1, weights 0, so
+ * the plans made from them hold no expert for it and a layer gives it the added part alone. */
 #define MAYA_ROUTER_NORM_NONE 0
 #define MAYA_ROUTER_NORM_CLAMP 1
 #define MAYA_ROUTER_NORM_HF 2

@@ -624,6 +624,17 @@ static void router_sigmoid_impl(const float* logits, const float* bias, int n_to
             pd[e] = 1.0 / (1.0 + exp(-(double) l[e]));
             sd[e] = bias ? pd[e] + (double) bias[e] : pd[e];
         }
+        /* a row with a non-finite logit or selection score is refused: no routes (ids -1, weights 0), as the engine's
+         * routers do (route_kernel src/kernels/cuda/glm_batch.cu:2077-2092; moe_route_kernel glm_fast.cu:4040) */
+        int bad = 0;
+        for (int e = 0; e < n_expert; ++e) bad |= !isfinite(l[e]) || !isfinite(sel[e]);
+        if (bad) {
+            for (int i = 0; i < k; ++i) {
+                ids[(size_t) t * k + i] = -1;
+                weights[(size_t) t * k + i] = 0.0f;
+            }
+            continue;
+        }
         for (int e = 0; e < n_expert; ++e) {
             int rank = 0;
             for (int f = 0; f < n_expert; ++f) {

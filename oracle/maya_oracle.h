@@ -119,7 +119,8 @@ void mo_expert(int gu_type, int d_type, const uint8_t* gate, const uint8_t* up, 
 void mo_router_topk(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights);
 void mo_router_topk_f64(const float* logits, int n_tokens, int n_expert, int k, int32_t* ids, float* weights);
 /* ---- the sigmoid router (src/kernels/cuda/router_sigmoid.cu:44-73, moe_route_kernel src/kernels/cuda/glm_fast.cu:4050-4297;
- * host form src/kernels/router_sigmoid_parity.cpp:36-86).  norm: 0 none, 1 / max(sum, 2^-14), 2 / (sum + 1e-20) */
+ * host form src/kernels/router_sigmoid_parity.cpp:36-86).  norm: 0 none, 1 / max(sum, 2^-14), 2 / (sum + 1e-20).
+ * A row with a non-finite logit or score gets ids -1 and weights 0 (src/kernels/cuda/glm_batch.cu:2077-2092). */
 void mo_router_sigmoid(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
                        int32_t* ids, float* weights);
 void mo_router_sigmoid_f64(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,

@@ -697,12 +697,18 @@ __device__ __forceinline__ void sigmoid_narrow(int n_expert, int k, const Router
 __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l, int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
     const int tid = threadIdx.x;
     float* sel = (float*) sm.ex;
+    int bad = 0;
     for (int e = tid; e < n_expert; e += 256) {
-        const float p = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-l[e])));
+        const float le = l[e];
+        const float p = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-le)));
+        const float sc = r.bias ? __fadd_rn(p, r.bias[e]) : p;
         sm.p[e] = p;
-        sel[e] = r.bias ? __fadd_rn(p, r.bias[e]) : p;
+        sel[e] = sc;
+        bad |= !isfinite(le) || !isfinite(sc);
     }
-    __syncthreads();
+    // a row with a non-finite logit or score is refused: no routes (the engine's routers,
+    // src/kernels/cuda/glm_batch.cu:2077-2092, glm_fast.cu:4040); it is still ranked below, its picks unused
+    bad = __syncthreads_or(bad);
     if (n_expert <= 256) {
         if (tid < 64) sigmoid_narrow(n_expert, k, r, sm);
     } else {
@@ -727,7 +733,10 @@ __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l,
         double s = 0.0;
         for (int i = 0; i < k; ++i) s += (double) __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
         const float inv = (float) (r.norm == 0 ? 1.0 : r.norm == 2 ? 1.0 / (s + 1e-20) : 1.0 / fmax(s, 6.103515625e-05));
-        if (tid < k) sm.w[tid] = (float) ((double) p * (double) inv * (double) r.w_scale);
+        if (tid < k) {
+            sm.w[tid] = bad ? 0.0f : (float) ((double) p * (double) inv * (double) r.w_scale);
+            if (bad) sm.id[tid] = -1;
+        }
     }
     __syncthreads();
 }

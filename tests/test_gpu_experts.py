@@ -128,6 +128,29 @@ def test_layer_with_the_sigmoid_router(lib, oracle, gt, dt, n_embd, n_ff, ne, k,
         assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
 
 
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt,packing", (
+    (22, 22, 7168, 2048, 9, 8, 1, 1), (22, 22, 1024, 512, 16, 4, 3, 0), (12, 12, 4096, 2048, 6, 4, 3, 1), (22, 12, 1024, 768, 300, 8, 2, 0)))
+def test_layer_refuses_a_token_with_non_finite_logits(lib, gt, dt, n_embd, n_ff, ne, k, nt, packing):
+    """A token whose router row holds a NaN gets no routes: ids -1, weights 0, and its output is the added part alone; the
+    other tokens' outputs are bit for bit what the layer gives without the bad row's NaN."""
+    seed = gt * 100 + dt + nt + 3
+    blobs = make_experts(gt, dt, n_embd, n_ff, min(ne, 12), seed)
+    blobs = [blobs[i % len(blobs)] for i in range(ne)]
+    rng = np.random.default_rng(seed + 1)
+    logits = (rng.standard_normal((nt, ne)) * 2).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    add = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    router = lib.Router(lib.ROUTER_SIGMOID, 1, 0, 2.5)
+    wi, ww, wout, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=packing, router=router, add=add)
+    bad = nt // 2
+    logits[bad, ne // 2] = np.nan
+    ids, w, out, _ = run_layer(lib, gt, dt, blobs, k, n_embd, n_ff, logits, x, packing=packing, router=router, add=add)
+    assert np.all(ids[bad] == -1) and np.all(w[bad] == 0.0) and np.array_equal(out[bad], add[bad])
+    for t in range(nt):
+        if t != bad:
+            assert np.array_equal(ids[t], wi[t]) and np.array_equal(w[t], ww[t]) and np.array_equal(out[t], wout[t])
+
+
 def test_mixed_gate_up_types(lib, oracle):
     gt, ut, dt, n_embd, n_ff, ne, k = 22, 29, 22, 512, 256, 6, 3
     blobs = make_experts(gt, dt, n_embd, n_ff, ne, 77, up_type=ut)

@@ -101,7 +101,7 @@ def test_plan_and_group(lib):
 # ---- the sigmoid router (router_sigmoid / moe_route's selection): ids bit-exact with the CPU checker, weights to the
 # reference's bar of 1e-5 (src/kernels/router_sigmoid_parity.cpp:137-143), on that test's case shapes and wider ones
 
-from test_oracle_formats import SIGMOID_CASES, sigmoid_case
+from test_oracle_formats import SIGMOID_CASES, non_finite_rows, sigmoid_case
 
 
 def _check_sigmoid(lib, oracle, logits, bias, k, w_scale, norm):
@@ -160,3 +160,25 @@ def test_route_plan_in_one_launch(lib):
             torch.cuda.synchronize()
             assert torch.equal(ids, wi) and torch.equal(w, ww)
             assert torch.equal(pl, lib.plan(wi.reshape(-1), table))
+
+
+@pytest.mark.parametrize("ne", (64, 256, 300))
+def test_sigmoid_router_refuses_non_finite_rows(lib, oracle, ne):
+    """A row with a NaN / Inf logit or score gets no routes (ids -1, weights 0, null plan entries), in the router call and
+    in the route-and-plan launch; its neighbours route as if it were not there."""
+    k = 8
+    logits = non_finite_rows(ne, 5)
+    bias = (np.random.default_rng(6).standard_normal(ne) * 0.1).astype(np.float32)
+    ids, w = _check_sigmoid(lib, oracle, logits, bias, k, 2.5, 1)
+    assert np.all(ids[1:4] == -1) and np.all(w[1:4] == 0.0) and ids[[0, 4]].min() >= 0
+    table = torch.arange(1, ne + 1, dtype=torch.int64, device="cuda") * 4096
+    bias_d = torch.from_numpy(bias).cuda()
+    pi, pw, pl = lib.route_plan(torch.from_numpy(logits).cuda(), k, table, lib.Router(lib.ROUTER_SIGMOID, 1, bias_d.data_ptr(), 2.5))
+    torch.cuda.synchronize()
+    assert np.array_equal(pi.cpu().numpy(), ids) and np.array_equal(pw.cpu().numpy(), w)
+    pl = pl.cpu().numpy().reshape(5, k)
+    assert np.all(pl[1:4] == 0) and np.array_equal(pl[[0, 4]], (ids[[0, 4]].astype(np.int64) + 1) * 4096)
+    bias[5] = np.inf
+    ids, w = _check_sigmoid(lib, oracle, logits, bias, k, 1.0, 2)
+    assert np.all(ids == -1) and np.all(w == 0.0)
+

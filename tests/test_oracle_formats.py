@@ -314,3 +314,32 @@ def test_sigmoid_router_closed_forms(oracle):
     _, w2 = oracle.router_sigmoid(logits, None, k, 1.0, 2)
     p = 1.0 / (1.0 + np.exp(30.0))
     assert np.allclose(w1, p / 6.103515625e-5, rtol=1e-5) and np.allclose(w2, 1.0 / k, rtol=1e-5)
+
+
+def non_finite_rows(ne, seed):
+    """Five rows: 0 and 4 ordinary, 1 with a NaN logit, 2 with +Inf, 3 with -Inf (its sigmoid is a finite 0)."""
+    logits = (np.random.default_rng(seed).standard_normal((5, ne)) * 2).astype(np.float32)
+    logits[1, ne // 3] = np.nan
+    logits[2, ne - 1] = np.inf
+    logits[3, 0] = -np.inf
+    return logits
+
+
+@pytest.mark.parametrize("ne", (64, 300))
+def test_sigmoid_router_refuses_non_finite_rows(oracle, ne):
+    """The engine's routers give a row with a non-finite logit or score no routes: ids -1, weights 0
+    (src/kernels/cuda/glm_batch.cu:2077-2092, tests/hip/glm_handoff.cpp:186-207); the other rows are not touched."""
+    k = 8
+    logits = non_finite_rows(ne, 5)
+    bias = (np.random.default_rng(6).standard_normal(ne) * 0.1).astype(np.float32)
+    for f64 in (False, True):
+        ids, w = oracle.router_sigmoid(logits, bias, k, 2.5, 1, f64=f64)
+        good = [0, 4]
+        gi, gw = oracle.router_sigmoid(logits[good], bias, k, 2.5, 1, f64=f64)
+        assert np.array_equal(ids[good], gi) and np.array_equal(w[good], gw) and gi.min() >= 0
+        assert np.all(ids[1:4] == -1) and np.all(w[1:4] == 0.0)
+    # a bias that makes one score infinite refuses every row
+    bias[5] = np.inf
+    ids, w = oracle.router_sigmoid(logits, bias, k, 1.0, 2)
+    assert np.all(ids == -1) and np.all(w == 0.0)
+
