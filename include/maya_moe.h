@@ -187,6 +187,40 @@ int maya_moe_route_sigmoid(const float* logits, const float* bias, int n_tokens,
 struct maya_router;
 int maya_moe_route_plan(const struct maya_router* router, const float* logits, int n_tokens, int n_expert, int k,
                         const uint64_t* expert_table, int32_t* ids, float* weights, uint64_t* plan_ptr, void* stream);
+/* The residency tiers of the routed experts, decided on the device per routed expert: glmf::MoeDev's tables
+ * (include/strata/kernels/glm_fast.hpp:284-296) and the plan part of moe_route that reads them
+ * (src/kernels/cuda/glm_fast.cu:4262-4375).  key = layer * n_expert + expert.  tab is ONE device array: tab[key] != 0 =
+ * the expert's blob is in HBM at that address (a hit); else tab[n_keys + key] != 0 = it is in the second tier at that
+ * address (pinned host memory mapped to the device, or any memory the device reads): it goes into one of the layer's
+ * MAYA_SPARES spare slots (tab[2 n_keys + layer * MAYA_SPARES + j] != 0 = a free HBM slot; the device takes it, clears it
+ * and writes tab[key] itself: resident from here on) or, with no spare left or fewer than promote_min counted routes,
+ * into the next unused slot of scratch[n_scratch]; fetch_src[e] names its source.  In neither table: plan_ptr[e] = 0 and
+ * the miss mask says so (moe_route hands those to the host over its request ring; that ring, its CPU lane, the next
+ * layer's prefetch and the disk tier stay the engine's).  masks[4 t + 0..3] = token t's entries (bit i = its i-th) that
+ * missed / have a fetch source / were promoted / found no slot (left out: plan_ptr 0).  counts ([n_keys] or NULL) are the
+ * routes a key (moe_route's dcnt), halved each time seq ([1] or NULL: the routes so far) reaches a multiple of 4096.
+ * The n_tokens rows are planned one after another, as one moe_route call a token of a window. */
+#define MAYA_SPARES 3
+typedef struct maya_residency {
+    uint64_t* tab;             /* [2 * n_keys + n_layers * MAYA_SPARES] */
+    int32_t n_keys;            /* n_layers * n_expert */
+    int32_t n_layers;
+    const uint64_t* scratch;   /* [n_scratch] HBM slots */
+    int32_t n_scratch;
+    int32_t reserved;
+    uint64_t* fetch_src;       /* [n_tokens * k] out */
+    uint32_t* counts;          /* [n_keys] or NULL */
+    uint32_t* seq;             /* [1] or NULL */
+    uint32_t* masks;           /* [n_tokens * 4] out */
+} maya_residency;
+int maya_moe_route_tiered(const struct maya_router* router, const float* logits, int n_tokens, int layer, int n_expert, int k,
+                          const maya_residency* r, int promote_min, int32_t* ids, float* weights, uint64_t* plan_ptr,
+                          void* stream);
+/* Copies every planned entry with a fetch source into its slot: moe_fetch (glm_fast.hpp:468-469, glm_fast.cu:4688-4704). */
+int maya_moe_fetch(const uint64_t* fetch_src, const uint64_t* plan_ptr, int n_entries, size_t blob_bytes, void* stream);
+/* tab[keys[i]] = vals[i], the engine's edits between tokens: tab_update (glm_fast.cu:7745-7754); n_words = the array's
+ * length (a key outside it is ignored). */
+int maya_moe_tab_update(uint64_t* tab, int n_words, const int32_t* keys, const uint64_t* vals, int n, void* stream);
 /* ids -> plan: plan_ptr[e] = expert_table[ids[e]] (0 stays 0: not resident), the plan part of moe_route_kernel
  * (src/kernels/cuda/glm_fast.cu:3998-4545) without its residency tiers. */
 int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_table, int n_expert, uint64_t* plan_ptr,

@@ -666,6 +666,66 @@ void mo_router_sigmoid_f64(const float* logits, const float* bias, int n_tokens,
     router_sigmoid_impl(logits, bias, n_tokens, n_expert, k, w_scale, norm, ids, weights, 1);
 }
 
+/* The residency plan of moe_route_kernel (src/kernels/cuda/glm_fast.cu:4262-4375; the tables: include/strata/kernels/
+ * glm_fast.hpp:284-296) over already routed ids, the device-side tiers only: a hit in tab; else a second-tier source in
+ * rtab = tab + n_keys: the layer's next free spare (it becomes resident: tab[key] written, the spare cleared) when
+ * promote_min <= 1 or the key's count reaches it, else the next unused scratch slot, else left out (the "full" mask); in
+ * neither table: a null entry and the miss mask.  counts ([n_keys] or NULL): ++ per routed key, all halved before a
+ * route when (seq + 1) % 4096 == 0 (glm_fast.cu:4032-4034, 4175); seq ([1] or NULL) counts the routes.  Tokens in order;
+ * masks[4 t + 0..3] = miss, fetch, promoted, full.  A refused row (ids -1) plans nothing. */
+void mo_plan_tiered(const int32_t* ids, int n_tokens, int layer, int n_expert, int k, uint64_t* tab, int n_keys,
+                    const uint64_t* scratch, int n_scratch, uint32_t* counts, uint32_t* seq, int promote_min,
+                    uint64_t* plan, uint64_t* fetch_src, uint32_t* masks) {
+    uint64_t* rtab = tab + n_keys;
+    uint64_t* spares = tab + 2 * (size_t) n_keys + (size_t) layer * 3;
+    int next_spare = 0, next_scratch = 0;
+    for (int t = 0; t < n_tokens; ++t) {
+        if (counts && seq && ((*seq + 1u) & 4095u) == 0u)
+            for (int i = 0; i < n_keys; ++i) counts[i] >>= 1;
+        uint32_t cnt[64];
+        for (int i = 0; i < k; ++i) {
+            const int id = ids[(size_t) t * k + i];
+            cnt[i] = (id >= 0 && counts) ? ++counts[(size_t) layer * n_expert + id] : 0u;
+        }
+        uint32_t miss = 0, fetch = 0, promo = 0, full = 0;
+        for (int i = 0; i < k; ++i) {
+            const int id = ids[(size_t) t * k + i];
+            uint64_t ptr = 0, src = 0;
+            if (id >= 0) {
+                const size_t key = (size_t) layer * n_expert + id;
+                ptr = tab[key];
+                if (ptr == 0) {
+                    src = rtab[key];
+                    if (src == 0) {
+                        miss |= 1u << i;
+                    } else {
+                        while (next_spare < 3 && spares[next_spare] == 0) ++next_spare;
+                        if (next_spare < 3 && (promote_min <= 1 || cnt[i] >= (uint32_t) promote_min)) {
+                            ptr = spares[next_spare];
+                            spares[next_spare] = 0;
+                            tab[key] = ptr;
+                            promo |= 1u << i;
+                        } else if (next_scratch < n_scratch) {
+                            ptr = scratch[next_scratch++];
+                        } else {
+                            full |= 1u << i;
+                            src = 0;
+                        }
+                        if (src != 0) fetch |= 1u << i;
+                    }
+                }
+            }
+            plan[(size_t) t * k + i] = ptr;
+            fetch_src[(size_t) t * k + i] = src;
+        }
+        masks[4 * t + 0] = miss;
+        masks[4 * t + 1] = fetch;
+        masks[4 * t + 2] = promo;
+        masks[4 * t + 3] = full;
+        if (seq) *seq += 1u;
+    }
+}
+
 /* src/kernels/cuda/native_moe.cu:36-52: sum = parts[0]*w[0]; sum += parts[i]*w[i] ... (each product and add rounded) */
 void mo_combine(const float* parts, const float* w, int k, int64_t n, float* out) {
     for (int64_t c = 0; c < n; ++c) {

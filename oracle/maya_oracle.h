@@ -126,6 +126,12 @@ void mo_router_sigmoid(const float* logits, const float* bias, int n_tokens, int
 void mo_router_sigmoid_f64(const float* logits, const float* bias, int n_tokens, int n_expert, int k, float w_scale, int norm,
                            int32_t* ids, float* weights);
 
+/* ---- the residency plan over routed ids (moe_route_kernel's tiers, src/kernels/cuda/glm_fast.cu:4262-4375): tab =
+ * [n_keys] HBM | [n_keys] second tier | [n_layers][3] spares, edited in place; see maya_oracle.c */
+void mo_plan_tiered(const int32_t* ids, int n_tokens, int layer, int n_expert, int k, uint64_t* tab, int n_keys,
+                    const uint64_t* scratch, int n_scratch, uint32_t* counts, uint32_t* seq, int promote_min,
+                    uint64_t* plan, uint64_t* fetch_src, uint32_t* masks);
+
 /* ---- combine (src/kernels/cuda/native_moe.cu:36-52): out[c] = sum_i w[i] * parts[i][c] in order i = 0..k-1 */
 void mo_combine(const float* parts, const float* w, int k, int64_t n, float* out);
 

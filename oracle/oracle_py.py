@@ -228,6 +228,27 @@ def router_sigmoid(logits, bias, k, w_scale=1.0, norm=1, f64=False):
     return ids, w
 
 
+def plan_tiered(ids, layer, n_expert, tab, scratch, counts=None, seq=None, promote_min=0):
+    """The residency plan of routed ids [nt, k] against tab (uint64, edited in place: HBM | second tier | spares); counts
+    (uint32 [n_keys]) and seq (uint32 [1]) are edited in place too.  Returns plan, fetch_src (uint64 [nt, k]), masks [nt, 4]."""
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    nt, k = ids.shape
+    assert tab.dtype == np.uint64 and tab.flags.c_contiguous
+    scratch = np.ascontiguousarray(scratch, dtype=np.uint64)
+    plan = np.zeros((nt, k), dtype=np.uint64)
+    src = np.zeros((nt, k), dtype=np.uint64)
+    masks = np.zeros((nt, 4), dtype=np.uint32)
+    f = lib().mo_plan_tiered
+    f.restype = None
+    f.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                  C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    n_layers = tab.size // (2 * n_expert + 3)
+    assert n_layers * (2 * n_expert + 3) == tab.size
+    f(_ptr(ids), nt, layer, n_expert, k, _ptr(tab), n_layers * n_expert, _ptr(scratch) if scratch.size else None, scratch.size,
+      None if counts is None else _ptr(counts), None if seq is None else _ptr(seq), promote_min, _ptr(plan), _ptr(src), _ptr(masks))
+    return plan, src, masks
+
+
 def combine(parts, w):
     parts = np.ascontiguousarray(parts, dtype=np.float32)
     w = np.ascontiguousarray(w, dtype=np.float32)

@@ -1231,6 +1231,7 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
 #include "maya_fastk.cuh"
 #include "maya_fastq.cuh"
 #include "maya_fastmv.cuh"
+#include "maya_tiers.cuh"
 
 namespace maya {
 
@@ -1822,6 +1823,50 @@ int maya_moe_route_plan(const maya_router* router, const float* logits, int n_to
     hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, dim3(1, (unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, rs,
                        expert_table, ids, weights, plan_ptr, nullptr, (int64_t) 0, maya_act{nullptr, nullptr, nullptr}, nullptr, 0);
     MAYA_LAUNCHED("layer_head_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_route_tiered(const maya_router* router, const float* logits, int n_tokens, int layer, int n_expert, int k,
+                          const maya_residency* r, int promote_min, int32_t* ids, float* weights, uint64_t* plan_ptr, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    RouterSpec rs;
+    if (!router_spec(router, rs)) return fail(MAYA_E_UNSUPPORTED, "route_tiered: router kind %d / normalisation %d", router->kind, router->norm);
+    if (!logits || !r || !r->tab || !r->fetch_src || !r->masks || !ids || !weights || !plan_ptr || (r->n_scratch > 0 && !r->scratch))
+        return fail(MAYA_E_ARG, "route_tiered: null pointer");
+    if (n_tokens <= 0 || n_tokens > 256 || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k <= 0 || k > MAYA_MAX_K || k > n_expert)
+        return fail(MAYA_E_SHAPE, "route_tiered: tokens %d experts %d k %d (limits 256 tokens, %d experts, k %d)", n_tokens, n_expert, k,
+                    MAYA_MAX_EXPERTS, MAYA_MAX_K);
+    if (r->n_layers <= 0 || layer < 0 || layer >= r->n_layers || r->n_scratch < 0 || (int64_t) r->n_layers * n_expert != (int64_t) r->n_keys)
+        return fail(MAYA_E_SHAPE, "route_tiered: layer %d of %d, %d keys for %d experts a layer, %d scratch slots", layer, r->n_layers,
+                    r->n_keys, n_expert, r->n_scratch);
+    const Tiers tr{r->tab, r->scratch, r->fetch_src, r->counts, r->seq, r->masks, r->n_keys, r->n_scratch};
+    hipLaunchKernelGGL(route_tiered_kernel, dim3(1), dim3(256), 0, as_stream(stream), logits, n_tokens, n_expert, k, rs, layer, tr,
+                       promote_min, ids, weights, plan_ptr);
+    MAYA_LAUNCHED("route_tiered_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_fetch(const uint64_t* fetch_src, const uint64_t* plan_ptr, int n_entries, size_t blob_bytes, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!fetch_src || !plan_ptr) return fail(MAYA_E_ARG, "fetch: null pointer");
+    if (n_entries <= 0 || n_entries > 65535 || blob_bytes == 0) return fail(MAYA_E_SHAPE, "fetch: %d entries of %zu bytes", n_entries, blob_bytes);
+    // (slices of at least 64 KB, at most 256 of them a blob: an entry with nothing to fetch costs its workgroups a load)
+    const unsigned slices = (unsigned) std::min<size_t>(256, (blob_bytes + 65535) / 65536);
+    hipLaunchKernelGGL(fetch_kernel, dim3(slices, (unsigned) n_entries), dim3(256), 0, as_stream(stream), fetch_src, plan_ptr, blob_bytes);
+    MAYA_LAUNCHED("fetch_kernel");
+    return MAYA_OK;
+}
+
+int maya_moe_tab_update(uint64_t* tab, int n_words, const int32_t* keys, const uint64_t* vals, int n, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (n == 0) return MAYA_OK;
+    if (!tab || !keys || !vals) return fail(MAYA_E_ARG, "tab_update: null pointer");
+    if (n < 0 || n_words <= 0) return fail(MAYA_E_SHAPE, "tab_update: %d edits of %d words", n, n_words);
+    hipLaunchKernelGGL(tab_update_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, as_stream(stream), tab, keys, vals, n, n_words);
+    MAYA_LAUNCHED("tab_update_kernel");
     return MAYA_OK;
 }
 

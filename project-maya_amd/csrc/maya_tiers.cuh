@@ -1,0 +1,120 @@
+// The routed experts' residency tiers, decided on the device per routed expert: the tables of glmf::MoeDev
+// (include/strata/kernels/glm_fast.hpp:284-296) and the plan part of moe_route_kernel that reads them
+// (src/kernels/cuda/glm_fast.cu:4262-4375), the fetch of moe_fetch_kernel (glm_fast.cu:4688-4704) and tab_update
+// (glm_fast.cu:7745-7754).  The request ring to the host, the CPU lane, the prefetch of the next layer and the disk tier
+// stay the engine's: an expert in neither table is reported in the miss mask and left out of the plan.
+#pragma once
+
+namespace maya {
+
+struct Tiers {
+    uint64_t* tab;             // [n_keys] HBM address | [n_keys] second-tier address | [n_layers][MAYA_SPARES] free HBM slots
+    const uint64_t* scratch;   // [n_scratch] HBM slots for fetched experts that are not promoted
+    uint64_t* fetch_src;       // [n_tokens * k] out
+    uint32_t* counts;          // [n_keys] or null
+    uint32_t* seq;             // [1] or null: the routes so far (the counts halve when it reaches a multiple of 4096)
+    uint32_t* masks;           // [n_tokens][4] out: miss, fetch, promoted, no slot left
+    int n_keys, n_scratch;
+};
+
+template <typename T> __device__ __forceinline__ T tier_load(const T* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One workgroup of 256; the tokens one after another (a window's tokens take the spares and the scratch slots in order,
+// as one moe_route call a token does).
+__global__ __launch_bounds__(256) void route_tiered_kernel(const float* __restrict__ logits, int n_tokens, int n_expert, int k,
+                                                           RouterSpec rs, int layer, Tiers r, int promote_min,
+                                                           int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                           uint64_t* __restrict__ plan) {
+    __shared__ RouterLds sm;
+    __shared__ uint64_t s_tab[MAYA_MAX_K], s_rtab[MAYA_MAX_K];
+    __shared__ uint32_t s_cnt[MAYA_MAX_K];
+    const int tid = threadIdx.x;
+    uint64_t* const rtab = r.tab + r.n_keys;
+    uint64_t* const spares = r.tab + 2 * (size_t) r.n_keys + (size_t) layer * MAYA_SPARES;
+    int next_spare = 0, next_scratch = 0;   // (thread 0's)
+    for (int t = 0; t < n_tokens; ++t) {
+        // (words an earlier token of this launch may have written are read past the CU's cache)
+        if (r.counts != nullptr && r.seq != nullptr && ((tier_load(r.seq) + 1u) & 4095u) == 0u) {
+            for (int i = tid; i < r.n_keys; i += 256) r.counts[i] = tier_load(r.counts + i) >> 1;
+            __threadfence();
+        }
+        route_any(logits + (size_t) t * n_expert, n_expert, k, rs, sm);
+        // a thread an entry: its count and its two table words (a route's keys are distinct)
+        if (tid < k) {
+            const int id = sm.id[tid];
+            if (id >= 0) {
+                const size_t key = (size_t) layer * n_expert + id;
+                s_cnt[tid] = r.counts != nullptr ? atomicAdd(r.counts + key, 1u) + 1u : 0u;
+                s_tab[tid] = tier_load(r.tab + key);
+                s_rtab[tid] = tier_load(rtab + key);
+            } else {
+                s_cnt[tid] = 0u, s_tab[tid] = 0ull, s_rtab[tid] = 0ull;
+            }
+        }
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t miss = 0u, fetch = 0u, promo = 0u, full = 0u;
+            for (int i = 0; i < k; ++i) {
+                const int id = sm.id[i];
+                uint64_t ptr = s_tab[i], src = 0ull;
+                if (id >= 0 && ptr == 0ull) {
+                    src = s_rtab[i];
+                    if (src == 0ull) {
+                        miss |= 1u << i;   // in neither tier: the engine's to provide
+                    } else {
+                        while (next_spare < MAYA_SPARES && tier_load(spares + next_spare) == 0ull) ++next_spare;
+                        if (next_spare < MAYA_SPARES && (promote_min <= 1 || s_cnt[i] >= (uint32_t) promote_min)) {
+                            ptr = tier_load(spares + next_spare);
+                            spares[next_spare] = 0ull;
+                            r.tab[(size_t) layer * n_expert + id] = ptr;   // resident from here on
+                            promo |= 1u << i;
+                        } else if (next_scratch < r.n_scratch) {
+                            ptr = r.scratch[next_scratch++];
+                        } else {
+                            full |= 1u << i;   // left out
+                            src = 0ull;
+                        }
+                        if (src != 0ull) fetch |= 1u << i;
+                    }
+                }
+                ids[(size_t) t * k + i] = id;
+                weights[(size_t) t * k + i] = sm.w[i];
+                plan[(size_t) t * k + i] = ptr;
+                r.fetch_src[(size_t) t * k + i] = src;
+            }
+            r.masks[4 * t + 0] = miss;
+            r.masks[4 * t + 1] = fetch;
+            r.masks[4 * t + 2] = promo;
+            r.masks[4 * t + 3] = full;
+            if (r.seq != nullptr) *r.seq = tier_load(r.seq) + 1u;
+        }
+        // (the next token reads the table words and the counter this one wrote)
+        __threadfence();
+        __syncthreads();
+    }
+}
+
+// grid (slices, entries): entry blockIdx.y's blob from its source into its slot, 16 bytes a lane where both are aligned
+__global__ __launch_bounds__(256) void fetch_kernel(const uint64_t* __restrict__ fetch_src, const uint64_t* __restrict__ plan, size_t n) {
+    const uint8_t* src = (const uint8_t*) fetch_src[blockIdx.y];
+    uint8_t* dst = (uint8_t*) plan[blockIdx.y];
+    if (src == nullptr || dst == nullptr) return;
+    const size_t i0 = (size_t) blockIdx.x * 256 + threadIdx.x, step = (size_t) gridDim.x * 256;
+    if ((((uintptr_t) src | (uintptr_t) dst) & 15) == 0) {
+        const size_t n16 = n >> 4;
+        for (size_t i = i0; i < n16; i += step) ((uint4*) dst)[i] = ((const uint4*) src)[i];
+        for (size_t i = (n16 << 4) + i0; i < n; i += step) dst[i] = src[i];
+    } else {
+        for (size_t i = i0; i < n; i += step) dst[i] = src[i];
+    }
+}
+
+__global__ void tab_update_kernel(uint64_t* __restrict__ tab, const int32_t* __restrict__ keys, const uint64_t* __restrict__ vals, int n,
+                                  int n_words) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && keys[i] >= 0 && keys[i] < n_words) tab[keys[i]] = vals[i];
+}
+
+}  // namespace maya

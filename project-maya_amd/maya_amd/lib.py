@@ -18,7 +18,8 @@ EXPORTS = [
     "maya_moe_block_values", "maya_moe_row_bytes", "maya_moe_layout_init", "maya_dequant_rows", "maya_quant_act",
     "maya_quant_i8x32", "maya_moe_route_topk", "maya_moe_plan", "maya_moe_group", "maya_moe_gate_up", "maya_moe_down",
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
-    "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan",
+    "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
+    "maya_moe_tab_update",
     "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
 
@@ -35,6 +36,14 @@ class MayaError(RuntimeError):
 
 class Router(C.Structure):
     _fields_ = [("kind", C.c_int32), ("norm", C.c_int32), ("bias", C.c_void_p), ("w_scale", C.c_float)]
+
+
+class Residency(C.Structure):
+    _fields_ = [("tab", C.c_void_p), ("n_keys", C.c_int32), ("n_layers", C.c_int32), ("scratch", C.c_void_p), ("n_scratch", C.c_int32),
+                ("reserved", C.c_int32), ("fetch_src", C.c_void_p), ("counts", C.c_void_p), ("seq", C.c_void_p), ("masks", C.c_void_p)]
+
+
+SPARES = 3
 
 
 class Layout(C.Structure):
@@ -89,6 +98,9 @@ def load():
     L.maya_quant_i8x32.argtypes = [vp, i32, i64, vp, i32, i64, vp, vp, vp]
     L.maya_moe_route_topk.argtypes = [vp, i32, i32, i32, vp, vp, vp]
     L.maya_moe_plan.argtypes = [vp, i32, vp, i32, vp, vp]
+    L.maya_moe_route_tiered.argtypes = [vp, vp, i32, i32, i32, i32, C.POINTER(Residency), i32, vp, vp, vp, vp]
+    L.maya_moe_fetch.argtypes = [vp, vp, i32, sz, vp]
+    L.maya_moe_tab_update.argtypes = [vp, i32, vp, vp, i32, vp]
     L.maya_moe_group.argtypes = [vp, i32, vp, vp, vp, vp, vp]
     L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
@@ -224,6 +236,42 @@ def route_plan(logits, k, expert_table, router=None, stream=None):
     check(load().maya_moe_route_plan(None if router is None else C.byref(router), _p(logits), nt, ne, k, _p(expert_table), _p(ids),
                                      _p(w), _p(pl), _stream(stream)))
     return ids, w, pl
+
+
+class Tiers:
+    """The residency tables of a model's routed experts on the device (glmf::MoeDev's tab, include/strata/kernels/
+    glm_fast.hpp:284-296): tab = [n_keys] HBM addresses | [n_keys] second-tier addresses | [n_layers][SPARES] free HBM
+    slots, scratch slots for what is fetched but not promoted, and the outputs of a route."""
+
+    def __init__(self, n_layers, n_expert, scratch, max_entries, with_counts=False):
+        self.n_layers, self.n_expert = n_layers, n_expert
+        self.n_keys = n_layers * n_expert
+        self.tab = torch.zeros(2 * self.n_keys + n_layers * SPARES, dtype=torch.int64, device="cuda")
+        self.scratch = scratch
+        self.fetch_src = torch.zeros(max_entries, dtype=torch.int64, device="cuda")
+        self.masks = torch.zeros(4 * max_entries, dtype=torch.int32, device="cuda")
+        self.counts = torch.zeros(self.n_keys, dtype=torch.int32, device="cuda") if with_counts else None
+        self.seq = torch.zeros(1, dtype=torch.int32, device="cuda") if with_counts else None
+        self.c = Residency(self.tab.data_ptr(), self.n_keys, n_layers, scratch.data_ptr() if scratch.numel() else None, scratch.numel(), 0,
+                           self.fetch_src.data_ptr(), None if self.counts is None else self.counts.data_ptr(),
+                           None if self.seq is None else self.seq.data_ptr(), self.masks.data_ptr())
+
+    def route(self, logits, layer, k, router=None, promote_min=0, stream=None):
+        """ids, weights, plan of logits [nt, n_expert] for this layer; fetch_src / masks are left in the object."""
+        nt, ne = logits.shape
+        assert nt * k <= self.fetch_src.numel()
+        ids = torch.empty((nt, k), dtype=torch.int32, device=logits.device)
+        w = torch.empty((nt, k), dtype=torch.float32, device=logits.device)
+        pl = torch.empty(nt * k, dtype=torch.int64, device=logits.device)
+        check(load().maya_moe_route_tiered(None if router is None else C.byref(router), _p(logits), nt, layer, ne, k, C.byref(self.c),
+                                           promote_min, _p(ids), _p(w), _p(pl), _stream(stream)))
+        return ids, w, pl
+
+    def fetch(self, plan_ptr, blob_bytes, stream=None):
+        check(load().maya_moe_fetch(_p(self.fetch_src), _p(plan_ptr), plan_ptr.numel(), blob_bytes, _stream(stream)))
+
+    def update(self, keys, vals, stream=None):
+        check(load().maya_moe_tab_update(_p(self.tab), self.tab.numel(), _p(keys), _p(vals), keys.numel(), _stream(stream)))
 
 
 def plan(ids, expert_table, stream=None):
