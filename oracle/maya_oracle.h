@@ -29,8 +29,13 @@
  *   sigmoid router ................... the reference's host form (router_sigmoid_parity.cpp:36-86, restated in double with a
  *                                       stable sort) on its own four case shapes incl. exact ties, to its tolerance (ids
  *                                       equal, weights 1e-5); closed forms (equal logits, a bias that selects but does not
- *                                       weigh, sum of weights = w_scale); the wrong readings the reference names must differ
+ *                                       weigh, sum of weights = w_scale); the wrong readings the reference names must differ; non-finite
+ *                                       rows refused as tests/hip/glm_handoff.cpp:186-207 expects (ids -1)
  *   combine .......................... closed form
+ *   residency plan (mo_plan_tiered) .. worked examples written out by hand from the documented rule (include/strata/kernels/
+ *                                       glm_fast.hpp:284-292): hits, spares in order, promotion, scratch, no slot left, a window's
+ *                                       later token, promote_min against the counts, the counts' halving; the reference test's
+ *                                       expectation for empty tables (miss mask 255, tests/hip/glm_handoff.cpp:118)
  *   EXL3 states / codebook ........... the reference's own golden vectors data/exl3-exllamav3 (13 .bin files made by exllamav3)
  *   EXL3 mat-vec ..................... reference build: exl3_ref.cpp bit-exact; H.H = I
  *   prompt-chunk rows ................ the pieces above, row by row (the Q8_K quantizer, the Q4_K row dots, SwiGLU, combine):
