@@ -301,7 +301,7 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
 /* ============================================================================================= prefill
  * A prompt chunk's routed experts as a grouped GEMM (the reference's expert_count_kernel / expert_scatter_kernel,
  * src/kernels/cuda/glm_batch.cu:2102-2133, with the host's prefix sum of src/prefill/glm_prefill.cu:3339-3361 done on
- * the device; mmq::quantize / Context::run / run_glu, src/kernels/cuda/moe_mmq.cu:120-228; the per-32 int8 activation
+ * the device; mmq::quantize / Context::run / run_glu, src/prefill/moe_mmq.cu:120-228; the per-32 int8 activation
  * format of src/prefill/moe_fused_rdna4.cu:87-109 and its requantized H, :620-660).
  * Entry e = t * k + j is token t's j-th expert.  The plan sorts the entries by expert, stably: expert x's rows are
  * bounds[x] .. bounds[x + 1], row r serves entry row_entry[r], entry e sits at row entry_row[e] (-1: its expert is not
@@ -319,7 +319,7 @@ typedef struct maya_prefill_plan {
  * int8 codes c = min(127, nearest_int(x * (-127 / max))) with max the signed value at the first largest magnitude of a
  * 256-value block, one F32 scale d = 1 / (-127 / max) per block, and s = d * (the sum of every 32 codes), which the
  * minimums of a Q4_K sub-block multiply.  The reference's two GPU prefill forms round per 32 values instead (q8_1,
- * src/kernels/cuda/moe_mmq.cu:120; int8 + F32, src/prefill/moe_fused_rdna4.cu:87-109); this one reproduces the integer
+ * src/prefill/moe_mmq.cu:120; int8 + F32, src/prefill/moe_fused_rdna4.cu:87-109); this one reproduces the integer
  * sums of the CPU path, which is what its results are checked against. */
 typedef struct maya_prefill_act {
     int8_t* q; /* [rows][k], 16-byte aligned */
