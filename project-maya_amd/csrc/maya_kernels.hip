@@ -1841,6 +1841,15 @@ int maya_moe_route_tiered(const maya_router* router, const float* logits, int n_
         return fail(MAYA_E_SHAPE, "route_tiered: layer %d of %d, %d keys for %d experts a layer, %d scratch slots", layer, r->n_layers,
                     r->n_keys, n_expert, r->n_scratch);
     const Tiers tr{r->tab, r->scratch, r->fetch_src, r->counts, r->seq, r->masks, r->n_keys, r->n_scratch};
+    if (n_tokens > 1 && n_tokens * k <= 256) {
+        // a window: the tokens routed side by side, then one workgroup plans their entries in order
+        hipLaunchKernelGGL(router_kernel, dim3((unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, rs, ids, weights);
+        MAYA_LAUNCHED("router_kernel");
+        hipLaunchKernelGGL(plan_tiered_kernel, dim3(1), dim3(256), 0, as_stream(stream), (const int32_t*) ids, n_tokens, n_expert, k, layer, tr,
+                           promote_min, plan_ptr);
+        MAYA_LAUNCHED("plan_tiered_kernel");
+        return MAYA_OK;
+    }
     hipLaunchKernelGGL(route_tiered_kernel, dim3(1), dim3(256), 0, as_stream(stream), logits, n_tokens, n_expert, k, rs, layer, tr,
                        promote_min, ids, weights, plan_ptr);
     MAYA_LAUNCHED("route_tiered_kernel");

@@ -96,6 +96,87 @@ __global__ __launch_bounds__(256) void route_tiered_kernel(const float* __restri
     }
 }
 
+// The same plan over already routed ids, for a window of tokens (n = n_tokens * k <= 256 entries): one workgroup, a thread
+// an entry fetches its table words, thread 0 then walks the entries in order out of LDS (a promotion is carried to the
+// later entries of the same expert), and every thread writes its entry's results.  The counts stay per token (a token
+// after a halving must see halved counts): one round of atomics a token, only when counts are kept.
+__global__ __launch_bounds__(256) void plan_tiered_kernel(const int32_t* __restrict__ ids, int n_tokens, int n_expert, int k, int layer,
+                                                          Tiers r, int promote_min, uint64_t* __restrict__ plan) {
+    __shared__ uint64_t s_tab[256], s_rtab[256], s_plan[256], s_src[256];
+    __shared__ uint32_t s_cnt[256], s_mask[256][4];
+    __shared__ int s_id[256];
+    const int tid = threadIdx.x, n = n_tokens * k;
+    uint64_t* const rtab = r.tab + r.n_keys;
+    uint64_t* const spares = r.tab + 2 * (size_t) r.n_keys + (size_t) layer * MAYA_SPARES;
+    const int id = tid < n ? ids[tid] : -1;
+    const size_t key = (size_t) layer * n_expert + (id >= 0 ? id : 0);
+    if (tid < n) {
+        s_id[tid] = id;
+        s_tab[tid] = id >= 0 ? tier_load(r.tab + key) : 0ull;
+        s_rtab[tid] = id >= 0 ? tier_load(rtab + key) : 0ull;
+        s_cnt[tid] = 0u;
+    }
+    if (r.counts != nullptr) {
+        const uint32_t seq0 = r.seq != nullptr ? tier_load(r.seq) : 1u;
+        for (int t = 0; t < n_tokens; ++t) {
+            if (r.seq != nullptr && ((seq0 + (uint32_t) t + 1u) & 4095u) == 0u) {
+                for (int i = tid; i < r.n_keys; i += 256) r.counts[i] = tier_load(r.counts + i) >> 1;
+                __threadfence();
+                __syncthreads();
+            }
+            if (tid >= t * k && tid < (t + 1) * k && id >= 0) s_cnt[tid] = atomicAdd(r.counts + key, 1u) + 1u;
+            __threadfence();
+            __syncthreads();
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int next_spare = 0, next_scratch = 0;
+        uint64_t sp[MAYA_SPARES];
+        for (int j = 0; j < MAYA_SPARES; ++j) sp[j] = tier_load(spares + j);
+        for (int t = 0; t < n_tokens; ++t) {
+            uint32_t miss = 0u, fetch = 0u, promo = 0u, full = 0u;
+            for (int i = 0; i < k; ++i) {
+                const int e = t * k + i, eid = s_id[e];
+                uint64_t ptr = s_tab[e], src = 0ull;
+                if (eid >= 0 && ptr == 0ull) {
+                    src = s_rtab[e];
+                    if (src == 0ull) {
+                        miss |= 1u << i;
+                    } else {
+                        while (next_spare < MAYA_SPARES && sp[next_spare] == 0ull) ++next_spare;
+                        if (next_spare < MAYA_SPARES && (promote_min <= 1 || s_cnt[e] >= (uint32_t) promote_min)) {
+                            ptr = sp[next_spare];
+                            sp[next_spare] = 0ull;
+                            spares[next_spare] = 0ull;
+                            r.tab[(size_t) layer * n_expert + eid] = ptr;
+                            for (int f = e + 1; f < n; ++f)
+                                if (s_id[f] == eid) s_tab[f] = ptr;   // resident for the window's later tokens
+                            promo |= 1u << i;
+                        } else if (next_scratch < r.n_scratch) {
+                            ptr = r.scratch[next_scratch++];
+                        } else {
+                            full |= 1u << i;
+                            src = 0ull;
+                        }
+                        if (src != 0ull) fetch |= 1u << i;
+                    }
+                }
+                s_plan[e] = ptr;
+                s_src[e] = src;
+            }
+            s_mask[t][0] = miss, s_mask[t][1] = fetch, s_mask[t][2] = promo, s_mask[t][3] = full;
+        }
+        if (r.seq != nullptr) *r.seq = tier_load(r.seq) + (uint32_t) n_tokens;
+    }
+    __syncthreads();
+    if (tid < n) {
+        plan[tid] = s_plan[tid];
+        r.fetch_src[tid] = s_src[tid];
+    }
+    if (tid < 4 * n_tokens) r.masks[tid] = s_mask[tid >> 2][tid & 3];
+}
+
 // grid (slices, entries): entry blockIdx.y's blob from its source into its slot, 16 bytes a lane where both are aligned
 __global__ __launch_bounds__(256) void fetch_kernel(const uint64_t* __restrict__ fetch_src, const uint64_t* __restrict__ plan, size_t n) {
     const uint8_t* src = (const uint8_t*) fetch_src[blockIdx.y];
