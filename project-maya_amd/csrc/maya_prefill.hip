@@ -31,13 +31,17 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // dynamic LDS: seg[kPlanWaves][n_expert] counts -> bases, base[n_expert + 1]
 __global__ __launch_bounds__(kPlanThreads) void prefill_plan_kernel(const int32_t* __restrict__ ids, int n_entries,
                                                                     const uint64_t* __restrict__ table, int n_expert,
-                                                                    maya_prefill_plan p, int max_tiles) {
-    extern __shared__ int32_t sm[];
+                                                                    maya_prefill_plan p, int max_tiles, int with_masks) {
+    extern __shared__ __attribute__((aligned(16))) int32_t sm[];
     int32_t* seg = sm;                               // [kPlanWaves][n_expert]
     int32_t* base = sm + kPlanWaves * n_expert;      // [n_expert + 1]
+    // (with_masks: [kPlanWaves][n_expert] 64-bit words behind base, 8-byte aligned)
+    unsigned long long* mask = with_masks ? (unsigned long long*) (sm + ((kPlanWaves * n_expert + n_expert + 1 + 1) & ~1)) : nullptr;
     __shared__ int32_t s_tiles;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     for (int i = tid; i < kPlanWaves * n_expert; i += kPlanThreads) seg[i] = 0;
+    if (mask != nullptr)
+        for (int i = tid; i < kPlanWaves * n_expert; i += kPlanThreads) mask[i] = 0ull;
     if (tid == 0) s_tiles = 0;
     __syncthreads();
     const int per = (((n_entries + kPlanWaves - 1) / kPlanWaves) + 63) & ~63;   // a wave's share, whole chunks of 64
@@ -62,9 +66,25 @@ __global__ __launch_bounds__(kPlanThreads) void prefill_plan_kernel(const int32_
         base[x + 1] = run;
     }
     __syncthreads();
-    if (tid == 0) {
-        base[0] = 0;
-        for (int x = 0; x < n_expert; ++x) base[x + 1] += base[x];
+    // base[x + 1] = the experts' running total: wave 0, a lane a run of experts, a scan over the lanes between two passes
+    if (tid < 64) {
+        const int per_lane = (n_expert + 63) >> 6, x0 = tid * per_lane;
+        int local = 0;
+        for (int i = 0; i < per_lane; ++i)
+            if (x0 + i < n_expert) local += base[x0 + i + 1];
+        int incl = local;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d, 64);
+            if (tid >= d) incl += up;
+        }
+        int run = incl - local;
+        for (int i = 0; i < per_lane; ++i)
+            if (x0 + i < n_expert) {
+                run += base[x0 + i + 1];
+                base[x0 + i + 1] = run;
+            }
+        if (tid == 0) base[0] = 0;
     }
     __syncthreads();
     for (int x = tid; x <= n_expert; x += kPlanThreads) p.bounds[x] = base[x];
@@ -85,7 +105,21 @@ __global__ __launch_bounds__(kPlanThreads) void prefill_plan_kernel(const int32_
         const int e = c0 + lane;
         const int x = e < hi ? expert_of(e) : -1;
         int rank = 0, cnt = 0;
-        unsigned long long todo = __ballot(x >= 0);
+        if (mask != nullptr) {
+            // every lane sets its bit in its expert's word; the word then tells each lane how many earlier lanes share its
+            // expert (LDS operations of one wave complete in order); the expert's last lane clears the word again
+            unsigned long long* mk = mask + (size_t) wave * n_expert;
+            if (x >= 0) atomicOr(&mk[x], 1ull << lane);
+            __builtin_amdgcn_wave_barrier();
+            if (x >= 0) {
+                const unsigned long long m = mk[x];
+                rank = __popcll(m & ((1ull << lane) - 1ull));
+                cnt = __popcll(m);
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (x >= 0 && rank == cnt - 1) mk[x] = 0ull;
+        }
+        unsigned long long todo = mask != nullptr ? 0ull : __ballot(x >= 0);
         while (todo) {
             const int leader = __ffsll((long long) todo) - 1;
             const int lx = __shfl(x, leader, 64);
@@ -676,10 +710,13 @@ int maya_moe_prefill_plan(const int32_t* ids, int n_entries, const uint64_t* exp
     if (!ids || !expert_table || !plan_ok(plan)) return fail(MAYA_E_ARG, "prefill_plan: null pointer");
     if (n_entries <= 0 || n_entries > (1 << 20) || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS)
         return fail(MAYA_E_SHAPE, "prefill_plan: entries %d experts %d", n_entries, n_expert);
-    const size_t lds = sizeof(int32_t) * ((size_t) kPlanWaves * n_expert + n_expert + 1);
+    // (up to 256 experts: a wave's 64-bit lane masks per expert ride along, 8 bytes x 16 waves an expert)
+    const int with_masks = n_expert <= 256;
+    size_t lds = sizeof(int32_t) * ((size_t) kPlanWaves * n_expert + n_expert + 1);
+    if (with_masks) lds = ((lds + 7) & ~(size_t) 7) + sizeof(unsigned long long) * (size_t) kPlanWaves * n_expert;
     if (lds > 65536) MAYA_HIP(hipFuncSetAttribute((const void*) prefill_plan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
     hipLaunchKernelGGL(prefill_plan_kernel, dim3(1), dim3(kPlanThreads), lds, as_stream(stream), ids, n_entries, expert_table,
-                       n_expert, *plan, maya_moe_prefill_max_tiles(n_entries, n_expert));
+                       n_expert, *plan, maya_moe_prefill_max_tiles(n_entries, n_expert), with_masks);
     MAYA_LAUNCHED("prefill_plan_kernel");
     return MAYA_OK;
 }
