@@ -61,17 +61,18 @@ typedef struct maya_moe_layout {
     int32_t reserved;
 } maya_moe_layout;
 
-/* Row packings.  GGUF: the file's own block sequence.  STREAM: the same bytes regrouped so that a wavefront's loads are
- * aligned, contiguous and addressed by position alone.  IQ2_S rows are taken four at a time (a quad; row counts are
- * multiples of 4): with nu = k / 32 sub-blocks a row, the quad's 4 * row_bytes bytes hold, for sub-block u of row r of
- * the quad, the (index word, sign word) pair at byte 8 (4 u + r), the (high-bit byte, scale byte) pair at
- * 32 nu + 2 (4 u + r), and block b's FP16 scale at 40 nu + 2 (4 b + r).  IQ1_S rows likewise in quads: sub-block u's four
- * index bytes at 4 (4 u + r), its qh word at 16 nu + 2 (4 u + r), block b's scale at 24 nu + 2 (4 b + r).  IQ1_M: index
- * bytes and qh words as IQ1_S, then 8 bytes a (block b, row r) at 24 nu + 8 (4 b + r) = the FP16 block scale (gathered from
- * the top nibbles of the block's four scale words) followed by those words' 4 x 12 bits of 3-bit scales.  A Q8_0 row holds its k codes first, then its
- * k / 32 FP16 scales (block b's scale at k + 2 b).  Other types are left as they are.  A row (a quad) keeps its size and
- * its position in the blob and every field keeps its bits, so dequantized values are unchanged.  Stream-packed blobs
- * and the offsets of their three row arrays are 16-byte aligned. */
+/* Row packings.  GGUF: the file's own block sequence.  STREAM: the same bytes regrouped so that a wavefront's loads
+ * are aligned, contiguous and addressed by position alone.  IQ2_S rows are taken four at a time (a quad; row counts
+ * are multiples of 4): with nu = k / 32 sub-blocks a row, the quad's 4 * row_bytes bytes hold, for sub-block u of row
+ * r of the quad, the (index word, sign word) pair at byte 8 (4 u + r), the (high-bit byte, scale byte) pair at 32 nu +
+ * 2 (4 u + r), and block b's FP16 scale at 40 nu + 2 (4 b + r).  IQ1_S rows likewise in quads: sub-block u's four
+ * index bytes at 4 (4 u + r), its qh word at 16 nu + 2 (4 u + r), block b's scale at 24 nu + 2 (4 b + r).  IQ1_M:
+ * index bytes and qh words as IQ1_S, then 8 bytes a (block b, row r) at 24 nu + 8 (4 b + r) = the FP16 block scale
+ * (gathered from the top nibbles of the block's four scale words) followed by those words' 4 x 12 bits of 3-bit
+ * scales.  A Q8_0 row holds its k codes first, then its k / 32 FP16 scales (block b's scale at k + 2 b).  Other types
+ * are left as they are.  A row (a quad) keeps its size and its position in the blob and every field keeps its bits, so
+ * dequantized values are unchanged.  Stream-packed blobs and the offsets of their three row arrays are 16-byte
+ * aligned. */
 #define MAYA_PACK_GGUF 0
 #define MAYA_PACK_STREAM 1
 

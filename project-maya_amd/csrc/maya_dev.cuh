@@ -68,14 +68,15 @@ __device__ __forceinline__ uint32_t neg_bytes(uint32_t g, uint32_t c) {
 template <int CTRL>
 __device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true); }
 
-// Q8_K rounding of a 256-value block held by 8 consecutive lanes, 32 values a lane: the arithmetic of the reference's quantize_q8_K_kernel (src/kernels/cuda/quantize_act.cu:161-207) and
-// codes, bit for bit, 4 codes a word in the order of v.  The block's scale comes from the signed value at the FIRST
-// largest magnitude.  Its magnitude is the largest magnitude; its sign depends on the order only when the largest
-// positive and the largest negative value share that magnitude.  So the common case needs two max3 chains over the raw
-// bits (as signed integers the largest is the largest positive value; as unsigned integers the largest is the negative
-// value of the largest magnitude) and three lane exchanges; only a wave that holds such a tie scans with indices
-// (index_of(i) = the index of v[i] inside the block, ascending in i).  A product never rounds beyond +-127
-// (|iscale * v| <= 127 (1 + 2^-23)), so the low byte of the magic-number sum is the code.
+// Q8_K rounding of a 256-value block held by 8 consecutive lanes, 32 values a lane: the arithmetic of the reference's
+// quantize_q8_K_kernel (src/kernels/cuda/quantize_act.cu:161-207) and codes, bit for bit, 4 codes a word in the order
+// of v.  The block's scale comes from the signed value at the FIRST largest magnitude.  Its magnitude is the largest
+// magnitude; its sign depends on the order only when the largest positive and the largest negative value share that
+// magnitude.  So the common case needs two max3 chains over the raw bits (as signed integers the largest is the
+// largest positive value; as unsigned integers the largest is the negative value of the largest magnitude) and three
+// lane exchanges; only a wave that holds such a tie scans with indices (index_of(i) = the index of v[i] inside the
+// block, ascending in i).  A product never rounds beyond +-127 (|iscale * v| <= 127 (1 + 2^-23)), so the low byte of
+// the magic-number sum is the code.
 template <typename IndexOf>
 __device__ __forceinline__ void q8k_round_lane32(const float (&v)[32], IndexOf index_of, int (&y)[8], float& d) {
     int pb = __float_as_int(v[0]);

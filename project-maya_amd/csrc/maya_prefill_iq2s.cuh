@@ -1,18 +1,17 @@
 // maya_prefill_iq2s.cuh - the prompt chunk's grouped GEMM on IQ2_S rows in the stream packing (included by
 // maya_prefill.hip inside namespace maya; the skeleton - tiles, the activations' copies, the barriers - is pf_tile's).
-//
-// out[row][n] = 1/8 sum over blocks b of (d_w[n][b] d_x[row][b]) * sum over the block's 16-value groups j of
-// (2 ls_j + 1) (w_j . c_j), w = the grid magnitudes with their signs: the integer sums of the CPU path's IQ2_S x Q8_K
-// row dot (src/kernels/cpu/iq_avx2.cpp:160-176, 225-250).  The scale belongs to 16 values and (2 ls + 1) x 43 does not fit
-// int8, so a 32-deep matrix instruction takes ONE group: a lane (row ln, k-group kg) decodes grid entry kg of a
-// sub-block - 8 signed bytes (the grid's magnitudes and a sign-mask table sit in LDS), its whole operand - and the two groups of a sub-block come from two instructions whose
-// operands are zero in the lanes of the other group (kg < 2: values 0..15, kg >= 2: 16..31).  The vector ALU then adds
-// (2 ls + 1) x the group's sums to the block's int32 sums: two multiply-adds an output a sub-block.
-//
-// Weights go global -> LDS without registers, one super-block ahead: per tile of 16 rows (4 quads) the 8 sub-blocks'
-// index + sign words (1024 bytes: one 16-byte copy a lane) and their qh / scale bytes (256 bytes: one 4-byte copy a
-// lane), each lane's source chosen so that LDS holds [sub-block][quad][row]: the 16 rows of a read then sit in 16
-// different bank pairs.  The block scales (2 bytes a row a block) come through a register.
+// out[row][n] = 1/8 sum over blocks b of (d_w[n][b] d_x[row][b]) * sum over the block's 16-value groups j of (2 ls_j +
+// 1) (w_j . c_j), w = the grid magnitudes with their signs: the integer sums of the CPU path's IQ2_S x Q8_K row dot
+// (src/kernels/cpu/iq_avx2.cpp:160-176, 225-250).  The scale belongs to 16 values and (2 ls + 1) x 43 does not fit
+// int8, so a 32-deep matrix instruction takes ONE group: a lane (row ln, k-group kg) decodes grid entry kg of a sub-
+// block - 8 signed bytes (the grid's magnitudes and a sign-mask table sit in LDS), its whole operand - and the two
+// groups of a sub-block come from two instructions whose operands are zero in the lanes of the other group (kg < 2:
+// values 0..15, kg >= 2: 16..31).  The vector ALU then adds (2 ls + 1) x the group's sums to the block's int32 sums:
+// two multiply-adds an output a sub-block.  Weights go global -> LDS without registers, one super-block ahead: per
+// tile of 16 rows (4 quads) the 8 sub-blocks' index + sign words (1024 bytes: one 16-byte copy a lane) and their qh /
+// scale bytes (256 bytes: one 4-byte copy a lane), each lane's source chosen so that LDS holds [sub-block][quad][row]:
+// the 16 rows of a read then sit in 16 different bank pairs.  The block scales (2 bytes a row a block) come through a
+// register.
 
 constexpr int kIqTileBytes = 1280, kIqWaveBytes = 2 * kIqTileBytes, kIqBufBytes = 4 * kIqWaveBytes;
 
