@@ -453,23 +453,55 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
 // meet in LDS and are summed in slot order.
 template <int ROWS, int DEPTH, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
-    static_assert(ROWS % 8 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads; the ring holds one or two");
+    static_assert(ROWS % 4 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads (the last may be one); the ring holds one or two");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ int lds[kFastLdsWords];
     __shared__ float part[8][ROWS];
-    if (a.skip && *a.skip) return;
-    stage_iq2s_tables(lds, cb, 512);
+    __shared__ float s_w[8];
+    __shared__ int s_on[8];
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r0 = blockIdx.x * ROWS;
     const int e0 = blockIdx.y * a.k;   // the token's first entry; wave w = its slot w
-    const int ent = e0 + wave;
-    const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
+    // Everything the workgroup needs before its weights is requested side by side, ahead of the one barrier: the skip
+    // flag, the plan (the wave's slot; the slots' presence and weights for the combine), the slot's h and the tables.
+    // A wave past slot k - 1 reads that slot's data and drops it: no branch, and no load waits on another.
+    const int skipv = a.skip ? *a.skip : 0;
+    const int ent = e0 + min(wave, a.k - 1);
+    uint64_t blob = a.plan_ptr[ent];
+    const int ci = e0 + min((int) threadIdx.x & 7, a.k - 1);
+    const uint64_t c_ptr = a.plan_ptr[ci];
+    const float c_w = a.plan_w[ci];
+    const bool on = NU == 64 || lane < NU;   // (an idle lane reads the last position's data and uses zeros)
+    const int pos = on ? lane : NU - 1;
+    const bool rounded = a.hq.q != nullptr;
+    int y[8];
+    float dy8 = 0.0f;
+    float v[32];
+    if (rounded) {
+        const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
+        const int4 ya = q[2 * pos], yb = q[2 * pos + 1];
+        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+        dy8 = a.hq.d[(size_t) ent * NU + pos] * 0.125f;
+    } else {
+        const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float4 t = hv[i];
+            v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+        }
+    }
+    stage_iq2s_tables(lds, cb, 512);
+    if (threadIdx.x < 8) {
+        s_on[threadIdx.x] = (int) threadIdx.x < a.k && c_ptr != 0ull;
+        s_w[threadIdx.x] = c_w;
+    }
     __syncthreads();
+    if (skipv) return;
+    if (wave >= a.k) blob = 0ull;
     if (blob != 0ull) {
-        // the first rows' weights are requested before h is rounded: their latency hides behind that arithmetic
         constexpr uint32_t qb = NU / 8 * 82 * 4;
         // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
         // scalar registers for the buffer resource
@@ -477,40 +509,23 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
         const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
         const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        // (an idle lane reads the last position's weights again and meets them with zero activations)
-        const bool on = NU == 64 || lane < NU;
-        const int pos = on ? lane : NU - 1;
         const QuadOffs qo = quad_offs<NU>(0u, pos);
         const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
         constexpr int NQ = ROWS / 4;
+        // the first rows' weights are requested before h is rounded: their latency hides behind that arithmetic
         QuadIQ2S ring[DEPTH];
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
-        int y[8];
-        float dy8;
-        if (!on) {
+        if (rounded) {
+            if (!on) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) y[i] = 0;
-            dy8 = 0.0f;
-        }
-        if (a.hq.q) {
-            if (on) {
-                const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
-                const int4 ya = q[2 * lane], yb = q[2 * lane + 1];
-                y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
-                dy8 = a.hq.d[(size_t) ent * NU + lane] * 0.125f;
+                for (int i = 0; i < 8; ++i) y[i] = 0;
+                dy8 = 0.0f;
             }
         } else {
             // no rounded h given: the wave rounds its slot's h to Q8_K itself (quant_q8k_block's arithmetic): a lane holds
             // sub-block `lane`, a 256-value block is 8 lanes; the block's signed maximum is the value at the FIRST largest
             // magnitude - inside a lane the scan keeps the first, between lanes the lower lane wins a tie
-            const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
-            float v[32];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float4 t = hv[i];
-                v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
-            }
             if (!on) {
 #pragma unroll
                 for (int i = 0; i < 32; ++i) v[i] = 0.0f;
@@ -531,14 +546,18 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
                 if (q + DEPTH < NQ) ring[0] = load_quad(rs, qo, quad0 + (uint32_t) (q + DEPTH) * qb);
                 quad_values<0>(cur, grid, stab, y, yn, dy8, acc);
             }
-            {
+            if (NQ % 2 == 0 || q + 1 < NQ) {
                 const QuadIQ2S cur = ring[1 % DEPTH];
                 if (q + 1 + DEPTH < NQ) ring[1 % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + 1 + DEPTH) * qb);
                 quad_values<4>(cur, grid, stab, y, yn, dy8, acc);
+            } else {
+#pragma unroll
+                for (int i = 4; i < 8; ++i) acc[i] = 0.0f;   // an odd number of quads: the last batch's second half is empty
             }
             float v = reduce8_half(acc, lane);
             v += __shfl_xor(v, 32, kWave);
-            if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
+            const int rr = r + ((lane >> 2) & 7);
+            if ((lane & 35) == 0 && (ROWS % 8 == 0 || rr < ROWS)) part[wave][rr] = v;
         }
     }
     __syncthreads();
@@ -546,18 +565,20 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         const int c = threadIdx.x;
         float sum = 0.0f;
         bool first = true;
-        for (int i = 0; i < a.k; ++i) {
-            if (a.plan_ptr[e0 + i] == 0ull) continue;
-            const float p = __fmul_rn(part[i][c], a.plan_w[e0 + i]);
-            sum = first ? p : __fadd_rn(sum, p);
-            first = false;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {   // the present slots in slot order; the first product starts the sum
+            const bool have = s_on[i] != 0;
+            const float p = __fmul_rn(part[i][c], s_w[i]);
+            const float t = first ? p : __fadd_rn(sum, p);
+            sum = have ? t : sum;
+            first = first && !have;
         }
         const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
         if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
         a.out[o] = sum;
         if (a.part)
             for (int i = 0; i < a.k; ++i)
-                if (a.plan_ptr[e0 + i] != 0ull) a.part[(size_t) (e0 + i) * n_embd + r0 + c] = part[i][c];
+                if (s_on[i]) a.part[(size_t) (e0 + i) * n_embd + r0 + c] = part[i][c];
     }
 }
 

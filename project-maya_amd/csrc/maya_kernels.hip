@@ -1318,7 +1318,8 @@ int launch_gate_up_iq2s_gguf(const maya_moe_args& a, const DeviceState& st, hipS
     MAYA_LAUNCHED("gate_up_iq2s_1tok_kernel");
     return MAYA_OK;
 }
-// the position-mapped kernels: 16 rows a workgroup; gate/up at the 6 waves a SIMD its registers allow, down at 7 (8 spill)
+// the position-mapped kernels: gate/up 16 rows a workgroup at the 6 waves a SIMD its registers allow; down 16 rows at 7
+// waves a SIMD (8 spill), or n_embd / 256 rows for the wide rows
 template <int NW>
 int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
     constexpr int kRows = 16;
@@ -1330,11 +1331,25 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 // the rows the position-mapped down kernels take on one wave: n_ff = 1024, 1536 or 2048
 static bool down_pos_nff_ok(int n_ff) { return n_ff == 1024 || n_ff == 1536 || n_ff == 2048; }
 int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
-    constexpr int kRows = 16;
-    const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
-    if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7, 32>), grid, dim3(512), 0, s, a, st.cb);
-    else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7, 48>), grid, dim3(512), 0, s, a, st.cb);
-    else hipLaunchKernelGGL((down_iq2s_pos_kernel<kRows, 1, 7>), grid, dim3(512), 0, s, a, st.cb);
+    // Rows a workgroup: n_embd / 256 for the wide rows (20 ... 32: one workgroup a compute unit on a single token, every
+    // SIMD the same number of rows, and half as many waves rounding h as with 16), else 16.
+    const int n_embd = a.layout.n_embd;
+    const int wide = n_embd % 1024 == 0 && n_embd >= 5120 && n_embd <= 8192 ? n_embd / 256 : 16;
+#define MAYA_ROWS(R, MINW)                                                                                             \
+    {                                                                                                                  \
+        const dim3 grid((unsigned) (n_embd / R), (unsigned) a.n_tokens);                                               \
+        if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 32>), grid, dim3(512), 0, s, a, st.cb);      \
+        else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 48>), grid, dim3(512), 0, s, a, st.cb); \
+        else hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW>), grid, dim3(512), 0, s, a, st.cb);                  \
+    }
+    switch (wide) {
+        case 20: MAYA_ROWS(20, 4) break;
+        case 24: MAYA_ROWS(24, 4) break;
+        case 28: MAYA_ROWS(28, 4) break;
+        case 32: MAYA_ROWS(32, 4) break;
+        default: MAYA_ROWS(16, 7) break;
+    }
+#undef MAYA_ROWS
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
     return MAYA_OK;
 }

@@ -86,6 +86,10 @@ CASES = [
     (19, 19, 5120, 1536, 4, 3, 1),
     (29, 29, 3072, 1024, 4, 2, 2),
     (19, 29, 2048, 1536, 3, 2, 3),
+    # IQ2_S down rows with n_embd / 256 rows a workgroup (24, 28, 32; 28 has an odd number of row quads), windows too
+    (22, 22, 6144, 2048, 5, 3, 2),
+    (22, 22, 7168, 2048, 9, 8, 4),
+    (22, 22, 8192, 1536, 4, 4, 3),
 ]
 
 
