@@ -1503,11 +1503,21 @@ int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
     return MAYA_OK;
 }
 int launch_down_q4k_pos(const maya_moe_args& a, hipStream_t s) {
-    constexpr int kRows = 16;
-    const dim3 grid((unsigned) (a.layout.n_embd / kRows), (unsigned) a.n_tokens);
-    if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8, 32>), grid, dim3(512), 0, s, a);
-    else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8, 48>), grid, dim3(512), 0, s, a);
-    else hipLaunchKernelGGL((down_q4k_pos_kernel<kRows, 8>), grid, dim3(512), 0, s, a);
+    // Rows a workgroup: 32 when that still leaves two workgroups a compute unit (half as many waves rounding h); 8 for
+    // one or two slots on few tokens (more, shorter waves: the rows of one expert alone are latency-bound); else 16.
+    // A workgroup has one wave a slot.
+    const int n_embd = a.layout.n_embd;
+    const int rows = (long long) (n_embd / 32) * a.n_tokens >= 512 && n_embd % 32 == 0 ? 32
+                     : a.k <= 2 && (long long) (n_embd / 16) * a.n_tokens < 1024 && n_embd % 8 == 0 ? 8 : 16;
+    const dim3 grid((unsigned) (n_embd / rows), (unsigned) a.n_tokens), block(64u * (unsigned) a.k);
+#define MAYA_ROWS(R)                                                                                              \
+    if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_q4k_pos_kernel<R, 8, 32>), grid, block, 0, s, a);          \
+    else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_q4k_pos_kernel<R, 8, 48>), grid, block, 0, s, a);     \
+    else hipLaunchKernelGGL((down_q4k_pos_kernel<R, 8>), grid, block, 0, s, a);
+    if (rows == 32) { MAYA_ROWS(32) }
+    else if (rows == 8) { MAYA_ROWS(8) }
+    else { MAYA_ROWS(16) }
+#undef MAYA_ROWS
     MAYA_LAUNCHED("down_q4k_pos_kernel");
     return MAYA_OK;
 }
