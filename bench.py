@@ -134,8 +134,8 @@ def cpu_baseline(np, torch, oracle_py, pool, blob_bytes, logits_row, x_f32, gpu_
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-graph", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--workload", default="decode_iq2s",
