@@ -1437,9 +1437,14 @@ int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     return MAYA_OK;
 }
 int launch_down_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
-    const dim3 grid((unsigned) (a.layout.n_embd / 16), (unsigned) a.n_tokens);
+    // 32 rows a workgroup for the wide rows (half as many waves rounding h, as in the IQ2_S kernel), else 16
+    const bool wide = a.layout.n_embd >= 5120 && a.layout.n_embd % 32 == 0;
+    const dim3 grid((unsigned) (a.layout.n_embd / (wide ? 32 : 16)), (unsigned) a.n_tokens);
 #define MAYA_D1(NUV)                                                                                                     \
-    if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<16, 7, NUV>), grid, dim3(512), 0, s, a, st.cb); \
+    if (wide) {                                                                                                          \
+        if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<32, 7, NUV>), grid, dim3(512), 0, s, a, st.cb); \
+        else hipLaunchKernelGGL((down_iq1s_pos_kernel<32, 7, NUV>), grid, dim3(512), 0, s, a, st.cb);                    \
+    } else if (a.layout.down_type == kIQ1_M) hipLaunchKernelGGL((down_iq1m_pos_kernel<16, 7, NUV>), grid, dim3(512), 0, s, a, st.cb); \
     else hipLaunchKernelGGL((down_iq1s_pos_kernel<16, 7, NUV>), grid, dim3(512), 0, s, a, st.cb);
     if (a.layout.n_ff == 1024) { MAYA_D1(32) } else if (a.layout.n_ff == 1536) { MAYA_D1(48) } else { MAYA_D1(64) }
 #undef MAYA_D1
