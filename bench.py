@@ -18,7 +18,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "tests")):
+for _p in (os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -166,7 +166,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if args.workload != "decode_iq2s":
-        from maya_amd import workloads
+        import bench_workloads as workloads
         if args.workload not in workloads.WORKLOADS:
             sys.exit("bench.py: unknown workload %r" % args.workload)
         r = workloads.WORKLOADS[args.workload](args.steps, args.warmup)

@@ -7,10 +7,15 @@ import time
 import numpy as np
 import torch
 
-from . import exl3, lib, prefill, synth
+from maya_amd import exl3, lib, prefill
 
 HBM_PEAK = 8.0e12
 INT8_PEAK = 5.0e15
+
+
+def zipf_bias(n_expert, s=1.1):
+    """The prefill configuration's routing skew: b_e = log(1 / (e + 1)^s), added to N(0, 1) router logits."""
+    return (-s * np.log(np.arange(1, n_expert + 1, dtype=np.float64))).astype(np.float32)
 
 
 def random_blocks(n_bytes, block, fields, seed):
@@ -199,7 +204,7 @@ def _prefill(K, W, gt, dt, what, types):
         pool = random_blocks(NE * bb, 144, BLOCK_FIELDS[lib.Q4_K][1], 11)
     table = torch.tensor([pool.data_ptr() + e * bb for e in range(NE)], dtype=torch.int64, device="cuda")
     rng = np.random.default_rng(12)
-    logits = torch.from_numpy((rng.standard_normal((T, NE)) + synth.zipf_bias(NE)).astype(np.float32)).cuda()
+    logits = torch.from_numpy((rng.standard_normal((T, NE)) + zipf_bias(NE)).astype(np.float32)).cuda()
     x = torch.randn(T, E, device="cuda")
     layer = prefill.PrefillLayer(layout, NE, TK, T, out_dtype=torch.bfloat16)
     stream = torch.cuda.Stream()

@@ -106,9 +106,6 @@ typedef struct maya_moe_args {
     const float* add;          /* NULL or [n_tokens][n_embd] added to the combined output (shared expert, CPU lane part) */
     const int32_t* add_flag;   /* NULL or a device flag: `add` is added only when it is non-zero */
     float* out;                /* [n_tokens][n_embd] */
-    int32_t* hq_sync;          /* NULL, or [n_tokens*k][n_ff/256] arrival counters, all zero at the call: a gate/up
-                                * kernel that can (maya_moe_gate_up_fuses_hq) then also writes hq, the Q8_K rounding of
-                                * h, from the last workgroup to finish each 256-value block */
 } maya_moe_args;
 
 /* ---- probes: glmf::moe_supported, iq::supported / block_bytes / row_bytes (src/ds4/ds4_iq.cuh:40-52) */
@@ -154,7 +151,10 @@ int maya_dequant_rows_packed(int ggml_type, int packing, const void* w, size_t r
 /* ---- activation quantizers.  act_type = the WEIGHT type whose dot will consume the activation:
  * Q8_K rounding for the 256-value types - quantize_q8_K (src/kernels/cuda/quantize_act.cu:161-207), q8k_quant_kernel
  * (src/ds4/ds4_gguf.cu:299-336), native_quant_act / native_quant_h (src/kernels/cpu/native_expert.cpp:262-268);
- * Q8_0 rounding for Q8_0 weights - quantize_q8_0 (include/strata/kernels/quantize_act.hpp:28-31).
+ * Q8_0 rounding for Q8_0 weights - the CPU expert path's on x86, ggml-cpu's quantize_row_q8_0 as the reference restates it
+ * (quantize_oracle_q8_0, src/kernels/cpu/expert.cpp:92-130): FP16 d = amax / 127, q = nearest-even(x * (127 / amax)); the
+ * reference's GPU quantize_q8_0 (include/strata/kernels/quantize_act.hpp:28-31; rint of the double quotient x / d) gives
+ * the same scale and differs by one code on the rare value next to a rounding boundary.
  * x: rows x k of x_dtype, x_stride elements apart (0: k). */
 int maya_quant_act(int act_type, const void* x, int x_dtype, int64_t x_stride, int rows, int64_t k, maya_act out,
                    void* stream);
@@ -240,9 +240,6 @@ int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, i
  *   glmf::moe_down (glm_fast.hpp:499-501), iq::down (ds4_iq.cuh:90-91), native_down_rows_split
  *   (native_expert.cpp:395-417), native_moe_combine (src/kernels/cuda/native_moe.cu:36-52). */
 int maya_moe_gate_up(const maya_moe_args* a, void* stream);
-/* 1 when maya_moe_gate_up, given hq_sync, writes hq itself for these arguments (the caller then skips maya_quant_act
- * of h), 0 when it leaves hq alone. */
-int maya_moe_gate_up_fuses_hq(const maya_moe_args* a);
 /* 1 when maya_moe_down, given hq = {NULL, NULL, NULL}, rounds h to the down type's activation format itself for these
  * arguments (native_quant_h's arithmetic, in the kernel's prologue; part may then be NULL), 0 when hq must be given. */
 int maya_moe_down_rounds_h(const maya_moe_args* a);

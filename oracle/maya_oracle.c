@@ -292,8 +292,14 @@ void mo_quant_q8k(const float* x, int64_t k, mo_q8k* out) {
     }
 }
 
-/* ggml's quantize_row_q8_0_ref as the reference states it (include/strata/kernels/quantize_act.hpp:28-31):
- * d = amax / 127 stored as FP16, q = roundf(x * (1 / d)) with d the F32 value before the FP16 rounding */
+/* The Q8_0 activation rounding of the CPU expert path on x86, ggml-cpu's quantize_row_q8_0 (arch/x86/quants.c) as the
+ * reference restates it in quantize_oracle_q8_0 (src/kernels/cpu/expert.cpp:92-130, "the pinned ggml CPU Q8_0 contract":
+ * FP16-rounded scales and x86 nearest-even codes, include/strata/kernels/cpu/expert.hpp:55-57):
+ *   d = amax / 127 (65504 when that is larger: the FP16 scale stays finite), stored as FP16 (nearest even);
+ *   q = nearest-even(x * (127 / amax)), the product rounded to F32 first; an all-zero block is all zeros.
+ * Two other statements of this quantizer exist and differ from it on values next to a rounding boundary: ggml's scalar
+ * quantize_row_q8_0_ref (roundf(x * (1 / d)): halves away from zero) and the reference's GPU quantize_q8_0
+ * (src/kernels/cuda/quantize_act.cu:47-78: rint of the double quotient x / d); tests/test_oracle_pins.py counts how often. */
 void mo_quant_q80(const float* x, int64_t k, mo_q80* out) {
     for (int64_t b = 0; b < k / 32; ++b) {
         const float* xb = x + b * 32;
@@ -302,10 +308,15 @@ void mo_quant_q80(const float* x, int64_t k, mo_q80* out) {
             const float ax = fabsf(xb[j]);
             if (ax > amax) amax = ax;
         }
-        const float d = amax / 127.0f;
-        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const int big = amax / 127.0f > 65504.0f;
+        const float d = big ? 65504.0f : amax / 127.0f;
+        const float inv = amax == 0.0f ? 0.0f : big ? 1.0f / 65504.0f : 127.0f / amax;
         out[b].d = mo_f32_to_f16(d);
-        for (int j = 0; j < 32; ++j) out[b].qs[j] = (int8_t) roundf(xb[j] * id);
+        for (int j = 0; j < 32; ++j) {
+            float r = nearbyintf(xb[j] * inv); /* the default rounding mode: to nearest, ties to even */
+            r = r > 127.0f ? 127.0f : r < -128.0f ? -128.0f : r;
+            out[b].qs[j] = (int8_t) r;
+        }
     }
 }
 
@@ -446,7 +457,7 @@ static float dot_iq1_m(const uint8_t* row, int nb, const mo_q8k* y) {
     return fmaf(0.125f, hsum8(deltaf), hsum8(accf));
 }
 
-/* IQ1_S x Q8_K: ggml's generic form (no ggml-free twin in the reference tree: PARITY UNPINNED, see the header);
+/* IQ1_S x Q8_K: ggml's generic form (no ggml-free twin in the reference tree; pinned through the IQ1_M carrier, see the header);
  * per block sumf += d * y.d * (sumi + IQ1S_DELTA * sumi1), following the decode of iq_kernels.cu:825-837 */
 static float dot_iq1_s(const uint8_t* row, int nb, const mo_q8k* y) {
     const uint64_t* grid = mo_iq1s_grid();
@@ -470,7 +481,7 @@ static float dot_iq1_s(const uint8_t* row, int nb, const mo_q8k* y) {
     return sumf;
 }
 
-/* Q8_0 x Q8_0: ggml's generic form (PARITY UNPINNED at the ggml boundary): sumf += sumi * (d_w * d_y) per 32 */
+/* Q8_0 x Q8_0: ggml's generic form: sumf += sumi * (d_w * d_y) per 32 (pinned by an independent float64 product) */
 static float dot_q8_0(const uint8_t* row, int nb, const mo_q80* y) {
     float sumf = 0.0f;
     for (int i = 0; i < nb; ++i) {

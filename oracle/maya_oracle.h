@@ -15,12 +15,25 @@
  *   IQ2_S dequant .................... structure check |w| = d(2ls+1)/8 * {8,25,43}; integer decode identical to the
  *                                       reference build's Fmt32<22>::decode through the row dots below; codebook CRC
  *   IQ1_M dequant .................... integer decode pinned through the reference build's iq256_rows(29,...)
- *   IQ1_S dequant / dot .............. PARITY UNPINNED at the ggml boundary (no ggml-free test in the reference tree);
- *                                       checked only against the double dot of its own dequantized values
+ *   IQ1_S dequant .................... an independent numpy decode written from the block layout and dq_iq1_s's formula
+ *                                       (ggml-common.h:425-430, src/kernels/cuda/iq_kernels.cu:825-837), bit for bit over every
+ *                                       grid index x 3-bit scale x delta sign and on random blocks; the same values, bit for bit,
+ *                                       as the IQ1_M block that carries the IQ1_S block's fields (tests/test_oracle_pins.py)
+ *   IQ1_S row dot .................... the IQ1_M dot of that carrier block (itself bit-exact with the reference build's
+ *                                       iq256_rows(29, ...)) and the reference build on the carrier, to 1e-6 of the terms'
+ *                                       magnitude (only the order of the float sums differs); the float64 dot of the independent
+ *                                       decode; block-permutation and block-scale invariants
  *   Q8_K activation quantizer ........ reference build: strata::ds4::par::quant (ds4_lane_parity.cpp:610-637) byte-exact;
  *                                       constructed exact ties
- *   Q8_0 activation quantizer / Q8_0 x Q8_0 dot ... PARITY UNPINNED at the ggml boundary (text spec only:
- *                                       include/strata/kernels/quantize_act.hpp:28-31); checked against its closed form
+ *   Q8_0 activation quantizer ........ the reference's own x86 quantizer (quantize_oracle_q8_0 behind act_quant_q8_1,
+ *                                       src/kernels/cpu/expert.cpp:92-130, compiled where it lies into oracle/_ref/libmaya_ref_q80.so):
+ *                                       byte-exact on tests/golden/refbuild_q80_vectors.npz (the reference test's five
+ *                                       distributions, both-sign maxima, scales past the FP16 range and in its subnormals) and live
+ *                                       where that build exists; an independent float32 numpy closed form incl. exact halves of
+ *                                       either sign and zero blocks; ggml's scalar form and the reference's GPU form counted
+ *                                       against it (one code apart on < 2e-4 of N(0,1) values)
+ *   Q8_0 x Q8_0 row dot .............. the float64 dot of both operands dequantized independently with numpy, 1e-6 of the terms'
+ *                                       magnitude; block-permutation and negation invariants (exact where they must be)
  *   row dots IQ2_S / Q4_K / IQ1_M .... reference build: strata::kernels::cpu::iq256_rows / iq256_gu_rows, BIT-EXACT
  *                                       (this file restates the 8 int32 lanes and the float steps in their order)
  *   IQ2_S expert in device arithmetic  reference build: strata::ds4::par::gate_up_ref / down_ref, bit-exact

@@ -1,4 +1,4 @@
-// maya_dev.cuh - device-side building blocks shared by the kernels: scalar conversions, unaligned loads, wave64
+// maya_dev.hpp - device-side building blocks shared by the kernels: scalar conversions, unaligned loads, wave64
 // reductions and the per-format decoders of a quantized block into int8 codes and integer scales.
 //
 // One decoded "unit" of a row is the work of one lane for one step.  Every format reduces to

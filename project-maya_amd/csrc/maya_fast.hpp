@@ -1,4 +1,4 @@
-// maya_fast.cuh - the single-token streaming kernels for IQ2_S experts (the decode layer's hot loops).
+// maya_fast.hpp - the single-token streaming kernels for IQ2_S experts (the decode layer's hot loops).
 //
 // Both kernels are HBM-bound streams over raw GGUF rows.  A lane owns the same 32-value sub-block positions of every
 // row it touches, so its slice of the int8 activation lives in registers for the whole kernel; a row's quantized bytes
@@ -10,7 +10,7 @@
 // because g ^ 0xff = -g - 1 as int8 and m = -1 there; every term is an exact integer.
 #pragma once
 
-#include "maya_dev.cuh"
+#include "maya_dev.hpp"
 
 namespace maya {
 
@@ -420,32 +420,9 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
                 g += part[buf][w][t];
                 up += part[buf][NW + w][t];
             }
-            // (a device-coherent store: another workgroup may read the row back to round h, with no cache flush between)
-            if (r0 + r + t < n_ff)
-                __hip_atomic_store(a.h + (size_t) e * n_ff + r0 + r + t, swiglu(g, up, a.limit), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (r0 + r + t < n_ff) a.h[(size_t) e * n_ff + r0 + r + t] = swiglu(g, up, a.limit);
         }
     }
-    if constexpr (NW < 4) return;   // (the block rounding below wants 256 threads; narrower rows leave it to the down kernel)
-    if (a.hq_sync == nullptr) return;
-    // The Q8_K rounding of h for the down rows: the last of the 256 / ROWS workgroups that share a 256-value block
-    // of h rounds it.  The rows of h are written and read back with device-coherent accesses, so no cache-wide
-    // fence is needed (on this multi-die part a device-scope fence writes back and invalidates whole L2 caches): a
-    // writer waits for its stores to be acknowledged, the workgroup meets, and only then is its arrival counted.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    __shared__ int s_last;
-    const int blk = r0 >> 8, nblk = n_ff >> 8;
-    if (t == 0) {
-        const int seen = __hip_atomic_fetch_add(a.hq_sync + e * nblk + blk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = seen == 256 / ROWS - 1;
-    }
-    __syncthreads();
-    if (!s_last) return;
-    const bool active = t < 256;
-    const float hv = active ? __hip_atomic_load(a.h + (size_t) e * n_ff + (size_t) blk * 256 + t, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT)
-                            : 0.0f;
-    quant_q8k_block(hv, t, active, lds, a.hq, (size_t) e * n_ff + (size_t) blk * 256);
 }
 
 // ---- down + combine, one token, n_ff = 32 NU <= 2048 (NU sub-blocks a row on the first NU lanes of one wave; NU a

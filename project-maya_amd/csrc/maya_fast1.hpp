@@ -1,5 +1,5 @@
-// maya_fast1.cuh - position-mapped decode kernels for IQ1_S rows in the stream packing: the skeleton of the IQ2_S ones
-// (maya_fast.cuh) with a cheaper unit.  A value is d (2 s + 1) (g + delta / 8), g in {-1, 0, +1} from the 2048-entry
+// maya_fast1.hpp - position-mapped decode kernels for IQ1_S rows in the stream packing: the skeleton of the IQ2_S ones
+// (maya_fast.hpp) with a cheaper unit.  A value is d (2 s + 1) (g + delta / 8), g in {-1, 0, +1} from the 2048-entry
 // grid, delta = +-1 a sub-block (third_party/ggml/ggml-common.h:425-430, src/kernels/cuda/iq_kernels.cu:825-837), i.e.
 // the int8 code 8 g + delta.  The grid sits in LDS as t = 8 g + 9 (bytes 1 / 9 / 17), so a looked-up word is the operand
 // of the dot products as it is, and

@@ -1,4 +1,4 @@
-// maya_fastk.cuh - position-mapped decode kernels for Q4_K rows in their own GGUF order (blobs 16-byte aligned): the same
+// maya_fastk.hpp - position-mapped decode kernels for Q4_K rows in their own GGUF order (blobs 16-byte aligned): the same
 // skeleton as the IQ2_S ones.  A lane owns one 16-byte piece of every block's codes - the low nibbles are 16 values of
 // sub-block 2j, the high nibbles 16 values of sub-block 2j + 1 - so its 32 activation codes, their two sums and the
 // block's activation scale stay in registers while it walks down the rows; 8 lanes read a block's 128 code bytes as one

@@ -1,4 +1,4 @@
-// maya_fastmv.cuh - dense mat-vec jobs on the position-mapped skeleton of the expert kernels: a workgroup of NW waves =
+// maya_fastmv.hpp - dense mat-vec jobs on the position-mapped skeleton of the expert kernels: a workgroup of NW waves =
 // the 2 * 32 NW positions of a pair of adjacent rows (2 p on the first half of the lanes, 2 p + 1 on the second) of
 // n_in = 1024 NW values; a lane keeps its position, so a column's 32 activation codes stay in registers while the lane
 // walks down the rows, and a row pair is read in whole contiguous runs.  Q8_0 rows in the stream packing (codes, then

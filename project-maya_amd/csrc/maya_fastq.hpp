@@ -1,4 +1,4 @@
-// maya_fastq.cuh - position-mapped kernels for Q8_0 rows in the stream packing (a row = its k codes, then its k / 32 FP16
+// maya_fastq.hpp - position-mapped kernels for Q8_0 rows in the stream packing (a row = its k codes, then its k / 32 FP16
 // scales: aligned 16-byte loads; the GGUF order interleaves a 2-byte scale with every 32 codes).  Made for the expert
 // every token takes (a shared expert, a dense FFN): the tokens of a group share one read of the weights.  A lane owns
 // one 32-value block position; the batch of a step is 8 (row, token) values - 8 / NT rows of NT tokens - so one

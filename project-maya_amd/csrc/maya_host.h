@@ -8,7 +8,7 @@
 #include <stdio.h>
 
 #include "../../include/maya_moe.h"
-#include "maya_dev.cuh"
+#include "maya_dev.hpp"
 
 namespace maya {
 

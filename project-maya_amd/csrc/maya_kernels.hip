@@ -406,8 +406,9 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const void* __restrict__
     quant_q8k_block(xv, j, true, sm, out, (size_t) row * k + (size_t) b * 256);
 }
 
-// Q8_0: 32-value blocks, d = amax / 127 kept as FP16, q = roundf(x / d) with the unrounded F32 d
-// (include/strata/kernels/quantize_act.hpp:28-31).  256 threads = 8 blocks.
+// Q8_0: 32-value blocks in the CPU expert path's rounding on x86 (ggml-cpu's quantize_row_q8_0 as the reference restates
+// it, src/kernels/cpu/expert.cpp:92-130): d = amax / 127 kept as FP16 (65504 when larger), q = nearest-even(x * (127 / amax))
+// with the product rounded to F32 first.  256 threads = 8 blocks.
 template <int DT>
 __global__ __launch_bounds__(256) void quant_q80_kernel(const void* __restrict__ x, int64_t x_stride, int64_t k,
                                                         maya_act out) {
@@ -417,9 +418,11 @@ __global__ __launch_bounds__(256) void quant_q80_kernel(const void* __restrict__
     float am = fabsf(xv);
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, kWave));
-    const float d = __fdiv_rn(am, 127.0f);
-    const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
-    const int q = (int) roundf(__fmul_rn(xv, id));
+    const float d0 = __fdiv_rn(am, 127.0f);
+    const bool big = d0 > 65504.0f;
+    const float d = big ? 65504.0f : d0;
+    const float inv = am == 0.0f ? 0.0f : big ? __fdiv_rn(1.0f, 65504.0f) : __fdiv_rn(127.0f, am);
+    const int q = max(-128, min(127, (int) rintf(__fmul_rn(xv, inv))));
     const size_t base = (size_t) row * k + v;
     out.q[base] = (int8_t) q;
     int s = q;
@@ -757,21 +760,18 @@ __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ l
 }
 
 // The layer's head in one launch, grid (1 + n_embd / 256, n_tokens): workgroup 0 of a token routes it, writes its
-// plan slots (blob addresses from the residency table) and - for token 0 - clears the gate/up kernels' arrival
-// counters; the other workgroups round one 256-value block of the hidden state each to Q8_K.
+// plan slots (blob addresses from the residency table); the other workgroups round one 256-value block of the hidden
+// state each to Q8_K.
 template <int DT>
 __global__ __launch_bounds__(256) void layer_head_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec rs,
                                                          const uint64_t* __restrict__ table, int32_t* __restrict__ ids,
                                                          float* __restrict__ weights, uint64_t* __restrict__ plan,
-                                                         const void* __restrict__ x, int64_t n_embd, maya_act xq,
-                                                         int32_t* __restrict__ counters, int n_counters) {
+                                                         const void* __restrict__ x, int64_t n_embd, maya_act xq) {
     __shared__ RouterLds sm;
     __shared__ int qs[264];
     __shared__ uint64_t s_table[MAYA_MAX_EXPERTS];
     const int t = blockIdx.y;
     if (blockIdx.x == 0) {
-        if (t == 0)
-            for (int i = threadIdx.x; i < n_counters; i += 256) counters[i] = 0;
         // the residency table rides along in registers while the token is routed: the plan's look-up then costs no second
         // trip to memory after the ids are known
         uint64_t tab[MAYA_MAX_EXPERTS / 256];
@@ -1226,12 +1226,12 @@ __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb,
 
 }  // namespace maya
 
-#include "maya_fast.cuh"
-#include "maya_fast1.cuh"
-#include "maya_fastk.cuh"
-#include "maya_fastq.cuh"
-#include "maya_fastmv.cuh"
-#include "maya_tiers.cuh"
+#include "maya_fast.hpp"
+#include "maya_fast1.hpp"
+#include "maya_fastk.hpp"
+#include "maya_fastq.hpp"
+#include "maya_fastmv.hpp"
+#include "maya_tiers.hpp"
 
 namespace maya {
 
@@ -1387,14 +1387,6 @@ int try_gate_up_iq2s_1tok(const maya_moe_args& a, const DeviceState& st, hipStre
     if (l.n_embd % 1024 != 0 || l.n_embd > 8192 || l.n_ff % 32 != 0) return 0;
     *rc = launch_gate_up_iq2s_gguf(a, st, s);
     return 1;
-}
-// whether try_gate_up_iq2s_1tok would take the position-mapped kernel, which can round h itself (hq_sync)
-bool gate_up_fuses_hq(const maya_moe_args& a) {
-    const maya_moe_layout& l = a.layout;
-    if (!(l.gate_type == kIQ2_S && l.up_type == kIQ2_S && a.n_tokens == 1 && l.packing == MAYA_PACK_STREAM)) return false;
-    if (l.n_ff % 256 != 0 || l.n_embd % 1024 != 0 || !q8k_act(l.down_type)) return false;
-    const int nw = l.n_embd / 1024;
-    return nw == 4 || nw == 6 || nw == 7 || nw == 8;
 }
 // ---- IQ1_S / IQ1_M in the stream packing: the position-mapped kernels
 bool gate_up_iq1s_pos_ok(const maya_moe_args& a) {
@@ -1849,9 +1841,9 @@ int maya_moe_route_plan(const maya_router* router, const float* logits, int n_to
     if (!logits || !expert_table || !ids || !weights || !plan_ptr) return fail(MAYA_E_ARG, "route_plan: null pointer");
     if (n_tokens <= 0 || n_tokens > 65535 || n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k <= 0 || k > MAYA_MAX_K || k > n_expert)
         return fail(MAYA_E_SHAPE, "route_plan: tokens %d experts %d k %d (limits %d experts, k %d)", n_tokens, n_expert, k, MAYA_MAX_EXPERTS, MAYA_MAX_K);
-    // (the layer head's routing workgroup alone: no activation blocks, no counters)
+    // (the layer head's routing workgroup alone: no activation blocks)
     hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, dim3(1, (unsigned) n_tokens), dim3(256), 0, as_stream(stream), logits, n_expert, k, rs,
-                       expert_table, ids, weights, plan_ptr, nullptr, (int64_t) 0, maya_act{nullptr, nullptr, nullptr}, nullptr, 0);
+                       expert_table, ids, weights, plan_ptr, nullptr, (int64_t) 0, maya_act{nullptr, nullptr, nullptr});
     MAYA_LAUNCHED("layer_head_kernel");
     return MAYA_OK;
 }
@@ -1961,7 +1953,6 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     return fail(MAYA_E_UNSUPPORTED, "gate_up: no kernel for gate type %d with up type %d", tg, tu);
 }
 
-int maya_moe_gate_up_fuses_hq(const maya_moe_args* a) { return a && a->hq_sync && gate_up_fuses_hq(*a) ? 1 : 0; }
 int maya_moe_down_rounds_h(const maya_moe_args* a) { return a && down_rounds_h(*a) ? 1 : 0; }
 
 int maya_moe_down(const maya_moe_args* a, void* stream) {
@@ -2109,7 +2100,7 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
 // workspace carve-up of maya_moe_layer_decode (every region 256-byte aligned)
 struct LayerWs {
     uint64_t *plan_ptr, *grp_ptr;
-    int32_t *grp_start, *grp_ent, *n_groups, *hq_sync;
+    int32_t *grp_start, *grp_ent, *n_groups;
     maya_act x, hq;
     float *h, *part;
     size_t bytes;
@@ -2128,7 +2119,6 @@ static LayerWs carve(const maya_moe_layout& l, int n_tokens, int k, uint8_t* bas
     w.grp_start = (int32_t*) take(sizeof(int32_t) * (ne + 1));
     w.grp_ent = (int32_t*) take(sizeof(int32_t) * ne);
     w.n_groups = (int32_t*) take(sizeof(int32_t));
-    w.hq_sync = (int32_t*) take(sizeof(int32_t) * (size_t) ne * (l.n_ff / 256));
     w.x.q = (int8_t*) take((size_t) n_tokens * l.n_embd);
     w.x.d = (float*) take(sizeof(float) * (size_t) n_tokens * (l.n_embd / 32));
     w.x.bsums = (int16_t*) take(sizeof(int16_t) * (size_t) n_tokens * (l.n_embd / 16));
@@ -2182,18 +2172,16 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
     a.add = add;
     a.out = out;
     if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
-        // one launch: route, plan, Q8_K of x, cleared counters
-        const int n_counters = n_tokens * k * (l->n_ff / 256);
+        // one launch: route, plan, Q8_K of x
         const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
         hipStream_t s = as_stream(stream);
         if (k > n_expert) return fail(MAYA_E_SHAPE, "layer_decode: k %d > n_expert %d", k, n_expert);
         switch (x_dtype) {
-            case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
-            case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
-            default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x, w.hq_sync, n_counters); break;
+            case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x); break;
+            case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x); break;
+            default: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x); break;
         }
         MAYA_LAUNCHED("layer_head_kernel");
-        a.hq_sync = down_rounds_h(a) ? nullptr : w.hq_sync;   // (the down kernel's own rounding of h is the cheaper one)
     } else {
         if (logits && n_expert <= MAYA_MAX_EXPERTS) {
             if ((rc = maya_moe_route_plan(router, logits, n_tokens, n_expert, k, expert_table, ids, weights, w.plan_ptr, stream))) return rc;
@@ -2214,7 +2202,7 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
     if (down_rounds_h(a)) {
         a.hq = maya_act{nullptr, nullptr, nullptr};
         a.part = nullptr;
-    } else if (!maya_moe_gate_up_fuses_hq(&a)) {
+    } else {
         if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
     }
     return maya_moe_down(&a, stream);

@@ -580,7 +580,7 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     }
 }
 
-#include "maya_prefill_iq2s.cuh"
+#include "maya_prefill_iq2s.hpp"
 
 // grid (bands of weight rows, tiles at most)
 template <bool GU>

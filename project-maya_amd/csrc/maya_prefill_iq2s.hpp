@@ -1,4 +1,4 @@
-// maya_prefill_iq2s.cuh - the prompt chunk's grouped GEMM on IQ2_S rows in the stream packing (included by
+// maya_prefill_iq2s.hpp - the prompt chunk's grouped GEMM on IQ2_S rows in the stream packing (included by
 // maya_prefill.hip inside namespace maya; the skeleton - tiles, the activations' copies, the barriers - is pf_tile's).
 // out[row][n] = 1/8 sum over blocks b of (d_w[n][b] d_x[row][b]) * sum over the block's 16-value groups j of (2 ls_j +
 // 1) (w_j . c_j), w = the grid magnitudes with their signs: the integer sums of the CPU path's IQ2_S x Q8_K row dot

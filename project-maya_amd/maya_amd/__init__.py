@@ -4,6 +4,4 @@ and thin helpers that keep the reference's operator vocabulary (expert blobs, pl
 PyTorch is used for device memory and streams only; every computation runs in the library's HIP kernels.  There is no
 CPU fallback: importing `maya_amd.lib` raises when the built library is missing.
 """
-from . import synth  # noqa: F401
-
-__all__ = ["synth"]
+__all__ = ["lib", "exl3", "prefill", "expert_files", "build"]

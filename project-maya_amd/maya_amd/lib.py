@@ -20,7 +20,7 @@ EXPORTS = [
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
     "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
     "maya_moe_tab_update",
-    "maya_dequant_rows_packed", "maya_moe_gate_up_fuses_hq", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
+    "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
 ]
 
 
@@ -60,8 +60,7 @@ class Args(C.Structure):
     _fields_ = [("layout", Layout), ("n_tokens", C.c_int32), ("k", C.c_int32), ("plan_ptr", C.c_void_p),
                 ("plan_w", C.c_void_p), ("grp_ptr", C.c_void_p), ("grp_start", C.c_void_p), ("grp_ent", C.c_void_p),
                 ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", Act), ("h", C.c_void_p),
-                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p),
-                ("hq_sync", C.c_void_p)]
+                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p)]
 
 
 class MvJob(C.Structure):
@@ -104,7 +103,6 @@ def load():
     L.maya_moe_group.argtypes = [vp, i32, vp, vp, vp, vp, vp]
     L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
-    L.maya_moe_gate_up_fuses_hq.argtypes = [C.POINTER(Args)]
     L.maya_moe_down_rounds_h.argtypes = [C.POINTER(Args)]
     L.maya_mv_supported.argtypes = [i32]
     L.maya_mv.argtypes = [C.POINTER(MvJob), i32, vp]

@@ -14,10 +14,10 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-sys.path[:0] = [os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle")]
+sys.path[:0] = [os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle"), os.path.join(ROOT, "tests")]
 
 import oracle_py  # noqa: E402
-from maya_amd import synth  # noqa: E402
+import synth  # noqa: E402
 
 
 def main():

@@ -2,7 +2,8 @@
 import numpy as np
 import torch
 
-from maya_amd import lib, synth
+import synth
+from maya_amd import lib
 
 
 def rel_l2(got, want):

@@ -62,8 +62,3 @@ def blob_offsets(gu_type, d_type, n_embd, n_ff, up_type=None):
     up_off = n_ff * row_bytes(gu_type, n_embd)
     down_off = up_off + n_ff * row_bytes(up_type, n_embd)
     return up_off, down_off, down_off + n_embd * row_bytes(d_type, n_ff)
-
-
-def zipf_bias(n_expert, s=1.1):
-    """The prefill config's routing skew: b_e = log(1 / (e + 1)^s), added to N(0, 1) router logits."""
-    return (-s * np.log(np.arange(1, n_expert + 1, dtype=np.float64))).astype(np.float32)

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from maya_amd import expert_files as ef
-from maya_amd import synth
+import synth
 
 
 def _s(x):

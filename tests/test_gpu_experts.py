@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from gpu_util import dev, make_experts, oracle_layer, rel_l2
-from maya_amd import synth
+import synth
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -107,6 +107,37 @@ def test_layer_matches_cpu_path(lib, oracle, gt, dt, n_embd, n_ff, ne, k, nt, pa
     assert np.array_equal(ids, wi)
     for t in range(nt):
         assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
+
+
+def encoded_q4k_expert(oracle, n_embd, n_ff, seed):
+    """One expert as BASELINE's single-expert configuration states it: gate / up [n_ff x n_embd] and down [n_embd x n_ff]
+    drawn from N(0, 0.02) in F32 and quantized to Q4_K (the checker's own encoder: the reference never quantizes weights)."""
+    rng = np.random.default_rng(seed)
+    return np.concatenate([oracle.encode_q4k((rng.standard_normal(rows * cols) * 0.02).astype(np.float32))
+                           for rows, cols in ((n_ff, n_embd), (n_ff, n_embd), (n_embd, n_ff))])
+
+
+@pytest.mark.parametrize("ne,k,nt,packing", ((1, 1, 1, 1), (2, 2, 2, 1), (1, 1, 1, 0), (2, 1, 2, 1)))
+def test_single_expert_glu_q4k_from_gaussian_weights(lib, oracle, ne, k, nt, packing):
+    """BASELINE's first configuration at its full size: one Q4_K expert GLU of 7168 x 2048 on one F32 token (and two experts
+    on two tokens).  One or two plan slots on few tokens select the kernels' smallest tiles - 8 gate/up row pairs and 8
+    down rows a workgroup - which no other case reaches."""
+    n_embd, n_ff = 7168, 2048
+    blobs = [encoded_q4k_expert(oracle, n_embd, n_ff, 500 + e) for e in range(ne)]
+    rng = np.random.default_rng(510 + nt)
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    x = rng.standard_normal((nt, n_embd)).astype(np.float32)
+    ids, w, out, _ = run_layer(lib, 12, 12, blobs, k, n_embd, n_ff, logits, x, packing=packing)
+    wi, ww, wout = oracle_layer(oracle, 12, 12, blobs, k, n_embd, n_ff, logits, x)
+    assert np.array_equal(ids, wi)
+    for t in range(nt):
+        assert np.abs(wout[t]).max() > 0
+        assert rel_l2(out[t], wout[t]) <= TOL, (t, rel_l2(out[t], wout[t]))
+    if ne == 1:
+        # out = down(silu(gate x) * (up x)) with weight 1: the expert alone
+        want = oracle.expert(12, 12, blobs[0], blobs[0][n_ff * (n_embd // 256) * 144:], blobs[0][2 * n_ff * (n_embd // 256) * 144:],
+                             n_embd, n_ff, x)
+        assert rel_l2(out[0], want[0]) <= TOL
 
 
 @pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt,packing,norm", (

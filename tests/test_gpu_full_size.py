@@ -7,7 +7,8 @@ import pytest
 import torch
 
 from gpu_util import oracle_layer, rel_l2
-from maya_amd import workloads
+import bench_workloads as workloads
+from bench_workloads import zipf_bias
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -91,11 +92,12 @@ def test_eight_tokens_mixed_experts_and_the_shared_expert(lib, oracle):
 def test_prompt_chunk_512_tokens_256_q4k_experts(lib, oracle):
     """configs[3]: 512 tokens, 256 Q4_K experts, top-8, Zipf(1.1)-skewed routing: the ids of every token, the chunk's rows of
     sampled tokens against the CPU path, and every sampled row against the decode layer's for that token alone."""
-    from maya_amd import prefill, synth
+    from maya_amd import prefill
+    import synth
     T = 512
     gguf, bb, view, packed, table = make_pool(lib, Q4_K, Q4_K, NE, 301)
     rng = np.random.default_rng(302)
-    logits = (rng.standard_normal((T, NE)) + synth.zipf_bias(NE)).astype(np.float32)
+    logits = (rng.standard_normal((T, NE)) + zipf_bias(NE)).astype(np.float32)
     x = rng.standard_normal((T, E)).astype(np.float32)
     xd, ld = torch.from_numpy(x).cuda(), torch.from_numpy(logits).cuda()
     chunk = prefill.PrefillLayer(lib.copy_layout(gguf, lib.PACK_STREAM), NE, TK, T, out_dtype=torch.float32)

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from gpu_util import dev, rel_l2
-from maya_amd import synth
+import synth
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3

@@ -4,6 +4,8 @@ reference's CPU expert path, stage by stage: every row of the chunk is that path
 import numpy as np
 import pytest
 
+from bench_workloads import zipf_bias
+
 pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
@@ -20,7 +22,7 @@ def pf():
 
 
 def make_blobs(oracle, n_expert, n_embd, n_ff, seed, encoded=False):
-    from maya_amd import synth
+    import synth
     rng = np.random.default_rng(seed)
     if not encoded:
         return [synth.expert_blob(Q4_K, Q4_K, n_embd, n_ff, rng) for _ in range(n_expert)]
@@ -36,9 +38,9 @@ PLAN_CASES = [(1, 1, 4, 0), (37, 2, 8, 1), (64, 8, 256, 2), (512, 8, 256, 3), (3
 
 @pytest.mark.parametrize("n_tokens,k,n_expert,seed", PLAN_CASES)
 def test_plan_matches_stable_sort(pf, oracle, n_tokens, k, n_expert, seed):
-    from maya_amd import synth
+    import synth
     rng = np.random.default_rng(seed)
-    logits = rng.standard_normal((n_tokens, n_expert)).astype(np.float32) + synth.zipf_bias(n_expert)
+    logits = rng.standard_normal((n_tokens, n_expert)).astype(np.float32) + zipf_bias(n_expert)
     ids = np.argsort(-logits, axis=1, kind="stable")[:, :min(k, n_expert)].astype(np.int32)
     if seed == 4:
         ids[5, 1] = -3            # out-of-range ids are dropped
@@ -101,7 +103,8 @@ LAYER_CASES = [
 
 @pytest.mark.parametrize("case", LAYER_CASES, ids=[str(c[:5]) for c in LAYER_CASES])
 def test_stages_and_layer_match_checker(pf, oracle, case):
-    from maya_amd import lib, synth
+    from maya_amd import lib
+    import synth
     n_embd, n_ff, n_expert, k, n_tokens, limit, encoded, absent = case
     blobs = make_blobs(oracle, n_expert, n_embd, n_ff, 50 + n_embd, encoded)
     up_off, down_off, _ = synth.blob_offsets(Q4_K, Q4_K, n_embd, n_ff)
@@ -112,7 +115,7 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
         table[e] = 0
         resident[e] = False
     rng = np.random.default_rng(n_tokens)
-    logits = (rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32)
+    logits = (rng.standard_normal((n_tokens, n_expert)) + zipf_bias(n_expert)).astype(np.float32)
     x = rng.standard_normal((n_tokens, n_embd)).astype(np.float32)
     want = oracle.prefill_layer(Q4_K, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit, resident)
     layout, _ = lib.layout(Q4_K, Q4_K, n_embd, n_ff)
@@ -172,7 +175,8 @@ IQ_CASES = [
 @pytest.mark.parametrize("case", IQ_CASES, ids=[str(c[:7]) for c in IQ_CASES])
 def test_iq2s_chunk_matches_checker(pf, oracle, case):
     """The IQ2_S GEMMs (stream packing) and their mix with Q4_K: h, the down rows and the layer against the CPU path."""
-    from maya_amd import lib, synth
+    from maya_amd import lib
+    import synth
     gt, dt, n_embd, n_ff, n_expert, k, n_tokens, limit, absent = case
     rng = np.random.default_rng(900 + n_embd + gt)
     blobs = [synth.expert_blob(gt, dt, n_embd, n_ff, rng) for _ in range(n_expert)]
@@ -185,7 +189,7 @@ def test_iq2s_chunk_matches_checker(pf, oracle, case):
     for e in absent:
         table[e] = 0
         resident[e] = False
-    logits = (rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32)
+    logits = (rng.standard_normal((n_tokens, n_expert)) + zipf_bias(n_expert)).astype(np.float32)
     x = rng.standard_normal((n_tokens, n_embd)).astype(np.float32)
     want = oracle.prefill_layer((gt, dt), blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit, resident)
     ids, w = lib.route_topk(dev(logits), k)
@@ -213,13 +217,14 @@ def test_chunk_tokens_equal_the_decode_layer(pf):
     """Two independent GPU paths, one contract: a token's row of the prompt chunk (grouped int8-MFMA GEMMs) is what the
     decode layer (dot-product mat-vecs) gives for that token alone - the same Q8_K codes and integer sums, F32 sums in
     another order."""
-    from maya_amd import lib, synth
+    from maya_amd import lib
+    import synth
     n_embd, n_ff, n_expert, k, n_tokens = 7168, 2048, 6, 3, 40
     rng = np.random.default_rng(77)
     blobs = [synth.expert_blob(Q4_K, Q4_K, n_embd, n_ff, rng) for _ in range(n_expert)]
     store = lib.ExpertStore(blobs)
     layout, _ = lib.layout(Q4_K, Q4_K, n_embd, n_ff)
-    logits = dev((rng.standard_normal((n_tokens, n_expert)) + synth.zipf_bias(n_expert)).astype(np.float32))
+    logits = dev((rng.standard_normal((n_tokens, n_expert)) + zipf_bias(n_expert)).astype(np.float32))
     x = dev(rng.standard_normal((n_tokens, n_embd)).astype(np.float32))
     chunk = pf.PrefillLayer(layout, n_expert, k, n_tokens, out_dtype=torch.float32).forward(store.table, logits, x, limit=5.0).clone()
     dec = lib.MoeLayer(Q4_K, Q4_K, n_embd, n_ff, n_expert, k, max_tokens=8)

@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from maya_amd import synth
+import synth
 
 
 def test_f16_to_f32_exhaustive(oracle):

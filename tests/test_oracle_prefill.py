@@ -7,7 +7,7 @@ Q4_K, Q8_0 = 12, 8
 
 
 def test_grouped_ref_equals_numpy_product(oracle):
-    from maya_amd import synth
+    import synth
     rng = np.random.default_rng(3)
     k, n, ne = 512, 24, 3
     mats = [synth.constructed_rows(Q4_K, n, k, rng) for _ in range(ne)]

@@ -6,7 +6,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from maya_amd import synth
+import synth
 
 TYPES_256 = (22, 12, 29)
 
