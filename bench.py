@@ -1,30 +1,35 @@
 #!/usr/bin/env python3
-"""bench.py - the routed MoE decode layer on one MI355X (BASELINE.json configs[1]).
+"""bench.py - the routed MoE expert block on one MI355X: BASELINE.json's metric on configs[1] (the decode layer), with
+configs[3] (the 512-token prompt chunk, the metric's second half) as a sub-object of the same line.
 
-A step is one pass of the layer over one token: router top-8 of 256 experts, plan, Q8_K rounding of the bf16 hidden
+A decode step is one pass of the layer over one token: router top-8 of 256 experts, plan, Q8_K rounding of the bf16 hidden
 state, fused dequant gate/up GLU mat-vec over the 8 routed IQ2_S experts, Q8_K rounding of h, down mat-vec, weighted
 combine.  All 256 experts (3.6 GB) are resident in HBM; consecutive steps route to disjoint expert sets (32 sets of 8),
-so no step re-reads weights that an earlier step left in the on-die caches.  The K timed steps are one HIP graph
-(the reference's timing method, tests/hip/expert_kernel_bench.cpp:136-172), bracketed by device synchronisations.
+so no step re-reads weights that an earlier step left in the on-die caches.  The K steps are one HIP graph (the
+reference's timing method, tests/hip/expert_kernel_bench.cpp:136-172): untimed replays until two in a row agree within
+1 %, then 7 timed replays bracketed by device synchronisations, the median.
 
 value = algorithmic HBM bytes of a step (weights of the 8 routed experts + logits + x + out) / time per step, GB/s.
-roofline = the gate/up kernel alone: its algorithmic bytes / its average duration measured with HIP events.
-cpu_baseline = the reference's CPU expert path on this host's cores, same inputs, a bounded sample.
+roofline = the dominant kernel (gate/up: two thirds of the bytes): its algorithmic bytes / its average launch duration
+measured with HIP events on the launch stream; roofline.layer = the same for the whole step.
+cpu_baseline = the reference's CPU expert path on this host's physical cores (pinned pool, rotating expert sets, median).
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle")):
+for _p in (ROOT, os.path.join(ROOT, "project-maya_amd"), os.path.join(ROOT, "oracle")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
 N_EMBD, N_FF, N_EXPERT, TOP_K = 7168, 2048, 256, 8
 IQ2_S = 22
 HBM_PEAK = 8.0e12
+PARITY_BAR = 1e-3
 # HBM bytes of one gate/up launch on this workload from rocprofv3's FETCH_SIZE and WRITE_SIZE (two runs, each scaled by
 # what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,783.1 KiB read + 64.0 KiB written
 # (profiles/decode_iq2s_hbm_traffic_pmc.txt)
@@ -65,118 +70,76 @@ def rotating_logits(np, n_sets, seed):
     return out
 
 
-def cpu_baseline(np, torch, oracle_py, pool, blob_bytes, logits_row, x_f32, gpu_out):
-    """The reference CPU expert path for one step's 8 routed experts on this host's cores: Q8_K activation, gate/up rows,
-    SwiGLU, Q8_K of h, down rows, weighted sum - rows split over the threads as ExpertPool::run_split_multi_native does.
-    Uses the reference build (oracle/_ref, the reference's own iq_avx2.cpp) when it travelled here, else the C port."""
-    import ctypes as C
-    from concurrent.futures import ThreadPoolExecutor
-    cores = max(1, min(16, len(os.sched_getaffinity(0))))
-    ids, w = oracle_py.router_topk(logits_row[None, :], TOP_K)
-    ids, w = ids[0], w[0]
-    blobs = [pool[int(e) * blob_bytes:(int(e) + 1) * blob_bytes].cpu().numpy() for e in ids]
-    gr, dr = oracle_py.row_bytes(IQ2_S, N_EMBD), oracle_py.row_bytes(IQ2_S, N_FF)
-    up_off, down_off = gr * N_FF, 2 * gr * N_FF
+def physical_cores(limit=16):
+    """One logical CPU per physical core among those this process may run on (the reference pins one worker per physical
+    core, include/strata/kernels/cpu/pool.hpp:66-72), at most `limit`; and the CPU's model string."""
+    allowed = sorted(os.sched_getaffinity(0))
+    seen, cpus = set(), []
+    for c in allowed:
+        try:
+            sib = open("/sys/devices/system/cpu/cpu%d/topology/thread_siblings_list" % c).read().strip()
+        except OSError:
+            sib = str(c)
+        if sib not in seen:
+            seen.add(sib)
+            cpus.append(c)
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return cpus[:limit], len(cpus), model
+
+
+def cpu_baseline(np, oracle_py, gguf_pool, blob_bytes, logits_np, x_f32, n_sets=5, max_seconds=10.0):
+    """The reference CPU expert path for one token's 8 routed experts on this host: oracle/cpu_bench.c's pinned spinning
+    pool, rows split over the threads as ExpertPool::run_split_multi_native does, n_sets disjoint expert sets (5 x 113 MB)
+    rotating so every call streams from DRAM, at least 7 passes over the sets, the median call.  The row kernels are the
+    reference's own iq_avx2.cpp (oracle/_ref, kind "reference") when that build travelled here, else the C port.
+    Returns the cpu_baseline object and the output of the last call (expert set n_sets - 1)."""
+    cpus, n_phys, model = physical_cores()
+    ids, w = oracle_py.router_topk(logits_np[:n_sets], TOP_K)
+    host = [gguf_pool[int(e) * blob_bytes:(int(e) + 1) * blob_bytes].cpu().numpy() for e in ids.reshape(-1)]
+    blobs = (C.c_void_p * len(host))(*[b.ctypes.data for b in host])
     ref = oracle_py.ref()
-    kind = "reference" if ref is not None else "port"
-    pool_ex = ThreadPoolExecutor(cores)
-
-    def one_layer():
-        act = oracle_py.quant_q8k(x_f32)
-        actp = (C.c_void_p * 1)(act.ctypes.data)
-        parts = np.zeros((TOP_K, N_EMBD), dtype=np.float32)
-        for i, b in enumerate(blobs):
-            h = np.zeros(N_FF, dtype=np.float32)
-            hp = (C.c_void_p * 1)(h.ctypes.data)
-            if ref is not None:
-                def gu(c):
-                    ref.ref_iq256_gu_rows(IQ2_S, b.ctypes.data, gr, up_off, N_EMBD, actp, 1, hp, c[0], c[1])
-            else:
-                def gu(c):
-                    oracle_py.lib().mo_gu_rows(IQ2_S, b.ctypes.data, b.ctypes.data + up_off, gr, N_EMBD, actp, 1, hp, c[0],
-                                               c[1], float("inf"))
-            step = N_FF // (cores * 4)
-            list(pool_ex.map(gu, [(r, min(N_FF, r + step)) for r in range(0, N_FF, step)]))
-            hq = oracle_py.quant_q8k(h)
-            hqp = (C.c_void_p * 1)(hq.ctypes.data)
-            op = (C.c_void_p * 1)(parts[i].ctypes.data)
-            if ref is not None:
-                def dn(c):
-                    ref.ref_iq256_rows(IQ2_S, b.ctypes.data + down_off, dr, N_FF, hqp, 1, op, c[0], c[1])
-            else:
-                def dn(c):
-                    oracle_py.lib().mo_rows(IQ2_S, b.ctypes.data + down_off, dr, N_FF, hqp, 1, op, c[0], c[1])
-            step = N_EMBD // (cores * 4)
-            list(pool_ex.map(dn, [(r, min(N_EMBD, r + step)) for r in range(0, N_EMBD, step)]))
-        return oracle_py.combine(parts, w)
-
-    if ref is None:
-        L = oracle_py.lib()
-        L.mo_gu_rows.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int64, C.c_void_p, C.c_int, C.c_void_p,
-                                 C.c_int, C.c_int, C.c_float]
-        L.mo_rows.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_int64, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int]
-    out = one_layer()  # warm-up, and the parity check of the GPU result
-    err = float(np.linalg.norm(out.astype(np.float64) - gpu_out.astype(np.float64)) / np.linalg.norm(out.astype(np.float64)))
-    times = []
-    t_end = time.perf_counter() + 12.0
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 40):
-        t0 = time.perf_counter()
-        one_layer()
-        times.append(time.perf_counter() - t0)
-    med = sorted(times)[len(times) // 2]
+    L = oracle_py.lib()
+    gu = C.cast(ref.ref_iq256_gu_rows, C.c_void_p) if ref is not None else None
+    rows = C.cast(ref.ref_iq256_rows, C.c_void_p) if ref is not None else None
+    rounds = 600
+    times = np.zeros(rounds * n_sets, dtype=np.float64)
+    n_done = C.c_int(0)
+    out = np.zeros(N_EMBD, dtype=np.float32)
+    cpu_arr = (C.c_int * len(cpus))(*cpus)
+    wts = np.ascontiguousarray(w, dtype=np.float32)
+    x = np.ascontiguousarray(x_f32, dtype=np.float32)
+    L.mo_bench_layer.restype = C.c_int
+    L.mo_bench_layer.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                 C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_double, C.c_void_p, C.c_void_p, C.c_void_p]
+    rc = L.mo_bench_layer(IQ2_S, blobs, n_sets, TOP_K, N_EMBD, N_FF, x.ctypes.data, wts.ctypes.data, gu, rows, len(cpus), cpu_arr,
+                          rounds, max_seconds, times.ctypes.data, C.byref(n_done), out.ctypes.data)
+    if rc != 0 or n_done.value < 1:
+        return None, None
+    t = np.sort(times[:n_done.value])
+    med = float(t[len(t) // 2])
     bytes_step = TOP_K * blob_bytes
-    return {"value": round(bytes_step / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind,
-            "us_per_step": round(med * 1e6, 1),
-            "sample": "%d layer calls of the same 8 routed IQ2_S experts (%d MB of weights each call), median" % (
-                len(times), bytes_step // 1000000)}, err
+    return {"value": round(bytes_step / med / 1e9, 2), "unit": "GB/s", "cores": len(cpus), "kind": "reference" if ref is not None else "port",
+            "us_per_step": round(med * 1e6, 1), "cpu_model": model, "physical_cores_available": n_phys,
+            "sample": "%d layer calls (%d passes over %d disjoint sets of the 8 routed IQ2_S experts, %d MB of weights a call, "
+                      "streamed from DRAM), one pinned thread a physical core, median call" % (
+                          n_done.value, n_done.value // n_sets, n_sets, bytes_step // 1000000)}, out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=32)
-    ap.add_argument("--no-graph", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="decode_iq2s",
-                    help="decode_iq2s (configs[1], the default and the headline metric), or one of the other BASELINE "
-                         "configurations: single_q4k, batch8_mixed, prefill_q4k, exl3_verify; the prefill chunk on other expert types: "
-                         "prefill_iq2s, prefill_mixed")
-    ap.add_argument("--calib-copy", action="store_true",
-                    help="also run one plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3's "
-                         "FETCH_SIZE / WRITE_SIZE counters by)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
+def rel_l2(np, got, want):
+    got, want = np.asarray(got, dtype=np.float64).reshape(-1), np.asarray(want, dtype=np.float64).reshape(-1)
+    den = np.linalg.norm(want)
+    return float(np.linalg.norm(got - want) / (den if den > 0 else 1.0))
 
-    import numpy as np
-    import torch
-    from maya_amd import lib
 
-    L = lib.load()
-    lib.check(L.maya_init())
-    info = L.maya_device_info().decode()
-    torch.cuda.set_device(0)
-    if args.calib_copy:
-        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    if args.workload != "decode_iq2s":
-        import bench_workloads as workloads
-        if args.workload not in workloads.WORKLOADS:
-            sys.exit("bench.py: unknown workload %r" % args.workload)
-        r = workloads.WORKLOADS[args.workload](args.steps, args.warmup)
-        r["config"]["device"] = info
-        line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
-                "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
-                "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
-                "cpu_baseline": None}
-        print(json.dumps(line))
-        return
+def decode_iq2s(args, np, torch, lib, L, info):
+    import bench_workloads as bw
     layer = lib.MoeLayer(IQ2_S, IQ2_S, N_EMBD, N_FF, N_EXPERT, TOP_K, max_tokens=1, packing=lib.PACK_STREAM)
     blob_bytes = layer.blob_bytes
     # GGUF blobs are made on the device, then regrouped into the stream packing as an engine's upload would do;
@@ -202,86 +165,74 @@ def main():
     def step(i):
         layer.forward(table, logits[i % n_sets:i % n_sets + 1], x)
 
-    with torch.cuda.stream(stream):
-        for i in range(W):
-            step(i)
-        stream.synchronize()
-        graph = None
-        if not args.no_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
+    if args.no_graph:
+        with torch.cuda.stream(stream):
+            for i in range(W):
+                step(i)
+            stream.synchronize()
+            times = []
+            for _ in range(bw.ROUNDS):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
                 for i in range(K):
                     step(W + i)
-            graph.replay()  # one untimed replay: the graph's first launch uploads it
-            stream.synchronize()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(K):
-                step(W + i)
-        stream.synchronize()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
+                stream.synchronize()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+            dt = sorted(times)[len(times) // 2]
+    else:
+        dt = bw.timed_graph(step, K, W, stream)
 
-        # ---- the dominant kernel alone (gate/up: 2/3 of the bytes), HIP events on the launch stream
-        import ctypes as C
+    # ---- the two weight-streaming kernels alone, HIP events on the launch stream (the stage calls of the C ABI on the
+    # same rotating plans; the down call given no rounded h rounds it itself, as it does inside the layer)
+    with torch.cuda.stream(stream):
         ids_all, w_all = lib.route_topk(logits, TOP_K)
         plans = lib.plan(ids_all.view(-1), table).view(n_sets, TOP_K)
         xq = lib.quant_act(IQ2_S, x.to(torch.float32))
         h = torch.empty((TOP_K, N_FF), dtype=torch.float32, device="cuda")
-        a = lib.Args()
-        a.layout = layer.layout
-        a.n_tokens, a.k = 1, TOP_K
-        a.limit = float("inf")
-        a.x = xq.c()
-        a.h = h.data_ptr()
+        outk = torch.empty((1, N_EMBD), dtype=torch.float32, device="cuda")
         arg_list = []
         for j in range(n_sets):
             b = lib.Args()
-            C.memmove(C.byref(b), C.byref(a), C.sizeof(a))
+            b.layout = layer.layout
+            b.n_tokens, b.k = 1, TOP_K
+            b.limit = float("inf")
+            b.x = xq.c()
+            b.h = h.data_ptr()
+            b.out = outk.data_ptr()
             b.plan_ptr = plans[j].data_ptr()
             b.plan_w = w_all[j].data_ptr()
             arg_list.append(b)
-        sp = C.c_void_p(stream.cuda_stream)
-        for j in range(8):
-            lib.check(L.maya_moe_gate_up(C.byref(arg_list[j]), sp))
-        stream.synchronize()
-        reps = max(K, 64)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        kg = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(kg, stream=stream):
-            for j in range(reps):
-                lib.check(L.maya_moe_gate_up(C.byref(arg_list[(8 + j) % n_sets]), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
-        kg.replay()
-        stream.synchronize()
-        e0.record(stream)
-        kg.replay()
-        e1.record(stream)
-        stream.synchronize()
-        gu_us = e0.elapsed_time(e1) * 1e3 / reps
+        assert L.maya_moe_down_rounds_h(C.byref(arg_list[0])) == 1
+        sp = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)   # noqa: E731
+        reps = 64
+        gu_s = bw.event_time(lambda i: lib.check(L.maya_moe_gate_up(C.byref(arg_list[(5 + i) % n_sets]), sp())), reps, stream)
+        dn_s = bw.event_time(lambda i: lib.check(L.maya_moe_down(C.byref(arg_list[(5 + i) % n_sets]), sp())), reps, stream)
 
-    step_us = dt / K * 1e6
+    sec = dt / K
     w_bytes = TOP_K * blob_bytes
     bytes_step = w_bytes + N_EXPERT * 4 + N_EMBD * 2 + N_EMBD * 4
-    value = bytes_step / (dt / K) / 1e9
+    value = bytes_step / sec / 1e9
     gu_bytes = TOP_K * 2 * N_FF * lib.row_bytes(IQ2_S, N_EMBD) + N_EMBD + (N_EMBD // 32) * 4 + TOP_K * N_FF * 4
-    gu_rate = gu_bytes / (gu_us * 1e-6) / 1e9
+    dn_bytes = TOP_K * N_EMBD * lib.row_bytes(IQ2_S, N_FF) + TOP_K * N_FF * 4 + N_EMBD * 4
+    gu_rate, dn_rate = gu_bytes / gu_s / 1e9, dn_bytes / dn_s / 1e9
 
-    # ---- parity of the timed configuration + CPU baseline on the same inputs
-    with torch.cuda.stream(stream):
-        out0 = layer.forward(table, logits[0:1], x).clone()
-        ids0 = layer.ids.clone()
-        stream.synchronize()
-    cpu, err = (None, None)
+    # ---- parity of the timed configuration + CPU baseline on the same inputs (after the timed regions)
+    cpu, err, ids_ok = None, None, None
     if not args.no_cpu:
         import oracle_py
-        cpu, err = cpu_baseline(np, torch, oracle_py, gguf_pool, blob_bytes, logits_np[0], x.to(torch.float32).cpu().numpy()[0],
-                                out0.cpu().numpy()[0])
-        wi, _ = oracle_py.router_topk(logits_np[0:1], TOP_K)
-        if not np.array_equal(wi, ids0.cpu().numpy()[:1]):
-            err = float("inf")
+        n_cpu_sets = 5
+        with torch.cuda.stream(stream):
+            out_g = layer.forward(table, logits[n_cpu_sets - 1:n_cpu_sets], x).clone()
+            ids_g = layer.ids.clone()
+            stream.synchronize()
+        cpu, out_c = cpu_baseline(np, oracle_py, gguf_pool, blob_bytes, logits_np, x.to(torch.float32).cpu().numpy()[0], n_cpu_sets)
+        wi, _ = oracle_py.router_topk(logits_np[n_cpu_sets - 1:n_cpu_sets], TOP_K)
+        ids_ok = bool(np.array_equal(wi, ids_g.cpu().numpy()[:1]))
+        if out_c is not None:
+            err = rel_l2(np, out_g.cpu().numpy()[0], out_c)
+    del pool, gguf_pool, table
+    torch.cuda.empty_cache()
 
     line = {
         "metric": "moe_layer_decode_hbm_gbps_1tok",
@@ -290,8 +241,8 @@ def main():
         "n_gpus": 1,
         "steps": K,
         "warmup": W,
-        "ms_per_step": round(step_us / 1e3, 6),
-        "us_per_layer": round(step_us, 3),
+        "ms_per_step": round(sec * 1e3, 6),
+        "us_per_layer": round(sec * 1e6, 3),
         "pct_of_hbm_peak": round(100.0 * value * 1e9 / HBM_PEAK, 2),
         "higher_is_better": True,
         "scaling": "weak",
@@ -303,14 +254,108 @@ def main():
                                "rotate over the steps",
                    "n_embd": N_EMBD, "n_ff": N_FF, "n_expert": N_EXPERT, "top_k": TOP_K, "tokens": 1,
                    "weight_bytes_per_step": w_bytes, "algorithmic_bytes_per_step": bytes_step,
-                   "timed_as": "eager launches" if args.no_graph else "one HIP graph of the K steps", "device": info},
+                   "timed_as": ("eager launches" if args.no_graph else "one HIP graph of the K steps") +
+                               ", median of %d replays after the clocks settled" % bw.ROUNDS, "device": info},
         "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_pos_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
                      "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
-                     "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 3)},
+                     "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_s * 1e6, 3),
+                     "down_kernel": {"kernel": "down_iq2s_pos_kernel", "achieved": round(dn_rate, 2), "frac": round(dn_rate * 1e9 / HBM_PEAK, 4),
+                                     "algorithmic_bytes_per_launch": dn_bytes, "avg_launch_us": round(dn_s * 1e6, 3)},
+                     "layer": {"achieved": round(value, 2), "frac": round(value * 1e9 / HBM_PEAK, 4),
+                               "algorithmic_bytes_per_step": bytes_step, "us_per_step": round(sec * 1e6, 3),
+                               "us_outside_the_two_kernels": round((sec - gu_s - dn_s) * 1e6, 3)}},
         "cpu_baseline": cpu,
         "parity_rel_l2_vs_cpu_path": err,
+        "parity_ids_exact": ids_ok,
     }
+    ok = args.no_cpu or (ids_ok and err is not None and err <= PARITY_BAR)
+    return line, ok
+
+
+def parity_of(np, torch, r):
+    """The CPU path's expert on a workload's own bytes (workloads that hand back a `_parity` record)."""
+    import oracle_py
+    p = r.pop("_parity", None)
+    if p is None:
+        return None
+    blob = p["blob"].cpu().numpy()
+    gr = oracle_py.row_bytes(p["type"], p["n_embd"])
+    up_off, down_off = gr * p["n_ff"], 2 * gr * p["n_ff"]
+    want = oracle_py.expert(p["type"], p["type"], blob, blob[up_off:], blob[down_off:], p["n_embd"], p["n_ff"],
+                            p["x"].to(torch.float32).cpu().numpy())
+    return rel_l2(np, p["out"].cpu().numpy(), want)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--no-graph", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity leg")
+    ap.add_argument("--no-prefill", action="store_true", help="leave the prompt-chunk sub-object out of the default line")
+    ap.add_argument("--workload", default="decode_iq2s",
+                    help="decode_iq2s (configs[1], the default and the headline metric), or one of the other BASELINE "
+                         "configurations: single_q4k, batch8_mixed, prefill_q4k, exl3_verify; the prefill chunk on other expert types: "
+                         "prefill_iq2s, prefill_mixed")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters by)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (nothing here uses a second GPU)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from maya_amd import lib
+    import bench_workloads as workloads
+
+    L = lib.load()
+    lib.check(L.maya_init())
+    info = L.maya_device_info().decode()
+    torch.cuda.set_device(0)
+    if args.calib_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.workload != "decode_iq2s":
+        if args.workload not in workloads.WORKLOADS:
+            sys.exit("bench.py: unknown workload %r" % args.workload)
+        r = workloads.WORKLOADS[args.workload](args.steps, args.warmup)
+        r["config"]["device"] = info
+        err = None if args.no_cpu else parity_of(np, torch, r)
+        r.pop("_parity", None)
+        line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
+                "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
+                "cpu_baseline": None, "parity_rel_l2_vs_cpu_path": err}
+        print(json.dumps(line))
+        if err is not None and not err <= PARITY_BAR:
+            print("bench.py: parity failed: relative L2 %g against the CPU path" % err, file=sys.stderr)
+            sys.exit(3)
+        return
+
+    line, ok = decode_iq2s(args, np, torch, lib, L, info)
+    if not args.no_prefill:
+        # BASELINE's second metric, the 512-token prompt chunk (configs[3]), in the same line; bench.py --workload prefill_q4k
+        # gives the same numbers alone
+        ksteps = max(4, min(16, args.steps))
+        r = workloads.prefill_q4k(ksteps, 2)
+        line["prefill"] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "ms_per_chunk": round(r["ms_per_step"], 4),
+                           "steps": ksteps, "pct_of_int8_peak": round(100.0 * r["value"] * 1e12 / workloads.INT8_PEAK, 2),
+                           "pct_of_hbm_peak": r["config"]["pct_of_hbm_peak"], "weight_gbps": r["config"]["weight_gbps"],
+                           "workload": r["config"]["workload"], "experts_with_rows": r["config"]["experts_with_rows"],
+                           "int8_ops_per_chunk": r["config"]["int8_ops_per_step"],
+                           "algorithmic_bytes_per_chunk": r["config"]["algorithmic_bytes_per_step"], "roofline": r["roofline"]}
     print(json.dumps(line))
+    if not ok:
+        print("bench.py: parity failed: ids exact %s, relative L2 %s against the CPU path (bar %g)" % (
+            line["parity_ids_exact"], line["parity_rel_l2_vs_cpu_path"], PARITY_BAR), file=sys.stderr)
+        sys.exit(3)
 
 
 if __name__ == "__main__":

@@ -105,6 +105,8 @@ typedef struct maya_moe_args {
     float* part;               /* [n_tokens*k][n_embd] each entry's down output (NULL in the fused 1-token form) */
     const float* add;          /* NULL or [n_tokens][n_embd] added to the combined output (shared expert, CPU lane part) */
     const int32_t* add_flag;   /* NULL or a device flag: `add` is added only when it is non-zero */
+    const float* add2;         /* NULL or [n_tokens][n_embd] added after `add`, always (glmf::moe_down's sh_out beside its
+                                * flagged cpu_part, include/strata/kernels/glm_fast.hpp:499-501) */
     float* out;                /* [n_tokens][n_embd] */
 } maya_moe_args;
 
@@ -388,8 +390,9 @@ typedef struct maya_exl3_args {
     float* h;           /* [n_tokens*k][n_ff] */
     float* part;        /* [n_tokens*k][n_embd]: down's per-entry outputs; given to maya_exl3_gate_up it also serves as
                          * scratch for gate/up's partial outputs (the faster, split form); NULL there: the fused form */
-    const float* add;   /* NULL or [n_tokens][n_embd] (shared expert / CPU lane part) */
+    const float* add;   /* NULL or [n_tokens][n_embd] (the CPU lane's part: exl3::MoeArgs::cpu_part / cpu_flag) */
     const int32_t* add_flag;
+    const float* add2;  /* NULL or [n_tokens][n_embd] added after `add`, always (exl3::moe_down's sh_out) */
     float* out;         /* [n_tokens][n_embd] */
 } maya_exl3_args;
 

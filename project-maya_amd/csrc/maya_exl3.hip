@@ -481,6 +481,7 @@ __global__ __launch_bounds__(256) void exl3_combine_kernel(maya_exl3_args a) {
         first = false;
     }
     if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[(size_t) t * n + c]);
+    if (a.add2) sum = __fadd_rn(sum, a.add2[(size_t) t * n + c]);
     a.out[(size_t) t * n + c] = sum;
 }
 

@@ -204,6 +204,7 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
         }
         const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
         if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
+        if (a.add2) sum = __fadd_rn(sum, a.add2[o]);
         a.out[o] = sum;
         if (a.part)
             for (int i = 0; i < a.k; ++i)

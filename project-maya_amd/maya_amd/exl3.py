@@ -21,7 +21,7 @@ class Exl3Args(C.Structure):
                 ("plan_w", C.c_void_p), ("grp_ptr", C.c_void_p), ("grp_start", C.c_void_p), ("grp_ent", C.c_void_p),
                 ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", C.c_void_p),
                 ("x_stride", C.c_int64), ("h", C.c_void_p), ("part", C.c_void_p), ("add", C.c_void_p),
-                ("add_flag", C.c_void_p), ("out", C.c_void_p)]
+                ("add_flag", C.c_void_p), ("add2", C.c_void_p), ("out", C.c_void_p)]
 
 
 EXPORTS = ["maya_exl3_supported", "maya_exl3_trellis_bytes", "maya_exl3_reconstruct_inner", "maya_exl3_gate_up",

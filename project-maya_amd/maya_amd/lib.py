@@ -60,7 +60,8 @@ class Args(C.Structure):
     _fields_ = [("layout", Layout), ("n_tokens", C.c_int32), ("k", C.c_int32), ("plan_ptr", C.c_void_p),
                 ("plan_w", C.c_void_p), ("grp_ptr", C.c_void_p), ("grp_start", C.c_void_p), ("grp_ent", C.c_void_p),
                 ("n_groups", C.c_void_p), ("skip", C.c_void_p), ("limit", C.c_float), ("x", Act), ("h", C.c_void_p),
-                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("out", C.c_void_p)]
+                ("hq", Act), ("part", C.c_void_p), ("add", C.c_void_p), ("add_flag", C.c_void_p), ("add2", C.c_void_p),
+                ("out", C.c_void_p)]
 
 
 class MvJob(C.Structure):

@@ -320,6 +320,51 @@ def test_down_rounds_h_itself_like_the_quantizer(lib, dt):
     assert np.abs(outs[0]).max() > 0
 
 
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,k,nt,packing", ((22, 22, 4096, 2048, 4, 1, 1), (12, 12, 1024, 512, 3, 2, 0), (8, 8, 4096, 2048, 2, 3, 1)))
+def test_down_adds_the_flagged_part_and_then_the_unconditional_one(lib, gt, dt, n_embd, n_ff, k, nt, packing):
+    """out = sum_i w_i part_i [+ add when *add_flag] + add2: the order of glmf::moe_down's cpu_part and sh_out
+    (include/strata/kernels/glm_fast.hpp:499-501), each sum rounded."""
+    import ctypes as C
+    L = lib.load()
+    ne = k + 1
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 41)
+    gguf, _ = lib.layout(gt, dt, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf if packing else None)
+    rng = np.random.default_rng(42)
+    h = dev(rng.standard_normal((nt * k, n_ff)).astype(np.float32))
+    hq = lib.quant_act(dt, h)
+    ids = torch.from_numpy(np.stack([rng.permutation(ne)[:k] for _ in range(nt)]).astype(np.int32)).cuda()
+    plan = lib.plan(ids.view(-1), store.table)
+    w = dev(rng.uniform(0.05, 0.3, nt * k).astype(np.float32))
+    add = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    add2 = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    outs = {}
+    for name, flag, second in (("plain", None, False), ("off", 0, False), ("on", 1, False), ("both", 1, True), ("second", None, True)):
+        a = lib.Args()
+        a.layout = lib.copy_layout(gguf, packing)
+        a.n_tokens, a.k = nt, k
+        a.plan_ptr, a.plan_w = plan.data_ptr(), w.data_ptr()
+        a.limit = float("inf")
+        a.h = h.data_ptr()
+        a.hq = hq.c()
+        part = torch.zeros((nt * k, n_embd), device="cuda")
+        out = torch.zeros((nt, n_embd), device="cuda")
+        a.part, a.out = part.data_ptr(), out.data_ptr()
+        fl = None
+        if flag is not None:
+            fl = torch.tensor([flag], dtype=torch.int32, device="cuda")
+            a.add, a.add_flag = add.data_ptr(), fl.data_ptr()
+        if second:
+            a.add2 = add2.data_ptr()
+        lib.check(L.maya_moe_down(C.byref(a), lib._stream()))
+        torch.cuda.synchronize()
+        outs[name] = out.clone()
+    assert torch.equal(outs["off"], outs["plain"]) and float(outs["plain"].abs().max()) > 0
+    assert torch.equal(outs["on"], outs["plain"] + add)
+    assert torch.equal(outs["both"], (outs["plain"] + add) + add2)
+    assert torch.equal(outs["second"], outs["plain"] + add2)
+
+
 def test_layers_take_tokens_that_are_already_routed(lib, oracle):
     """logits NULL: ids / weights are inputs.  The sigmoid router's ids and weights through the decode layer, the prompt-chunk
     layer and (in test_gpu_exl3) the EXL3 layer give what the routed layer gives."""
