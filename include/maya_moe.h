@@ -298,6 +298,19 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
                                  float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* The same layer for callers that cannot allocate or own a workspace (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the workspace is a file-scope device array of MAYA_STATIC_SCRATCH_BYTES inside the
+ * library, one copy a device, held until the process ends.  No counterpart in the reference (its callers own every buffer,
+ * include/strata/kernels/s2_expert_grouped.hpp:36-38).  The call allocates nothing and sets nothing up: maya_init() must
+ * have run on the current device (it fails with MAYA_E_ARG otherwise); a call whose maya_moe_workspace_bytes exceeds
+ * MAYA_STATIC_SCRATCH_BYTES fails with MAYA_E_SHAPE and launches nothing (7168 x 2048, k 8: up to 3 tokens).  Every call on a
+ * device shares that device's array: calls that overlap on one device (two streams, two threads) race; calls ordered on
+ * one stream do not, and nothing has to be cleared between them (every region is written before it is read). */
+#define MAYA_STATIC_SCRATCH_BYTES (1u << 20)
+int maya_moe_layer_decode_static(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                                 const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
+                                 float limit, const float* add, int32_t* ids, float* weights, float* out, void* stream);
+
 /* ============================================================================================= prefill
  * A prompt chunk's routed experts as a grouped GEMM (the reference's expert_count_kernel / expert_scatter_kernel,
  * src/kernels/cuda/glm_batch.cu:2102-2133, with the host's prefix sum of src/prefill/glm_prefill.cu:3339-3361 done on

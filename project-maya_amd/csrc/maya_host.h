@@ -31,6 +31,7 @@ struct DeviceState {
     Codebooks cb{};
     int lds_limit = 65536;
     int n_cu = 0;
+    void* static_scratch = nullptr;   // this device's copy of the file-scope scratch array (maya_moe_layer_decode_static)
 };
 // the current device's state, initialised on first use (gfx950 only); MAYA_OK or a status
 int current_state(DeviceState** out);

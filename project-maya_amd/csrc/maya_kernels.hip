@@ -41,6 +41,11 @@ constexpr int kMaxDevices = 16;
 DeviceState g_dev[kMaxDevices];
 std::mutex g_init_mu;
 
+// The scratch of maya_moe_layer_decode_static, the layer call for callers that cannot allocate: a file-scope device array
+// in place of the caller's workspace.  Every device the library runs on holds its own copy until the process ends; in host
+// code the name is only a handle for hipGetSymbolAddress (done once a device in current_state), never an address to pass on.
+static __device__ __align__(256) unsigned char scratch[MAYA_STATIC_SCRATCH_BYTES];
+
 int current_state(DeviceState** out) {
     int dev = 0;
     MAYA_HIP(hipGetDevice(&dev));
@@ -70,6 +75,10 @@ int current_state(DeviceState** out) {
             if (e == hipSuccess) e = hipMemcpy(d, host, sizeof(uint64_t) * (1024 + 2048), hipMemcpyHostToDevice);
             delete[] host;
             if (e != hipSuccess) return hip_fail(e, "codebook upload");
+            void* sp = nullptr;
+            e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));   // (this device is the current one)
+            if (e != hipSuccess || sp == nullptr) return hip_fail(e == hipSuccess ? hipErrorInvalidSymbol : e, "address of the static scratch");
+            s.static_scratch = sp;
             s.cb.iq2s = d;
             s.cb.iq1s = d + 1024;
             s.lds_limit = (int) p.sharedMemPerBlock;
@@ -2207,6 +2216,24 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
         if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
     }
     return maya_moe_down(&a, stream);
+}
+
+int maya_moe_layer_decode_static(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                                 const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                                 int32_t* ids, float* weights, float* out, void* stream) {
+    // No lazy set-up here: the first use of a device uploads the codebooks (an allocation and a synchronous copy), which
+    // this entry point must not do - maya_init() does, once, outside any capture.
+    int dev = 0;
+    MAYA_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices || !g_dev[dev].ready || !g_dev[dev].static_scratch)
+        return fail(MAYA_E_ARG, "layer_decode_static: call maya_init() on device %d first (this entry point sets nothing up)", dev);
+    const size_t need = maya_moe_workspace_bytes(l, n_tokens, k);
+    if (need == 0) return fail(MAYA_E_SHAPE, "layer_decode_static: layout, n_tokens %d or k %d not covered", n_tokens, k);
+    if (need > (size_t) MAYA_STATIC_SCRATCH_BYTES)
+        return fail(MAYA_E_SHAPE, "layer_decode_static: this call needs %zu bytes of scratch, the static buffer holds %zu (use maya_moe_layer_decode_routed with a workspace)",
+                    need, (size_t) MAYA_STATIC_SCRATCH_BYTES);
+    return maya_moe_layer_decode_routed(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out,
+                                        g_dev[dev].static_scratch, (size_t) MAYA_STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

@@ -20,7 +20,7 @@ EXPORTS = [
     "maya_moe_workspace_bytes", "maya_moe_layer_decode", "maya_moe_repack", "maya_moe_unpack", "maya_moe_pack_experts",
     "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
     "maya_moe_tab_update",
-    "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv",
+    "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv", "maya_moe_layer_decode_static",
 ]
 
 
