@@ -409,6 +409,21 @@ typedef struct maya_exl3_args {
     float* out;         /* [n_tokens][n_embd] */
 } maya_exl3_args;
 
+/* Offsets of the nine pieces of an expert blob (suh, svh, trellis of gate, up and down) for n_embd x n_ff experts at k2[3]
+ * (gate, up, down) and codebook cb; returns the blob's bytes (0: a shape or bitrate the kernels do not take).
+ * MAYA_EXL3_ORDER_SCALES_FIRST: a part is [suh | svh | trellis], every piece on a 16-byte boundary - the order of the reference
+ * test's blobs (tests/exl3_test.cu:415-439).  MAYA_EXL3_ORDER_TRELLIS_FIRST: a part is [trellis | suh | svh], every piece a
+ * multiple of 256 bytes - the blob the engine assembles from a pack (tools/exl3_pack.py:315-349). */
+#define MAYA_EXL3_ORDER_SCALES_FIRST 0
+#define MAYA_EXL3_ORDER_TRELLIS_FIRST 1
+size_t maya_exl3_layout_init(maya_exl3_layout* l, int n_embd, int n_ff, const int32_t* k2, int cb, int order);
+/* A layer's expert blobs assembled on the device from the experts' pieces where the model's files keep them, as the engine
+ * assembles them from exl3.txt's rows (tools/exl3_pack.py:315-349, 596-612: per expert and part a trellis, a suh and an svh
+ * range of a safetensors file): pieces[9 e + 3 r + {0, 1, 2}] = the address (device memory, or host memory mapped to the
+ * device) of expert e's part r's trellis / suh / svh, 0 = leave that piece alone; blob e at dst + e * dst_stride gets each
+ * piece at its offset in `l` (sizes from l's shape and bitrates). */
+int maya_exl3_pack_experts(const maya_exl3_layout* l, const uint64_t* pieces, int n_expert, void* dst, size_t dst_stride,
+                           void* stream);
 /* exl3::k2_supported (include/strata/kernels/exl3.hpp:56-58) */
 int maya_exl3_supported(int k2, int cb);
 /* bytes of a k x n trellis at k2: exl3::trellis_bytes_k2 (exl3.hpp:50-52) */

@@ -614,7 +614,79 @@ using namespace maya;
 extern "C" {
 
 int maya_exl3_supported(int k2, int cb) { return exl3_k2_ok(k2, cb) ? 1 : 0; }
+
+size_t maya_exl3_layout_init(maya_exl3_layout* l, int n_embd, int n_ff, const int32_t* k2, int cb, int order) {
+    if (!l || !k2 || n_embd <= 0 || n_ff <= 0 || n_embd % 128 || n_ff % 128 || (order != MAYA_EXL3_ORDER_SCALES_FIRST && order != MAYA_EXL3_ORDER_TRELLIS_FIRST))
+        return 0;
+    for (int r = 0; r < 3; ++r)
+        if (!exl3_k2_ok(k2[r], cb)) return 0;
+    *l = maya_exl3_layout{};
+    l->cb = cb;
+    l->n_embd = n_embd;
+    l->n_ff = n_ff;
+    // every piece starts on a multiple of `al` bytes: 16 for the compact order, 256 for the engine's assembled blobs
+    const size_t al = order == MAYA_EXL3_ORDER_TRELLIS_FIRST ? 256 : 16;
+    auto up = [al](size_t n) { return (n + al - 1) / al * al; };
+    size_t off = 0;
+    for (int r = 0; r < 3; ++r) {
+        const int64_t k = r == 2 ? n_ff : n_embd, n = r == 2 ? n_embd : n_ff;
+        const size_t tb = maya_exl3_trellis_bytes(k, n, k2[r]);
+        l->k2[r] = k2[r];
+        if (order == MAYA_EXL3_ORDER_TRELLIS_FIRST) {
+            l->trellis[r] = off, off += up(tb);
+            l->suh[r] = off, off += up(2 * (size_t) k);
+            l->svh[r] = off, off += up(2 * (size_t) n);
+        } else {
+            l->suh[r] = off, off += up(2 * (size_t) k);
+            l->svh[r] = off, off += up(2 * (size_t) n);
+            l->trellis[r] = off, off += up(tb);
+        }
+    }
+    return off;
+}
 size_t maya_exl3_trellis_bytes(int64_t k, int64_t n, int k2) { return (size_t) (k / 16) * (size_t) (n / 16) * 16u * (size_t) k2; }
+
+// nine pieces an expert (the trellis, suh and svh of gate, up and down) copied to their places in the expert's blob:
+// grid (blocks, 9, n_expert).  16 bytes a thread where source and destination allow it, else byte by byte.
+__global__ __launch_bounds__(256) void exl3_pack_kernel(const uint64_t* __restrict__ pieces, maya_exl3_layout l, uint8_t* __restrict__ dst,
+                                                        size_t dst_stride) {
+    const int piece = blockIdx.y, r = piece / 3, what = piece % 3, e = blockIdx.z;
+    const int64_t k = r == 2 ? l.n_ff : l.n_embd, n = r == 2 ? l.n_embd : l.n_ff;
+    const size_t bytes = what == 0 ? (size_t) (k / 16) * (size_t) (n / 16) * 16u * (size_t) l.k2[r] : what == 1 ? 2 * (size_t) k : 2 * (size_t) n;
+    const size_t off = what == 0 ? l.trellis[r] : what == 1 ? l.suh[r] : l.svh[r];
+    const uint8_t* src = (const uint8_t*) pieces[(size_t) e * 9 + piece];
+    uint8_t* d = dst + (size_t) e * dst_stride + off;
+    if (src == nullptr) return;
+    const size_t stride = (size_t) gridDim.x * 256;
+    if ((((uintptr_t) src | (uintptr_t) d) & 15) == 0) {
+        const size_t n16 = bytes >> 4;
+        for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) ((uint4*) d)[i] = ((const uint4*) src)[i];
+        for (size_t i = (n16 << 4) + (size_t) blockIdx.x * 256 + threadIdx.x; i < bytes; i += stride) d[i] = src[i];
+    } else {
+        for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < bytes; i += stride) d[i] = src[i];
+    }
+}
+
+int maya_exl3_pack_experts(const maya_exl3_layout* l, const uint64_t* pieces, int n_expert, void* dst, size_t dst_stride, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l || !pieces || !dst) return fail(MAYA_E_ARG, "exl3_pack_experts: null pointer");
+    if (n_expert <= 0 || n_expert > 65535) return fail(MAYA_E_SHAPE, "exl3_pack_experts: %d experts", n_expert);
+    if (l->n_embd <= 0 || l->n_ff <= 0 || l->n_embd % 128 || l->n_ff % 128) return fail(MAYA_E_SHAPE, "exl3_pack_experts: %d x %d", l->n_embd, l->n_ff);
+    size_t end = 0;
+    for (int r = 0; r < 3; ++r) {
+        if (!exl3_k2_ok(l->k2[r], l->cb)) return fail(MAYA_E_UNSUPPORTED, "exl3_pack_experts: k2 %d with codebook %d", l->k2[r], l->cb);
+        const int64_t k = r == 2 ? l->n_ff : l->n_embd, n = r == 2 ? l->n_embd : l->n_ff;
+        if ((l->trellis[r] & 3) || (l->suh[r] & 1) || (l->svh[r] & 1)) return fail(MAYA_E_ARG, "exl3_pack_experts: a trellis needs 4-byte, suh / svh 2-byte alignment");
+        end = end > l->trellis[r] + maya_exl3_trellis_bytes(k, n, l->k2[r]) ? end : l->trellis[r] + maya_exl3_trellis_bytes(k, n, l->k2[r]);
+        end = end > l->suh[r] + 2 * (size_t) k ? end : l->suh[r] + 2 * (size_t) k;
+        end = end > l->svh[r] + 2 * (size_t) n ? end : l->svh[r] + 2 * (size_t) n;
+    }
+    if (dst_stride < end) return fail(MAYA_E_ARG, "exl3_pack_experts: blobs of %zu bytes do not fit a stride of %zu", end, dst_stride);
+    hipLaunchKernelGGL(exl3_pack_kernel, dim3(64, 9, (unsigned) n_expert), dim3(256), 0, as_stream(stream), pieces, *l, (uint8_t*) dst, dst_stride);
+    MAYA_LAUNCHED("exl3_pack_kernel");
+    return MAYA_OK;
+}
 
 int maya_exl3_reconstruct_inner(const uint32_t* trellis, int64_t k, int64_t n, int k2, int cb, uint16_t* dst, void* stream) {
     DeviceState* st;

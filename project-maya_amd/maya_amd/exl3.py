@@ -25,7 +25,9 @@ class Exl3Args(C.Structure):
 
 
 EXPORTS = ["maya_exl3_supported", "maya_exl3_trellis_bytes", "maya_exl3_reconstruct_inner", "maya_exl3_gate_up",
-           "maya_exl3_down", "maya_exl3_workspace_bytes", "maya_exl3_layer_decode"]
+           "maya_exl3_down", "maya_exl3_workspace_bytes", "maya_exl3_layer_decode", "maya_exl3_layout_init",
+           "maya_exl3_pack_experts"]
+ORDER_SCALES_FIRST, ORDER_TRELLIS_FIRST = 0, 1
 
 _bound = False
 
@@ -43,6 +45,9 @@ def load():
         lib.maya_exl3_down.argtypes = [C.POINTER(Exl3Args), vp]
         lib.maya_exl3_workspace_bytes.restype = sz
         lib.maya_exl3_workspace_bytes.argtypes = [C.POINTER(Exl3Layout), i32, i32]
+        lib.maya_exl3_layout_init.restype = sz
+        lib.maya_exl3_layout_init.argtypes = [C.POINTER(Exl3Layout), i32, i32, C.POINTER(C.c_int32), i32, i32]
+        lib.maya_exl3_pack_experts.argtypes = [C.POINTER(Exl3Layout), vp, i32, vp, sz, vp]
         lib.maya_exl3_layer_decode.argtypes = [C.POINTER(Exl3Layout), vp, i32, i32, vp, vp, i32, f32, vp, vp, vp, vp, vp, sz, vp]
         _bound = True
     return lib
@@ -71,6 +76,23 @@ def make_layout(n_embd, n_ff, k2, cb):
         l.trellis[r] = off
         off += ((k // 16) * (n // 16) * 16 * k2[r] + 15) & ~15
     return l, off
+
+
+def layout_init(n_embd, n_ff, k2, cb, order=ORDER_SCALES_FIRST):
+    """(Exl3Layout, blob bytes) from the library (maya_exl3_layout_init); order: ORDER_SCALES_FIRST ([suh | svh | trellis], 16-byte
+    pieces: what make_layout gives) or ORDER_TRELLIS_FIRST ([trellis | suh | svh], 256-byte pieces: the engine's assembled blob)."""
+    k2 = [k2] * 3 if isinstance(k2, int) else list(k2)
+    l = Exl3Layout()
+    n = int(load().maya_exl3_layout_init(C.byref(l), n_embd, n_ff, (C.c_int32 * 3)(*k2), cb, order))
+    if n == 0:
+        raise L.MayaError(2, "maya_exl3_layout_init: %d x %d at k2 %s with codebook %d is not covered" % (n_embd, n_ff, k2, cb))
+    return l, n
+
+
+def pack_experts(l, pieces, n_expert, dst, dst_stride, stream=None):
+    """pieces: int64 device tensor [n_expert, 9] of addresses (trellis, suh, svh of gate, up, down); dst: uint8 device tensor."""
+    assert pieces.dtype == torch.int64 and pieces.numel() == 9 * n_expert and pieces.is_contiguous()
+    L.check(load().maya_exl3_pack_experts(C.byref(l), L._p(pieces), n_expert, L._p(dst), dst_stride, L._stream(stream)))
 
 
 def matrix_of(l, role):
