@@ -1,4 +1,5 @@
-"""Compiles the HIP sources into project-maya_amd/libmaya_moe.so for gfx950 (hipcc cross-compiles without a GPU)."""
+"""Compiles the HIP sources into project-maya_amd/libmaya_moe.so for gfx950 (hipcc cross-compiles without a GPU), and the
+stand-alone microbenchmark program project-maya_amd/maya_probe beside it."""
 import os
 import subprocess
 import sys
@@ -6,21 +7,26 @@ import sys
 PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmaya_moe.so")
+PROBE = os.path.join(PKG, "maya_probe")
 SOURCES = ["maya_kernels.hip", "maya_exl3.hip", "maya_prefill.hip"]
 # -packed-fp32-ops off: the compiler then forms no v_pk_*_f32 from scalar float code
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 
 
-def build(verbose=False):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+def _run(cmd, verbose):
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + err)
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose=False):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _run([hipcc] + FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES], verbose)
+    _run([hipcc] + [f for f in FLAGS if f not in ("-shared", "-fPIC")] + ["-o", PROBE, os.path.join(CSRC, "maya_probe.hip")], verbose)
     return LIB
 
 
