@@ -337,7 +337,8 @@ typedef struct maya_prefill_plan {
 typedef struct maya_prefill_act {
     int8_t* q; /* [rows][k], 16-byte aligned */
     float* d;  /* [rows][k / 256] */
-    float* s;  /* [rows][k / 32], 16-byte aligned */
+    uint16_t* s; /* [rows][k / 256][16] FP16, 16-byte aligned: a block's 8 sub-block code sums as two digits, sum = lo + 64 hi:
+                  * the 8 lo (0..63), then the 8 hi (-64..63) */
 } maya_prefill_act;
 
 int maya_moe_prefill_tile_rows(void);

@@ -347,7 +347,7 @@ def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=
     """A prompt chunk's routed experts as the reference's CPU expert path computes each of them (Q8_K rows of x, the
     gate / up row dots, the clamped SwiGLU, h rounded to Q8_K, the down row dots: src/kernels/cpu/native_expert.cpp:306-442)
     in the plan's row order (src/kernels/cuda/glm_batch.cu:2102-2133), and the weighted sum in slot order.  Returns a dict
-    of every stage: xq / xd / xs = the rows' codes, block scales and d * (sum of every 32 codes); h = the SwiGLU values."""
+    of every stage: xq / xd / xs = the rows' codes, block scales and the integer sum of every 32 codes; h = the SwiGLU values."""
     tg, td = t if isinstance(t, tuple) else (t, t)   # (gate/up type, down type)
     ids, w = router_topk(logits, k)
     ne = len(blobs)
@@ -356,7 +356,7 @@ def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=
     lim = float(limit) if limit and limit > 0 else float("inf")
     xq = np.zeros((rows, n_embd), dtype=np.int8)
     xd = np.zeros((rows, n_embd // 256), dtype=np.float32)
-    xs = np.zeros((rows, n_embd // 32), dtype=np.float32)
+    xs = np.zeros((rows, n_embd // 32), dtype=np.int32)
     h = np.zeros((rows, n_ff), dtype=np.float32)
     part = np.zeros((rows, n_embd), dtype=np.float32)
     acts = {}
@@ -366,7 +366,7 @@ def prefill_layer(t, blobs, up_off, down_off, n_embd, n_ff, logits, x, k, limit=
         if tok not in acts:
             a = quant_act(tg, x[tok])
             d, q, bs = q8k_fields(a)
-            acts[tok] = (a, q, d, (d[:, None] * (bs[:, 0::2] + bs[:, 1::2]).astype(np.float32)).reshape(-1))
+            acts[tok] = (a, q, d, (bs[:, 0::2].astype(np.int32) + bs[:, 1::2]).reshape(-1))
         a, xq[r], xd[r], xs[r] = acts[tok]
         b = blobs[e]
         g = rows_of(tg, b, n_embd, n_ff, a)

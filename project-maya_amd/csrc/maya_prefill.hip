@@ -157,11 +157,14 @@ __device__ __forceinline__ int pf_rint(float f) { return (int) rintf(f); }
 // Q8_K rows - the activation format of the reference's CPU expert path for the K-quants
 // (src/kernels/cuda/quantize_act.cu:161-207) - rounded 32 values a lane, 8 lanes a 256-value block (q8k_round_lane32: no
 // LDS, no barrier): the block's signed maximum is the value at the FIRST largest magnitude, iscale = -127 / max,
-// c = min(127, nearest_int(iscale x)), d = 1 / iscale; s = d * (the sum of each 32 codes), what the minimums of a Q4_K
-// sub-block multiply.
+// c = min(127, nearest_int(iscale x)), d = 1 / iscale; s = the sum of each 32 codes - what the minimums of a Q4_K
+// sub-block multiply - as two FP16 digits, sum = lo + 64 hi with lo in 0..63: both are exact in FP16, and so is every
+// product with a 6-bit minimum (times 64 for the high digit), which lets an FP16 matrix instruction form the integer
+// sum over a block's 8 sub-blocks exactly.
 struct PfLane {
     int y[8];      // 32 codes
-    float d, ds;
+    float d;
+    int sum;
 };
 template <int DT>
 __device__ __forceinline__ void pf_load32(const void* x, int64_t i0, bool on, float (&v)[32]) {
@@ -210,7 +213,7 @@ __device__ __forceinline__ PfLane pf_round_lane(const float (&v)[32], int lane) 
     int sum = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) sum = dot4(0x01010101, o.y[i], sum);
-    o.ds = __fmul_rn(o.d, (float) sum);
+    o.sum = sum;
     return o;
 }
 __device__ __forceinline__ void pf_store_lane(const maya_prefill_act& o, size_t row, int64_t k, int64_t v0, int lane, const PfLane& c) {
@@ -218,7 +221,10 @@ __device__ __forceinline__ void pf_store_lane(const maya_prefill_act& o, size_t 
     int4* q = (int4*) (o.q + at);
     q[0] = make_int4(c.y[0], c.y[1], c.y[2], c.y[3]);
     q[1] = make_int4(c.y[4], c.y[5], c.y[6], c.y[7]);
-    o.s[at >> 5] = c.ds;
+    // (a block's 16 halves: the low digits of its 8 sub-blocks, then the high digits)
+    _Float16* sp = (_Float16*) o.s + (at >> 8) * 16 + (lane & 7);
+    sp[0] = (_Float16) (float) (c.sum & 63);
+    sp[8] = (_Float16) (float) (c.sum >> 6);
     if ((lane & 7) == 0) o.d[at >> 8] = c.d;
 }
 
@@ -290,7 +296,7 @@ struct PfDma {
         wave = wave_;
         const int last = nrows - 1;
         rq = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.q + (size_t) row0 * a.k), 0, (int) (nrows * a.k), 0x00020000);
-        rs = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.s + (size_t) row0 * (a.k >> 5)), 0, (int) (nrows * (a.k >> 5) * 4), 0x00020000);
+        rs = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.s + (size_t) row0 * (a.k >> 4)), 0, (int) (nrows * (a.k >> 5) * 4), 0x00020000);
         rd = __builtin_amdgcn_make_buffer_rsrc((void*) (a.x.d + (size_t) row0 * (a.k >> 8)), 0, (int) (nrows * (a.k >> 8) * 4), 0x00020000);
 #pragma unroll
         for (int n = 0; n < NMT; ++n) {
@@ -379,6 +385,15 @@ template <int N, typename T> __device__ __forceinline__ void pf_lds_wait(T (&r)[
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
     }
 }
+// the registers r have landed once at most BUT later LDS reads are outstanding (LDS operations complete in order)
+template <int BUT, int N> __device__ __forceinline__ void pf_lds_wait_but(v4i (&r)[N]) {
+    static_assert(N == 1 || N == 2, "1 or 2 registers");
+    if constexpr (N == 1) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(r[0]) : "n"(BUT));
+    else asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(r[0]), "+v"(r[1]) : "n"(BUT));
+}
+template <int BUT> __device__ __forceinline__ void pf_lds_wait_tail(v4i& a, v4f (&d)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(a), "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3]) : "n"(BUT));
+}
 // (compile-time loops over the row groups of a tile)
 template <int M, int NMT, typename F> __device__ __forceinline__ void pf_for_m(F&& f) {
     if constexpr (M < NMT) {
@@ -387,35 +402,44 @@ template <int M, int NMT, typename F> __device__ __forceinline__ void pf_for_m(F
     }
 }
 
-// one tile of NMT x 16 rows against the wave's two tiles of 16 weight rows (gate/up: the gate and the up rows of 16
-// features)
-template <bool GU, int NMT>
+typedef int pf_v16i __attribute__((ext_vector_type(16)));
+typedef float pf_v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 pf_v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 pf_v2h __attribute__((ext_vector_type(2)));
+
+// One tile of NM x 32 rows against the wave's 32 weight rows (gate/up: the gate rows of 16 features, then their up rows;
+// down: 32 output rows), on the 32x32 matrix instructions: lane (ln = lane & 31, kh = lane >> 5) holds 16 of a
+// sub-block's 32 values of activation row ln (A operand, from LDS) and of weight row ln (B operand, decoded in
+// registers), and 16 outputs: weight row ln against the rows 8 b + 4 kh + r (b, r = 0..3) of the 32.  These
+// instructions take 32 cycles, and the vector ALU issues about four instructions under each of them; the 16-cycle
+// 16x16 forms leave it no slot (measured: project-maya_amd/csrc/maya_probe.hip, section 5), which is what bounds a
+// kernel that has as many vector instructions as this one.
+template <bool GU, int NM>
 __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b1, uint8_t* b2, int ex, int row0, int nrows) {
     // (global address space: a generic pointer's loads would count as LDS operations too, and every wait for them
     // would also wait for the copies into LDS behind them)
     typedef const __attribute__((address_space(1))) uint8_t* wptr;
+    constexpr int NMT = 2 * NM;   // groups of 16 rows: what the copies into LDS count in
     wptr blob = (wptr) a.table[ex];
-    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 31, kh = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    wptr wrow[2];
+    wptr wrow;
     int64_t n0;   // the wave's first feature (gate/up) or output row (down)
     if constexpr (GU) {
         n0 = (int64_t) blockIdx.x * 64 + wave * 16;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) wrow[t] = blob + a.off[t] + (size_t) (n0 + ln) * a.row_bytes;
+        wrow = blob + a.off[ln >> 4] + (size_t) (n0 + (ln & 15)) * a.row_bytes;
     } else {
         n0 = (int64_t) blockIdx.x * 128 + wave * 32;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) wrow[t] = blob + a.off[0] + (size_t) (n0 + 16 * t + ln) * a.row_bytes;
+        wrow = blob + a.off[0] + (size_t) (n0 + ln) * a.row_bytes;
     }
     const bool wave_on = n0 < a.n;   // (a.n is a multiple of the wave's rows: checked on the host)
 
-    v4f acc[2][NMT];
+    pf_v16f acc[NM];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int m = 0; m < NM; ++m)
 #pragma unroll
-        for (int m = 0; m < NMT; ++m) acc[t][m] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int i = 0; i < 16; ++i) acc[m][i] = 0.0f;
 
     const int nsb = (int) (a.k >> 8);
     // The activations run two super-blocks ahead through three LDS buffers, the weights one ahead in registers.  The
@@ -425,134 +449,119 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     dma.init(a, row0, nrows, wave, lane);
     dma.copy(b0, 0);
     if (nsb > 1) dma.copy(b1, 1);
-    // the weights of a super-block - the 16-byte header of each of the lane's two rows and two 16-byte pieces of its
-    // codes: bytes 64 h + 16 g of the row's 128, h = 0, 1 (so the four lanes of a row read 64 bytes in a run)
+    // the weights of a super-block: the 16-byte header of the lane's row and four 16-byte pieces of its codes, bytes
+    // 32 c + 16 kh of the row's 128 (c = 0..3): the low nibbles are 16 values of sub-block 2 c, the high ones of 2 c + 1
     typedef uint32_t w4 __attribute__((ext_vector_type(4)));
-    w4 q[2][2], qn[2][2];           // [piece h][row tile]
-    uint32_t hdr[2][4], hdrn[2][4];
-    auto load_block = [&](int sb, w4 (&dq)[2][2], uint32_t (&dh)[2][4]) {
+    w4 q[4], qn[4], hdr, hdrn;
+    auto load_block = [&](int sb, w4 (&dq)[4], w4& dh) {
+        wptr blk = wrow + (size_t) sb * 144;
+        dh = *(const __attribute__((address_space(1))) w4*) blk;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            wptr blk = wrow[t] + (size_t) sb * 144;
-            const w4 h = *(const __attribute__((address_space(1))) w4*) blk;
-            dh[t][0] = h.x, dh[t][1] = h.y, dh[t][2] = h.z, dh[t][3] = h.w;
-#pragma unroll
-            for (int j = 0; j < 2; ++j) dq[j][t] = *(const __attribute__((address_space(1))) w4*) (blk + 16 + 64 * j + 16 * g);
-        }
+        for (int c = 0; c < 4; ++c) dq[c] = *(const __attribute__((address_space(1))) w4*) (blk + 16 + 32 * c + 16 * kh);
     };
     if (wave_on) load_block(0, q, hdr);
-    // a lane's 16 codes of a matrix instruction: values 16 (g & 1) .. + 15 of sub-block 4 h + 2 (g >> 1) + n = the row's
-    // 16-byte chunk 8 h + 2 n + 4 (g >> 1) + (g & 1), which sits at that index ^ the row
-    const int a_base = ln * 256, a_swz = (ln ^ (4 * (g >> 1) + (g & 1))) << 4;
+    // a lane's 16 codes of sub-block j: the row's 16-byte chunk 2 j + kh, which sits at that index ^ (the row & 15)
+    const int a_base = ln * 256, a_swz = ((ln & 15) ^ kh) << 4;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     auto step = [&](int sb, const uint8_t* buf, uint8_t* buf2) {   // super-block sb from buf; sb + 2 is copied into buf2
-        float d[2], dmin[2];
-        uint32_t sc[2][2], mn[2][2];
+        float d = 0.0f, ndmin = 0.0f;
+        uint32_t sc[2], mn[2];
         if (wave_on) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                d[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] & 0xffffu));
-                dmin[t] = f16_bits_to_f32((uint16_t) (hdr[t][0] >> 16));
-                q4k_unpack_scales(hdr[t][1], hdr[t][2], hdr[t][3], sc[t], mn[t]);
-            }
+            d = f16_bits_to_f32((uint16_t) (hdr.x & 0xffffu));
+            ndmin = -f16_bits_to_f32((uint16_t) (hdr.x >> 16));
+            q4k_unpack_scales(hdr.y, hdr.z, hdr.w, sc, mn);
             if (sb + 1 < nsb) load_block(sb + 1, qn, hdrn);
         }
         // (after the weights' loads, so that waiting for everything but these copies covers the weights too)
         if (sb + 2 < nsb) dma.copy(buf2, sb + 2);
         if (wave_on) {
-            // the minimums' term, -(dmin m) . s over the 8 sub-blocks, on the matrix cores in F32: A = the tokens' s
-            // (row = token, k = sub-block), B = this lane's row's -dmin m, accumulated straight into acc
             const uint32_t lbuf = pf_lds_addr(buf);
-            {
-                float sa[2 * NMT];
-                const uint32_t at = lbuf + kPfSOff + ln * 32 + g * 4;
-                pf_for_m<0, NMT>([&](auto mc) {
+            // The two plane products of the block, int32: [m][0] = (q lo) . c, [1] = (q hi) . c, a matrix instruction a
+            // sub-block and plane, accumulated over the 8 sub-blocks.  The activation operand of sub-block jj + 1 is
+            // requested from LDS before the arithmetic of sub-block jj, and the operands of the block's closing stage
+            // (the code sums, the block scales) before the last sub-block: a read issued just ahead of its use leaves
+            // the wave waiting for LDS eight times a step.
+            pf_v16i dot[NM][2];
+            v4i xr[2][NM];
+            auto read_x = [&](int jj, v4i (&dst)[NM]) {
+                const uint32_t at = lbuf + a_base + (a_swz ^ ((2 * jj) << 4));
+                pf_for_m<0, NM>([&](auto mc) {
                     constexpr int m = decltype(mc)::value;
-                    sa[2 * m] = pf_lds_f32<m * 512>(at);
-                    sa[2 * m + 1] = pf_lds_f32<m * 512 + 16>(at);
+                    dst[m] = pf_lds_i32x4<m * 8192>(at);
                 });
-                float nb[2][2];
-#pragma unroll
-                for (int half = 0; half < 2; ++half)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) nb[half][t] = -__fmul_rn(dmin[t], (float) ((mn[t][half] >> (8 * g)) & 0xffu));
-                pf_lds_wait(sa);
-#pragma unroll
-                for (int half = 0; half < 2; ++half)
-#pragma unroll
-                    for (int m = 0; m < NMT; ++m)
-#pragma unroll
-                        for (int t = 0; t < 2; ++t)
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[2 * m + half], nb[half][t], acc[t][m], 0, 0, 0);
-            }
-            // The two plane products of the block, int32: [t][m][0] = (q lo) . c, [1] = (q hi) . c.  One 64-deep matrix
-            // instruction takes the low (n = 0) or the high (n = 1) nibbles of the four lanes' pieces h: two whole
-            // sub-blocks, 4 h + n and 4 h + 2 + n, a lane's 16 operand bytes = 16 values of one of them times that
-            // sub-block's factor; the activations' operand is the same 16 codes (one 16-byte LDS read).
-            v4i dot[2][NMT][2];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                uint32_t s2[2];
-#pragma unroll
-                for (int t = 0; t < 2; ++t) s2[t] = sc[t][h] >> (16 * (g >> 1));   // the scales of sub-blocks 4 h + 2 (g >> 1), + 1
-#pragma unroll
-                for (int n = 0; n < 2; ++n) {
-                    v4i xr[NMT];
-                    {
-                        const uint32_t at = lbuf + a_base + (a_swz ^ ((8 * h + 2 * n) << 4));
-                        pf_for_m<0, NMT>([&](auto mc) {
-                            constexpr int m = decltype(mc)::value;
-                            xr[m] = pf_lds_i32x4<m * 4096>(at);
-                        });
-                    }
-                    v4i wl[2], wh[2];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const uint32_t f = (s2[t] >> (8 * n)) & 0x3fu, flo = f & 7u, fhi = f >> 3;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const uint32_t w = (q[h][t][i] >> (4 * n)) & 0x0f0f0f0fu;
-                            wl[t][i] = (int) pf_scale_codes(w, flo);
-                            wh[t][i] = (int) pf_scale_codes(w, fhi);
-                        }
-                    }
-                    pf_lds_wait(xr);
-#pragma unroll
-                    for (int m = 0; m < NMT; ++m) {
-#pragma unroll
-                        for (int t = 0; t < 2; ++t) {
-                            const v4i z = {0, 0, 0, 0};
-                            dot[t][m][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xr[m], wl[t], (h | n) ? dot[t][m][0] : z, 0, 0, 0);
-                            dot[t][m][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xr[m], wh[t], (h | n) ? dot[t][m][1] : z, 0, 0, 0);
-                        }
-                    }
-                }
-            }
-            // once a block: lo + 8 hi = the block's integer sum (< 2^25), then its two scales
-            v4f dxr[NMT];
-            pf_for_m<0, NMT>([&](auto mc) {
+            };
+            v4i sa[NM];
+            v4f dxr[NM][4];
+            auto read_tail = [&](auto mc) {   // the closing stage's operands of row group m: its code sums and block scales
                 constexpr int m = decltype(mc)::value;
-                dxr[m] = pf_lds_f32x4<kPfDOff + m * 64>(lbuf + 16 * g);
-            });
-            pf_lds_wait(dxr);
+                sa[m] = pf_lds_i32x4<kPfSOff + m * 1024>(lbuf + ln * 32 + kh * 16);
+                const uint32_t at = lbuf + 16 * kh;
+                dxr[m][0] = pf_lds_f32x4<kPfDOff + m * 128>(at);
+                dxr[m][1] = pf_lds_f32x4<kPfDOff + m * 128 + 32>(at);
+                dxr[m][2] = pf_lds_f32x4<kPfDOff + m * 128 + 64>(at);
+                dxr[m][3] = pf_lds_f32x4<kPfDOff + m * 128 + 96>(at);
+            };
+            read_x(0, xr[0]);
 #pragma unroll
-            for (int m = 0; m < NMT; ++m) {
-                const float dx[4] = {dxr[m][0], dxr[m][1], dxr[m][2], dxr[m][3]};
+            for (int jj = 0; jj < 8; ++jj) {
+                const int c = jj >> 1, j = jj & 1;
+                if (jj < 7) read_x(jj + 1, xr[(jj + 1) & 1]);
+                if (jj == 7) read_tail(std::integral_constant<int, 0>{});
+                const uint32_t f = (sc[c >> 1] >> (16 * (c & 1) + 8 * j)) & 0x3fu, flo = f & 7u, fhi = f >> 3;
+                v4i wl, wh;
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t w = (q[c][i] >> (4 * j)) & 0x0f0f0f0fu;
+                    wl[i] = (int) pf_scale_codes(w, flo);
+                    wh[i] = (int) pf_scale_codes(w, fhi);
+                }
+                // this sub-block's operand has landed once only the reads issued after it are outstanding (LDS answers in order)
+                if (jj < 7) pf_lds_wait_but<NM>(xr[jj & 1]);
+                else pf_lds_wait_but<5>(xr[jj & 1]);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        acc[t][m][i] = fmaf(__fmul_rn(dx[i], d[t]), (float) (dot[t][m][0][i] + 8 * dot[t][m][1][i]), acc[t][m][i]);
+                for (int m = 0; m < NM; ++m) {
+                    const pf_v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    dot[m][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xr[jj & 1][m], wl, jj ? dot[m][0] : z, 0, 0, 0);
+                    dot[m][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(xr[jj & 1][m], wh, jj ? dot[m][1] : z, 0, 0, 0);
                 }
             }
-            if (sb + 1 < nsb) {
+            // The minimums' integer term sum_j m_j (sum of sub-block j's codes), exactly, from one FP16 matrix instruction:
+            // k = 0..7 pairs m_j with the sums' low digits, k = 8..15 pairs 64 m_j with their high digits (every operand
+            // and every partial sum an integer below 2^24).
+            pf_v8h mb;
+            {
+                const float mul = kh ? 64.0f : 1.0f;
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int w = 0; w < 2; ++w)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) hdr[t][i] = hdrn[t][i];
-                    q[0][t] = qn[0][t], q[1][t] = qn[1][t];
+                    for (int i = 0; i < 2; ++i) {
+                        const pf_v2h t = __builtin_bit_cast(pf_v2h, __builtin_amdgcn_cvt_pkrtz(__fmul_rn((float) ((mn[w] >> (16 * i)) & 0xffu), mul),
+                                                                                              __fmul_rn((float) ((mn[w] >> (16 * i + 8)) & 0xffu), mul)));
+                        mb[4 * w + 2 * i] = t[0], mb[4 * w + 2 * i + 1] = t[1];
+                    }
+            }
+            // once a block: lo + 8 hi = the block's integer sum (< 2^25), then d_x (d_w sum - dmin_w minimums)
+            pf_for_m<0, NM>([&](auto mc) {
+                constexpr int m = decltype(mc)::value;
+                if constexpr (m + 1 < NM) {
+                    read_tail(std::integral_constant<int, m + 1>{});
+                    pf_lds_wait_tail<5>(sa[m], dxr[m]);
+                } else {
+                    pf_lds_wait_tail<0>(sa[m], dxr[m]);
                 }
+                const pf_v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const pf_v16f mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_v8h, sa[m]), mb, z, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float t = fmaf(ndmin, mins[i], __fmul_rn(d, (float) (dot[m][0][i] + 8 * dot[m][1][i])));
+                    acc[m][i] = fmaf(dxr[m][i >> 2][i & 3], t, acc[m][i]);
+                }
+            });
+            if (sb + 1 < nsb) {
+                hdr = hdrn;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) q[c] = qn[c];
             }
         }
         // super-block sb + 1 has landed once only this iteration's copies (of sb + 2) may still be in flight
@@ -566,16 +575,19 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
     }
     if (!wave_on) return;
 
-    // outputs: lane (ln, g) holds weight row ln of each tile for the tokens 16 m + 4 g + i
+    // outputs: lane (ln, kh) holds weight row ln for the tile's rows 32 m + 8 b + 4 kh + r (i = 4 b + r)
 #pragma unroll
-    for (int m = 0; m < NMT; ++m) {
+    for (int m = 0; m < NM; ++m) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = 16 * m + 4 * g + i;
-            if (r >= nrows) continue;
-            float* o = a.out + (size_t) (row0 + r) * a.n + n0 + ln;
-            if constexpr (GU) o[0] = pf_swiglu(acc[0][m][i], acc[1][m][i], a.limit);
-            else o[0] = acc[0][m][i], o[16] = acc[1][m][i];
+        for (int i = 0; i < 16; ++i) {
+            const int r = 32 * m + 8 * (i >> 2) + 4 * kh + (i & 3);
+            if constexpr (GU) {
+                // the up row of a feature sits 16 lanes above its gate row
+                const float up = __shfl(acc[m][i], (lane + 16) & 63, kWave);
+                if (ln < 16 && r < nrows) a.out[(size_t) (row0 + r) * a.n + n0 + ln] = pf_swiglu(acc[m][i], up, a.limit);
+            } else {
+                if (r < nrows) a.out[(size_t) (row0 + r) * a.n + n0 + ln] = acc[m][i];
+            }
         }
     }
 }
@@ -590,12 +602,8 @@ __global__ __launch_bounds__(256, 2) void prefill_q4k_kernel(PfGemm a) {
     if (tile >= *a.plan.n_tiles) return;
     const int ex = a.plan.tile_expert[tile], row0 = a.plan.tile_row0[tile];
     const int nrows = min(kPfRows, a.plan.bounds[ex + 1] - row0);
-    switch ((nrows + 15) >> 4) {
-        case 1: pf_tile<GU, 1>(a, b0, b1, b2, ex, row0, nrows); break;
-        case 2: pf_tile<GU, 2>(a, b0, b1, b2, ex, row0, nrows); break;
-        case 3: pf_tile<GU, 3>(a, b0, b1, b2, ex, row0, nrows); break;
-        default: pf_tile<GU, 4>(a, b0, b1, b2, ex, row0, nrows); break;
-    }
+    if (nrows <= 32) pf_tile<GU, 1>(a, b0, b1, b2, ex, row0, nrows);
+    else pf_tile<GU, 2>(a, b0, b1, b2, ex, row0, nrows);
 }
 
 template <int ODT>
@@ -870,7 +878,7 @@ static PrefillWs prefill_carve(const maya_moe_layout& l, int n_tokens, int k, in
     auto take_act = [&](maya_prefill_act& a, size_t k) {
         a.q = (int8_t*) take(ne * k);
         a.d = (float*) take(ne * (k / 256) * 4);
-        a.s = (float*) take(ne * (k / 32) * 4);
+        a.s = (uint16_t*) take(ne * (k / 32) * 4);
     };
     take_act(w.x, (size_t) l.n_embd);
     take_act(w.h, (size_t) l.n_ff);

@@ -1,4 +1,4 @@
-// maya_probe: what this GPU gives the IQ2_S decode kernels to work with, measured with the kernels' own pieces.
+// maya_probe: what this GPU gives the expert kernels to work with, measured with the kernels' own pieces.
 //
 // A standalone program (no part of libmaya_moe.so), printing
 //   1. the shader clock (clock64 against the 100 MHz wall clock);
@@ -6,8 +6,10 @@
 //   3. the LDS pipe's time for the codebook gather (ds_read_b64 at a random index) beside a conflict-free read;
 //   4. the memory floor of the two expert kernels: their loads alone - same launch shape, same buffer-resource
 //      addressing of the stream-packed quads (load_quad), every quad requested up front, the words folded into one
-//      that is never stored - over rotating expert sets larger than the last-level cache.
-// The decode kernels' distance from the HBM roofline is read against these figures.
+//      that is never stored - over rotating expert sets larger than the last-level cache;
+//   5. the matrix instructions the prefill GEMMs use: time an instruction, alone and with vector instructions between them;
+//   6. the prefill GEMM's weight stream alone, in the GEMM's own access pattern.
+// The kernels' distances from their rooflines are read against these figures.
 //
 //   maya_probe [n_embd n_ff]      (default 7168 2048: the north-star expert; k = 8, 64 experts in rotation)
 #include <hip/hip_runtime.h>
@@ -72,8 +74,11 @@ __global__ void clock_kernel(long long* out, int iters) {
 #define A_PERM(d) "v_perm_b32 " #d ", %8, %9, " #d
 #define A_BFE(d) "v_bfe_u32 " #d ", " #d ", 3, 8"
 #define A_LSHL(d) "v_lshlrev_b32 " #d ", 3, " #d
+#define A_PKMUL(d) "v_pk_mul_lo_u16 " #d ", %8, " #d
+#define A_LSHLADD(d) "v_lshl_add_u32 " #d ", " #d ", 3, %8"
+#define A_MULLO(d) "v_mul_lo_u32 " #d ", %8, " #d
 OPK(xor, A_XOR) OPK(add, A_ADD) OPK(dot4, A_DOT4) OPK(andor, A_ANDOR) OPK(mul24, A_MUL24) OPK(cvt, A_CVT) OPK(fma, A_FMA) OPK(perm, A_PERM)
-OPK(bfe, A_BFE) OPK(lshl, A_LSHL)
+OPK(bfe, A_BFE) OPK(lshl, A_LSHL) OPK(pkmul16, A_PKMUL) OPK(lshladd, A_LSHLADD) OPK(mullo32, A_MULLO)
 
 // ---- 3. LDS reads: four chains a lane, the next index taken from the value read
 template <int MODE>  // 0: b64 at a random index of 1024 (the IQ2_S codebook gather); 1: b64 conflict-free; 2: b32 random; 3: b64 one address
@@ -100,6 +105,89 @@ __global__ __launch_bounds__(512) void lds_kernel(unsigned* out, int iters) {
         acc ^= v0.y ^ v1.y ^ v2.y ^ v3.y;
     }
     if (acc + a0 + a1 + a2 + a3 == 0x12345) out[0] = acc;
+}
+
+// ---- 5. matrix instructions: 4 independent accumulators a wave, NV vector instructions (independent xor chains) after each
+typedef int pr_v4i __attribute__((ext_vector_type(4)));
+typedef int pr_v16i __attribute__((ext_vector_type(16)));
+typedef float pr_v4f __attribute__((ext_vector_type(4)));
+#define VALU_FILL(NV)                                                                                     \
+    if (NV >= 1) asm volatile("v_xor_b32 %0, %1, %0" : "+v"(x0) : "v"(k0));                               \
+    if (NV >= 2) asm volatile("v_xor_b32 %0, %1, %0" : "+v"(x1) : "v"(k0));                               \
+    if (NV >= 3) asm volatile("v_xor_b32 %0, %1, %0" : "+v"(x2) : "v"(k0));                               \
+    if (NV >= 4) asm volatile("v_xor_b32 %0, %1, %0" : "+v"(x3) : "v"(k0));                               \
+    if (NV >= 5) asm volatile("v_xor_b32 %0, %1, %0\n v_xor_b32 %2, %1, %2" : "+v"(x0), "+v"(x1) : "v"(k0)); \
+    if (NV >= 7) asm volatile("v_xor_b32 %0, %1, %0\n v_xor_b32 %2, %1, %2" : "+v"(x2), "+v"(x3) : "v"(k0));
+// KIND 0: v_mfma_i32_16x16x64_i8, 1: v_mfma_i32_32x32x32_i8, 2: v_mfma_f32_16x16x4_f32, 3: v_mfma_i32_16x16x32_i8
+template <int KIND, int NV>
+__global__ __launch_bounds__(256) void mfma_kernel(int* out, int iters) {
+    pr_v4i a = {(int) threadIdx.x, 1, 2, 3}, b = {(int) threadIdx.x * 3, 5, 6, 7};
+    int x0 = threadIdx.x, x1 = 1, x2 = 2, x3 = 3, k0 = 0x55;
+    int r = 0;
+    if constexpr (KIND == 1) {
+        pr_v16i c[4] = {};
+        for (int i = 0; i < iters; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(c[j]) : "v"(a), "v"(b));
+                VALU_FILL(NV)
+            }
+        }
+        r = c[0][0] + c[1][1] + c[2][2] + c[3][3];
+    } else if constexpr (KIND == 2) {
+        pr_v4f c[4] = {};
+        float fa = threadIdx.x, fb = 1.5f;
+        for (int i = 0; i < iters; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+v"(c[j]) : "v"(fa), "v"(fb));
+                VALU_FILL(NV)
+            }
+        }
+        r = (int) (c[0][0] + c[1][1] + c[2][2] + c[3][3]);
+    } else {
+        pr_v4i c[4] = {};
+        for (int i = 0; i < iters; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (KIND == 0) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c[j]) : "v"(a), "v"(b));
+                else asm volatile("v_mfma_i32_16x16x32_i8 %0, %1, %2, %0" : "+v"(c[j]) : "v"(*(long*) &a), "v"(*(long*) &b));
+                VALU_FILL(NV)
+            }
+        }
+        r = c[0][0] + c[1][1] + c[2][2] + c[3][3];
+    }
+    if (r + x0 + x1 + x2 + x3 == 0x7fffffff) out[0] = r;
+}
+
+// ---- 6. the prefill GEMM's weight stream alone: waves that sweep 32 Q4_K rows (144-byte blocks) a super-block a step, the
+// next step's loads in flight during a token amount of arithmetic, a barrier a step - the GEMM's loop without its arithmetic
+typedef unsigned int pr_u4 __attribute__((ext_vector_type(4)));
+template <int LDSKB>
+__global__ __launch_bounds__(256) void q4k_sweep_kernel(const unsigned char* pool, size_t expert_bytes, int row_bytes, unsigned* sink) {
+    __shared__ unsigned char pad[LDSKB * 1024];   // (sets the workgroups a CU: 2 at 56 KB, as the GEMM's)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 31, kh = lane >> 5;
+    const unsigned char* row = pool + (size_t) blockIdx.y * expert_bytes + (size_t) (blockIdx.x * 128 + wave * 32 + n) * row_bytes;
+    const int steps = row_bytes / 144;
+    pr_u4 cur[5], nxt[5];
+    auto ld = [&](int st, pr_u4* d) {
+        const unsigned char* blk = row + (size_t) st * 144;
+        d[0] = *(const pr_u4*) blk;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) d[1 + c] = *(const pr_u4*) (blk + 16 + 32 * c + 16 * kh);
+    };
+    ld(0, cur);
+    unsigned x = 0;
+    for (int s = 0; s < steps; ++s) {
+        if (s + 1 < steps) ld(s + 1, nxt);
+#pragma unroll
+        for (int p = 0; p < 5; ++p) x ^= cur[p].x ^ cur[p].y ^ cur[p].z ^ cur[p].w;
+        for (int i = 0; i < 32; ++i) x = x * 1664525u + 1013904223u;
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < 5; ++p) cur[p] = nxt[p];
+    }
+    if (x == 0x12345678u) sink[0] = x, pad[threadIdx.x] = 1;
 }
 
 // ---- 4. the expert kernels' loads alone
@@ -217,7 +305,7 @@ int main(int argc, char** argv) {
         const double instr = (double) wgs * 8 * iters * 8, rate = instr / (us * 1e3) / simds;                         \
         printf("   %-8s %.2f  (%.1f clk)\n", #NAME, rate, shader_mhz * 1e-3 / rate);                                  \
     }
-        RUN_OP(xor) RUN_OP(add) RUN_OP(fma) RUN_OP(dot4) RUN_OP(andor) RUN_OP(mul24) RUN_OP(cvt) RUN_OP(perm) RUN_OP(bfe) RUN_OP(lshl)
+        RUN_OP(xor) RUN_OP(add) RUN_OP(fma) RUN_OP(dot4) RUN_OP(andor) RUN_OP(mul24) RUN_OP(cvt) RUN_OP(perm) RUN_OP(bfe) RUN_OP(lshl) RUN_OP(pkmul16) RUN_OP(lshladd) RUN_OP(mullo32)
     }
     {
         printf("3. LDS reads, 16 waves a CU, 4 chains a wave (clk a wave-instruction a CU)\n");
@@ -229,6 +317,26 @@ int main(int argc, char** argv) {
         printf("   %-34s %.1f\n", NAME, us * 1e3 / (instr / cus) * shader_mhz * 1e-3);                                 \
     }
         RUN_LDS(0, "b64 at a random index of 1024") RUN_LDS(1, "b64 conflict-free") RUN_LDS(2, "b32 at a random index of 1024") RUN_LDS(3, "b64 one address")
+    }
+    {
+        printf("5. matrix instructions, W waves a SIMD, 4 accumulators a wave, NV xor after each (clk a matrix instruction a SIMD)\n");
+        printf("   %-28s %8s %8s %8s %8s %8s\n", "", "NV=0", "NV=2", "NV=4", "NV=6", "NV=8");
+        const int iters = 2000;
+#define RUN_MFMA_1(KIND, NV, W, dst)                                                                                               \
+    {                                                                                                                              \
+        const float us = time_us(s, 2, [&](int) { hipLaunchKernelGGL((mfma_kernel<KIND, NV>), dim3(W * cus), dim3(256), 0, s, (int*) dclk, iters); }); \
+        dst = us * 1e3 / ((double) W * iters * 4) * shader_mhz * 1e-3;                                                             \
+    }
+#define RUN_MFMA(KIND, W, NAME)                                                                                                    \
+    {                                                                                                                              \
+        double c0, c2, c4, c6, c8;                                                                                                 \
+        RUN_MFMA_1(KIND, 0, W, c0) RUN_MFMA_1(KIND, 2, W, c2) RUN_MFMA_1(KIND, 4, W, c4) RUN_MFMA_1(KIND, 6, W, c6) RUN_MFMA_1(KIND, 8, W, c8) \
+        printf("   %-22s W=%d %8.1f %8.1f %8.1f %8.1f %8.1f\n", NAME, W, c0, c2, c4, c6, c8);                                      \
+    }
+        RUN_MFMA(0, 1, "i32_16x16x64_i8") RUN_MFMA(0, 2, "i32_16x16x64_i8") RUN_MFMA(0, 4, "i32_16x16x64_i8")
+        RUN_MFMA(3, 1, "i32_16x16x32_i8") RUN_MFMA(3, 2, "i32_16x16x32_i8")
+        RUN_MFMA(1, 1, "i32_32x32x32_i8") RUN_MFMA(1, 2, "i32_32x32x32_i8")
+        RUN_MFMA(2, 1, "f32_16x16x4_f32") RUN_MFMA(2, 2, "f32_16x16x4_f32")
     }
     {
         const size_t gr = (size_t) E / 256 * 82, dr = (size_t) FF / 256 * 82;
@@ -264,6 +372,16 @@ int main(int argc, char** argv) {
         printf("   down, 28 rows a workgroup (the kernel's shape)     %6.2f us  %.0f GB/s\n", t, dn_bytes / t / 1e3);
         t = time_us(s, 64, [&](int i) { hipLaunchKernelGGL((down_loads_kernel<56, 64>), dim3(E / 56), dim3(512), 0, s, args(i % NSETS), sink); });
         printf("   down, 56 rows a workgroup                          %6.2f us  %.0f GB/s\n", t, dn_bytes / t / 1e3);
+        {
+            // 6: the pool read as 48 "experts" of 4096 Q4_K rows of 7168 values (4032 bytes a row)
+            const int rows = 4096, row_bytes = 4032, ne = 48;
+            const size_t eb = (size_t) rows * row_bytes;
+            if ((size_t) ne * eb <= (size_t) NE * blob) {
+                const float tq = time_us(s, 4, [&](int) { hipLaunchKernelGGL(q4k_sweep_kernel<56>, dim3(rows / 128, ne), dim3(256), 0, s, pool, eb, row_bytes, sink); });
+                printf("6. the prefill GEMM's weight stream alone (Q4_K rows of 4032 bytes, 32 rows a wave, 144 bytes a row a step, 2 workgroups a CU)\n");
+                printf("   %d x %d rows  %8.2f us  %.0f GB/s\n", ne, rows, tq, (double) ne * eb / tq / 1e3);
+            }
+        }
         t = time_us(s, 16, [&](int i) { CK(hipMemcpyAsync(pool + (size_t) ((i + 1) % NSETS) * K * blob, pool + (size_t) (i % NSETS) * K * blob, (size_t) K * blob, hipMemcpyDeviceToDevice, s)); });
         printf("   for scale: a device copy of one set (%.0f MB read + written)  %6.2f us  %.0f GB/s\n", 2.0 * blob * K / 1e6, t, 2.0 * blob * K / t / 1e3);
     }

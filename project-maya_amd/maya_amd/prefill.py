@@ -64,8 +64,14 @@ class ActRows:
     def __init__(self, rows, k, device="cuda"):
         self.q = torch.zeros((rows, k), dtype=torch.int8, device=device)
         self.d = torch.zeros((rows, k // 256), dtype=torch.float32, device=device)
-        self.s = torch.zeros((rows, k // 32), dtype=torch.float32, device=device)
+        # a block's 8 sub-block code sums as two FP16 digits: [rows][k / 256][the 8 low digits, then the 8 high ones]
+        self.s = torch.zeros((rows, k // 256, 16), dtype=torch.float16, device=device)
         self.c = PAct(self.q.data_ptr(), self.d.data_ptr(), self.s.data_ptr())
+
+    def sums(self):
+        """The integer sum of every 32 codes [rows][k / 32], from the two digits (lo + 64 hi)."""
+        v = self.s.to(torch.float32)
+        return (v[:, :, :8] + 64.0 * v[:, :, 8:]).reshape(v.shape[0], -1).to(torch.int32)
 
 
 def plan(ids, expert_table, stream=None):

@@ -84,11 +84,13 @@ def test_quantized_rows_match_checker(pf, oracle):
         torch.cuda.synchronize()
         xf = xt.to(torch.float32).numpy()
         row_entry = p.row_entry.cpu().numpy()
-        q, d, s = a.q.cpu().numpy(), a.d.cpu().numpy(), a.s.cpu().numpy()
+        q, d, s = a.q.cpu().numpy(), a.d.cpu().numpy(), a.sums().cpu().numpy()
+        digits = a.s.cpu().numpy().astype(np.float32)
+        assert (digits[:, :, :8] >= 0).all() and (digits[:, :, :8] <= 63).all() and (np.abs(digits[:, :, 8:]) <= 64).all()
         for r in range(n_tokens * k):
             wd, wq, wbs = oracle.q8k_fields(oracle.quant_q8k(xf[row_entry[r] // k]))
             assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
-            assert np.array_equal(s[r], (wd[:, None] * (wbs[:, 0::2] + wbs[:, 1::2]).astype(np.float32)).reshape(-1))
+            assert np.array_equal(s[r], (wbs[:, 0::2].astype(np.int32) + wbs[:, 1::2]).reshape(-1))
 
 
 LAYER_CASES = [
@@ -132,17 +134,17 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
     assert np.array_equal(ids.cpu().numpy(), want["ids"])
     assert np.array_equal(p.row_entry.cpu().numpy()[:rows], want["row_entry"])
     assert np.array_equal(xq.q.cpu().numpy()[:rows], want["xq"])
-    assert np.array_equal(xq.d.cpu().numpy()[:rows], want["xd"]) and np.array_equal(xq.s.cpu().numpy()[:rows], want["xs"])
+    assert np.array_equal(xq.d.cpu().numpy()[:rows], want["xd"]) and np.array_equal(xq.sums().cpu().numpy()[:rows], want["xs"])
 
     # gate/up: the same integer sums as the CPU path's row dots, so only F32 summation order apart
     h = hq.f32.cpu().numpy()[:rows]
     assert rel_l2(h, want["h"]) <= 1e-5
     # H: the quantizer's bytes on the GPU's own h
-    gq, gd, gs = hq.q.cpu().numpy()[:rows], hq.d.cpu().numpy()[:rows], hq.s.cpu().numpy()[:rows]
+    gq, gd, gs = hq.q.cpu().numpy()[:rows], hq.d.cpu().numpy()[:rows], hq.sums().cpu().numpy()[:rows]
     for r in range(0, rows, max(1, rows // 40)):
         wd, wq, wbs = oracle.q8k_fields(oracle.quant_q8k(h[r]))
         assert np.array_equal(gq[r], wq) and np.array_equal(gd[r].view(np.uint32), wd.view(np.uint32)), r
-        assert np.array_equal(gs[r], (wd[:, None] * (wbs[:, 0::2] + wbs[:, 1::2]).astype(np.float32)).reshape(-1))
+        assert np.array_equal(gs[r], (wbs[:, 0::2].astype(np.int32) + wbs[:, 1::2]).reshape(-1))
     # down over the GPU's own H
     flat_ids = want["ids"].reshape(-1)
     for r in range(0, rows, max(1, rows // 12)):
@@ -150,9 +152,28 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
         want_part = oracle.rows(Q4_K, blobs[e][down_off:], n_ff, n_embd, oracle.quant_act(Q4_K, h[r]))
         assert rel_l2(part.cpu().numpy()[r], want_part) <= 1e-5, r
 
+    # The layer's outputs against the CPU path's, 1e-3.  The GPU's h is the CPU path's to 1e-5, but h is then rounded to
+    # Q8_K, where a value that sits on a rounding boundary can take the neighbouring code; ONE such code among a toy
+    # shape's 512 moves a row's output by about 1e-3 (a quarter of that at the real 2048).  A token past 1e-3 must
+    # therefore be explained by exactly that: the CPU path's down rows and weighted sum over the GPU's own h give the
+    # GPU's output to 1e-5, and the output is still within 3e-3 of the CPU path's.
     got = out.cpu().numpy()
+    part_h = part.cpu().numpy()
+    entry_row = want["entry_row"]
     for t in range(n_tokens):
-        assert rel_l2(got[t], want["out"][t]) <= 1e-3, t
+        err = rel_l2(got[t], want["out"][t])
+        if err <= 1e-3:
+            continue
+        assert n_ff < 2048 and err <= 3e-3, (t, err)
+        sel = [j for j in range(k) if entry_row[t * k + j] >= 0]
+        parts = []
+        for j in sel:
+            r = int(entry_row[t * k + j])
+            e = int(flat_ids[want["row_entry"][r]])
+            parts.append(oracle.rows(Q4_K, blobs[e][down_off:], n_ff, n_embd, oracle.quant_act(Q4_K, h[r])))
+            assert rel_l2(part_h[r], parts[-1]) <= 1e-5, (t, r)
+        explained = oracle.combine(np.stack(parts), np.array([want["w"][t, j] for j in sel], dtype=np.float32))
+        assert rel_l2(got[t], explained) <= 1e-5, (t, err)
     assert torch.equal(out16, out.to(torch.bfloat16))
 
     # the one-call layer gives the same bits as the stages
