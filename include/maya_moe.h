@@ -137,7 +137,10 @@ int maya_moe_pack_experts(const maya_moe_layout* l, const void* gate_exps, const
 const char* maya_last_error(void);
 /* Device and library identification: "gfx950 ..." (host string, valid until the next call on this thread). */
 const char* maya_device_info(void);
-/* Loads the device code and uploads the codebooks on the current device; idempotent.  Every other entry point calls it. */
+/* Loads the device code and uploads the codebooks on the current device; idempotent.  Every other entry point calls it on
+ * its first use of a device - and this set-up is the one place that allocates (the codebooks' 24 KB) and copies
+ * synchronously: call maya_init() once a device BEFORE the first call made under stream capture (a set-up attempted
+ * while the stream is capturing fails with the runtime's error, < 0, and launches nothing). */
 int maya_init(void);
 
 /* ---- dequantization to F32, bit-exact with the block formats' reference decode:

@@ -763,7 +763,8 @@ static int prefill_check(const char* what, const maya_moe_layout* l, const uint6
     // (IQ2_S: the 16-byte copies of a quad's index words want quads of a multiple of 16 bytes: 328 bytes a block)
     if (type_a == kIQ2_S && k % 512) return fail(MAYA_E_SHAPE, "%s: IQ2_S rows of %lld values: a multiple of 512 wanted", what, (long long) k);
     if ((l->gate_off | l->up_off | l->down_off) & 15) return fail(MAYA_E_ARG, "%s: matrix offsets not 16-byte aligned", what);
-    if (n_entries <= 0 || n_entries > 65535 * kPfRows || n_expert <= 0) return fail(MAYA_E_SHAPE, "%s: entries %d experts %d", what, n_entries, n_expert);
+    // (an entry is a row of the second grid dimension in the quantizers' launches)
+    if (n_entries <= 0 || n_entries > 65535 || n_expert <= 0) return fail(MAYA_E_SHAPE, "%s: entries %d (1..65535) experts %d", what, n_entries, n_expert);
     return MAYA_OK;
 }
 
@@ -896,8 +897,23 @@ int maya_moe_prefill_layer(const maya_moe_layout* l, const uint64_t* expert_tabl
                            const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
                            float* weights, void* out, int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
     if (!l || !expert_table || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "prefill_layer: null pointer");
-    if (n_tokens <= 0 || n_tokens > 8192 || k <= 0 || k > MAYA_MAX_K) return fail(MAYA_E_SHAPE, "prefill_layer: tokens %d k %d", n_tokens, k);
+    if (n_tokens <= 0 || n_tokens > 8192 || k <= 0 || k > MAYA_MAX_K || (int64_t) n_tokens * k > 65535)
+        return fail(MAYA_E_SHAPE, "prefill_layer: tokens %d k %d (at most 65535 entries a call)", n_tokens, k);
     if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "prefill_layer: workspace not 256-byte aligned");
+    // everything a stage would refuse is refused here, before the first launch ("> 0: not covered, nothing launched")
+    {
+        DeviceState* st;
+        if (const int rc0 = current_state(&st)) return rc0;
+        if (n_expert <= 0 || n_expert > MAYA_MAX_EXPERTS || k > n_expert)
+            return fail(MAYA_E_SHAPE, "prefill_layer: experts %d (1..%d) k %d", n_expert, MAYA_MAX_EXPERTS, k);
+        if (x_dtype < 0 || x_dtype > 2 || out_dtype < 0 || out_dtype > 2) return fail(MAYA_E_UNSUPPORTED, "prefill_layer: dtypes %d / %d", x_dtype, out_dtype);
+        maya_prefill_plan probe{};   // (the plan's pointers come from the workspace: only the layout's side is checked here)
+        int32_t dummy = 0;
+        probe.bounds = probe.row_entry = probe.entry_row = probe.tile_expert = probe.tile_row0 = probe.n_tiles = &dummy;
+        if (const int rc0 = prefill_check("prefill_layer", l, expert_table, n_expert, &probe, n_tokens * k, l->gate_type, l->up_type, l->n_embd)) return rc0;
+        if (const int rc0 = prefill_check("prefill_layer", l, expert_table, n_expert, &probe, n_tokens * k, l->down_type, l->down_type, l->n_ff)) return rc0;
+        if (l->n_embd % 32) return fail(MAYA_E_SHAPE, "prefill_layer: n_embd %d", l->n_embd);
+    }
     const PrefillWs w = prefill_carve(*l, n_tokens, k, n_expert, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "prefill_layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     const int ne = n_tokens * k;

@@ -275,3 +275,25 @@ def test_unsupported_and_bad_arguments(pf):
     bad.n_ff = 200
     with pytest.raises(lib.MayaError):
         pf.gate_up(bad, table, p, xq)
+    # the one-call layer refuses what a later stage would refuse BEFORE its first launch: the router has not run
+    # (ids keep their sentinel)
+    good, _ = lib.layout(Q4_K, Q4_K, 512, 256)
+    layer = pf.PrefillLayer(good, 4, 2, 16, out_dtype=torch.float32)
+    logits = torch.zeros((16, 4), dtype=torch.float32, device="cuda")
+    x = torch.zeros((16, 512), dtype=torch.float32, device="cuda")
+    for wrong in (lib.copy_layout(lib.layout(19, 19, 512, 256)[0], lib.PACK_STREAM),      # IQ1_S: no prompt GEMM
+                  lib.layout(22, 22, 512, 256)[0],                                         # IQ2_S rows in the GGUF packing
+                  lib.layout(Q4_K, 8, 512, 256)[0]):                                       # a Q8_0 down
+        layer.layout = wrong
+        layer.ids.fill_(-7)
+        with pytest.raises(lib.MayaError):
+            layer.forward(table, logits, x)
+        torch.cuda.synchronize()
+        assert bool((layer.ids == -7).all())
+    big = pf.PrefillLayer(lib.layout(Q4_K, Q4_K, 256, 256)[0], 16, 16, 4096, out_dtype=torch.float32)   # 65536 entries
+    big.ids.fill_(-7)
+    with pytest.raises(lib.MayaError):
+        big.forward(torch.arange(1, 17, dtype=torch.int64, device="cuda") * 4096, torch.zeros((4096, 16), dtype=torch.float32, device="cuda"),
+                    torch.zeros((4096, 256), dtype=torch.float32, device="cuda"))
+    torch.cuda.synchronize()
+    assert bool((big.ids == -7).all())
