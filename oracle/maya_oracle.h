@@ -50,7 +50,8 @@
  *                                       later token, promote_min against the counts, the counts' halving; the reference test's
  *                                       expectation for empty tables (miss mask 255, tests/hip/glm_handoff.cpp:118)
  *   EXL3 states / codebook ........... the reference's own golden vectors data/exl3-exllamav3 (13 .bin files made by exllamav3)
- *   EXL3 mat-vec ..................... reference build: exl3_ref.cpp bit-exact; H.H = I
+ *   EXL3 mat-vec ..................... reference build: exl3_ref.cpp bit-exact; H.H = I; the reference's CPU lane (exl3_cpu.cpp,
+ *                                      unrounded weights: a second statement of the product) to 3e-4, golden vectors of whole experts
  *   prompt-chunk rows ................ the pieces above, row by row (the Q8_K quantizer, the Q4_K row dots, SwiGLU, combine):
  *                                       a chunk's row is the CPU path's expert on that row's token
  *   mo_grouped_ref / mo_quant_i8x32 .. helpers of the tests (a double product of dequantized weights x dequantized int8 rows,

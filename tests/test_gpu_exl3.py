@@ -203,3 +203,25 @@ def test_skip_flag_and_bad_shapes(ex):
     bad2, _ = ex.make_layout(256, 128, 9, 0)
     with pytest.raises(lib.MayaError):
         ex.gate_up(ex.make_args(bad2, 1, 1, plan, w, x, h, part, out))
+
+
+def test_expert_matches_the_reference_cpu_lane(ex):
+    """Whole experts against the reference's CPU lane for EXL3 (exl3_cpu.cpp: weights and rotated input unrounded): the
+    vectors of tests/golden/refbuild_exl3cpu_vectors.npz, k = 1 with weight 1 so the layer's output is the expert's."""
+    from maya_amd import lib
+    from test_oracle_pins import _exl3cpu_case, _exl3cpu_golden
+    g = _exl3cpu_golden()
+    checked = 0
+    for i, row in enumerate(g["cases"]):
+        l, blob, x, crc = _exl3cpu_case(ex, row)
+        if crc != int(g["crc_%d" % i]):
+            continue
+        store = lib.ExpertStore([blob])
+        layer = ex.Exl3Layer(l, 1, 1, max_tokens=1)
+        out = layer.forward(store.table, torch.zeros((1, 1), dtype=torch.float32, device="cuda"), torch.from_numpy(x[None]).cuda(),
+                            limit=float(g["limits"][i])).cpu().numpy()[0]
+        torch.cuda.synchronize()
+        err = rel_l2(out, g["out_%d" % i])
+        assert err <= TOL, (i, err)
+        checked += 1
+    assert checked == len(g["cases"])

@@ -332,3 +332,76 @@ def test_iq1s_row_dot_invariants(oracle, iq1_grid):
     g2 = oracle.rows_of(IQ1_S, w2.reshape(-1), k, n, act)
     blk = (iq1s_numpy(w[:, 2], iq1_grid).astype(np.float64) * xa[None, 512:768]).sum(axis=1)
     assert np.max(np.abs((g2 - got) - blk) / mag) < 1e-6
+
+
+# ---------------------------------------------------------------------------------------------------------------- EXL3
+# The reference's CPU lane for EXL3 experts (exl3_cpu.cpp, what ds4's CPU flow runs) against the checker's EXL3 mat-vec:
+# two independent statements of the same matrix product - the lane keeps weights and rotated input unrounded, the
+# checker (exl3_ref.cpp's form, the device's) rounds both to FP16 - so they agree to the roundings: about 3e-4, bar 1e-3.
+def _exl3cpu_golden():
+    return np.load(os.path.join(HERE, "golden", "refbuild_exl3cpu_vectors.npz"))
+
+
+def _exl3cpu_case(exl3, row):
+    import zlib
+    n_embd, n_ff, kg, ku, kd, bseed, xseed = (int(v) for v in row)
+    l, nbytes = exl3.make_layout(n_embd, n_ff, [kg, ku, kd], 2)
+    blob = exl3.synth_blob(l, nbytes, bseed)
+    x = np.random.default_rng(xseed).standard_normal(n_embd).astype(np.float32)
+    return l, blob, x, zlib.crc32(x.tobytes(), zlib.crc32(blob.tobytes()))
+
+
+def _swiglu32(g, u, limit):
+    g, u = g.astype(np.float32), u.astype(np.float32)
+    if limit > 0:
+        g = np.minimum(g, np.float32(limit))
+        u = np.clip(u, -np.float32(limit), np.float32(limit))
+    return (g / (np.float32(1) + np.exp(-g)) * u).astype(np.float32)
+
+
+def test_exl3_expert_agrees_with_the_reference_cpu_lane(oracle):
+    exl3 = pytest.importorskip("maya_amd.exl3")
+    g = _exl3cpu_golden()
+    checked = 0
+    for i, row in enumerate(g["cases"]):
+        if row[0] > 2048:
+            continue                      # (the full shape is the GPU test's: seconds of scalar checker here)
+        l, blob, x, crc = _exl3cpu_case(exl3, row)
+        if crc != int(g["crc_%d" % i]):
+            continue                      # another numpy generator: the stored expectations are not for these bytes
+        mats = []
+        for r in range(3):
+            k, n = exl3.matrix_of(l, r)
+            tr, suh, svh = exl3.parts_of(l, blob, r)
+            mats.append((oracle.exl3_inner(tr, k, n, l.k2[r], 2), suh, svh))
+        h = _swiglu32(oracle.exl3_mv(*mats[0], x), oracle.exl3_mv(*mats[1], x), float(g["limits"][i]))
+        out = oracle.exl3_mv(*mats[2], h)
+        eh = np.linalg.norm(h - g["h_%d" % i]) / np.linalg.norm(g["h_%d" % i])
+        eo = np.linalg.norm(out - g["out_%d" % i]) / np.linalg.norm(g["out_%d" % i])
+        assert eh <= 1e-3 and eo <= 1e-3, (i, eh, eo)
+        assert eh > 1e-6            # not the same arithmetic: the FP16 roundings are there
+        checked += 1
+    assert checked >= 3
+
+
+def test_exl3_cpu_lane_live_where_it_was_built(oracle):
+    """Where oracle/_ref holds the CPU lane (the build container): fresh random matrices at every bitrate it takes."""
+    import ctypes as C
+    path = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "libmaya_ref_exl3cpu.so")
+    if not os.path.exists(path):
+        pytest.skip("no reference build of the CPU lane here")
+    R = C.CDLL(path)
+    R.ref_exl3_cpu_mv.argtypes = [C.c_void_p] * 3 + [C.c_int] * 3 + [C.c_void_p] * 2
+    rng = np.random.default_rng(77)
+    for k, n, k2 in ((256, 128, 2), (256, 256, 3), (384, 128, 4), (128, 256, 5), (256, 128, 6), (256, 128, 7), (128, 128, 8),
+                     (256, 128, 10), (128, 256, 12), (256, 128, 14), (128, 128, 16)):
+        words = rng.integers(0, 2 ** 32, (k // 16) * (n // 16) * 4 * k2, dtype=np.uint64).astype(np.uint32)
+        suh = (rng.integers(0, 2, k) * 2 - 1).astype(np.float16).view(np.uint16)
+        svh = ((rng.integers(0, 2, n) * 2 - 1) * rng.uniform(0.5, 1.5, n)).astype(np.float16).view(np.uint16)
+        x = rng.standard_normal(k).astype(np.float32)
+        want = np.zeros(n, dtype=np.float32)
+        assert R.ref_exl3_cpu_mv(words.ctypes.data, suh.ctypes.data, svh.ctypes.data, k, n, k2, x.ctypes.data, want.ctypes.data) == 0
+        got = oracle.exl3_mv(oracle.exl3_inner(words, k, n, k2, 2), suh, svh, x)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3, (k, n, k2)
+        # a transposed operand, a dropped scale or a wrong rotation is not a rounding: far outside the bar
+        assert np.linalg.norm(oracle.exl3_mv(oracle.exl3_inner(words, k, n, k2, 2), suh, svh, x[::-1].copy()) - want) / np.linalg.norm(want) > 0.1
