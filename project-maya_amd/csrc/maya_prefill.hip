@@ -552,10 +552,19 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
                 }
                 const pf_v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                 const pf_v16f mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_v8h, sa[m]), mb, z, 0, 0, 0);
+                // (a lane's outputs 4 b .. 4 b + 3 are the tile's rows 32 m + 8 b + 4 kh + 0..3: blocks of 8 rows past the
+                // tile's last row are skipped - most tiles of a skewed routing hold 8 rows or fewer)
+                const int nb = (nrows - 32 * m + 7) >> 3;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float t = fmaf(ndmin, mins[i], __fmul_rn(d, (float) (dot[m][0][i] + 8 * dot[m][1][i])));
-                    acc[m][i] = fmaf(dxr[m][i >> 2][i & 3], t, acc[m][i]);
+                for (int b = 0; b < 4; ++b) {
+                    if (b < nb) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int i = 4 * b + r;
+                            const float t = fmaf(ndmin, mins[i], __fmul_rn(d, (float) (dot[m][0][i] + 8 * dot[m][1][i])));
+                            acc[m][i] = fmaf(dxr[m][b][r], t, acc[m][i]);
+                        }
+                    }
                 }
             });
             if (sb + 1 < nsb) {
