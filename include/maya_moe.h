@@ -95,7 +95,8 @@ typedef struct maya_moe_args {
     const float* plan_w;       /* [n_tokens*k] combine weights */
     const uint64_t* grp_ptr;   /* [<= n_tokens*k] or NULL */
     const int32_t* grp_start;  /* [groups+1] */
-    const int32_t* grp_ent;    /* [n_tokens*k] */
+    const int32_t* grp_ent;    /* [n_tokens*k]; given WITHOUT grp_ptr: only the order in which the entry-by-entry kernels take
+                                * the entries (an expert's entries side by side: its rows come from DRAM once), -1 = the end */
     const int32_t* n_groups;   /* device count of groups (NULL: n_tokens*k) */
     const int32_t* skip;       /* NULL or a device flag: non-zero makes every kernel of the call a no-op */
     float limit;               /* SwiGLU clamp; +inf or <= 0: none */

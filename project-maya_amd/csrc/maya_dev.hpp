@@ -68,6 +68,21 @@ __device__ __forceinline__ uint32_t neg_bytes(uint32_t g, uint32_t c) {
 template <int CTRL>
 __device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true); }
 
+// The down kernels' grid is (row blocks, tokens).  A window's tokens that route the same expert read the same rows of it,
+// so the workgroups of ONE row block for all the tokens should run at the same time on the same XCD (workgroups go to the
+// XCDs in turn by their linear index, x fastest).  With the row blocks a multiple of 8: runs of 8 row blocks x all tokens -
+// index -> row block (index / (8 T)) 8 + index % 8, token (index / 8) % T - keep a row block on XCD (row block % 8) for
+// every token and its tokens' workgroups within 8 T of each other in launch order.  One token, or row blocks not a
+// multiple of 8: the grid as it is.
+__device__ __forceinline__ void down_block_of_grid(int& row_block, int& token) {
+    row_block = (int) blockIdx.x, token = (int) blockIdx.y;
+    if (gridDim.y > 1 && (gridDim.x & 7u) == 0) {
+        const unsigned id = blockIdx.y * gridDim.x + blockIdx.x, nt = gridDim.y;
+        row_block = (int) ((id / (8u * nt)) * 8u + (id & 7u));
+        token = (int) ((id >> 3) % nt);
+    }
+}
+
 // Q8_K rounding of a 256-value block held by 8 consecutive lanes, 32 values a lane: the arithmetic of the reference's
 // quantize_q8_K_kernel (src/kernels/cuda/quantize_act.cu:161-207) and codes, bit for bit, 4 codes a word in the order
 // of v.  The block's scale comes from the signed value at the FIRST largest magnitude.  Its magnitude is the largest

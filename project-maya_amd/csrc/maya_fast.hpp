@@ -365,7 +365,9 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     __shared__ int lds[kFastLdsWords];
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
-    const int e = blockIdx.y;
+    // (a window's entries in the order of grp_ent where one is given: the entries of an expert side by side; -1 ends it)
+    const int e = (a.grp_ent && !a.grp_ptr) ? a.grp_ent[blockIdx.y] : (int) blockIdx.y;
+    if (e < 0) return;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
     stage_iq2s_tables(lds, cb, 64 * NW);
@@ -441,8 +443,10 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     const uint2* stab = (const uint2*) (lds + 2048);
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int r0 = blockIdx.x * ROWS;
-    const int e0 = blockIdx.y * a.k;   // the token's first entry; wave w = its slot w
+    int bx, by;
+    down_block_of_grid(bx, by);
+    const int r0 = bx * ROWS;
+    const int e0 = by * a.k;   // the token's first entry; wave w = its slot w
     // Everything the workgroup needs before its weights is requested side by side, ahead of the one barrier: the skip
     // flag, the plan (the wave's slot; the slots' presence and weights for the combine), the slot's h and the tables.
     // A wave past slot k - 1 reads that slot's data and drops it: no branch, and no load waits on another.
@@ -551,7 +555,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
             sum = have ? t : sum;
             first = first && !have;
         }
-        const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
+        const size_t o = (size_t) by * n_embd + r0 + c;
         if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
         if (a.add2) sum = __fadd_rn(sum, a.add2[o]);
         a.out[o] = sum;

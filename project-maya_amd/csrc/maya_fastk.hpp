@@ -67,7 +67,9 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe
     constexpr int NU = 32 * NW;
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
-    const int e = blockIdx.y;
+    // (a window's entries in the order of grp_ent where one is given: the entries of an expert side by side; -1 ends it)
+    const int e = (a.grp_ent && !a.grp_ptr) ? a.grp_ent[blockIdx.y] : (int) blockIdx.y;
+    if (e < 0) return;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
@@ -122,8 +124,10 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
     if (a.skip && *a.skip) return;
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int r0 = blockIdx.x * ROWS;
-    const int e0 = blockIdx.y * a.k, ent = e0 + wave;
+    int bx, by;
+    down_block_of_grid(bx, by);
+    const int r0 = bx * ROWS;
+    const int e0 = by * a.k, ent = e0 + wave;
     const uint64_t blob = wave < a.k ? a.plan_ptr[ent] : 0ull;
     if (blob != 0ull) {
         // (an idle lane reads the last position's weights again and meets them with zero activations)
@@ -202,7 +206,7 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
             sum = first ? pv : __fadd_rn(sum, pv);
             first = false;
         }
-        const size_t o = (size_t) blockIdx.y * n_embd + r0 + c;
+        const size_t o = (size_t) by * n_embd + r0 + c;
         if (a.add && (!a.add_flag || *a.add_flag)) sum = __fadd_rn(sum, a.add[o]);
         if (a.add2) sum = __fadd_rn(sum, a.add2[o]);
         a.out[o] = sum;

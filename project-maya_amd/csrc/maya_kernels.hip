@@ -871,6 +871,8 @@ __global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__
     const int ng = s_ng;
     if (e <= ng) grp_start[e] = s_start[e];
     if (g >= 0) grp_ent[s_start[g] + rank] = e;
+    // (past the grouped entries: -1, so that grp_ent read as a list of length n says where it ends)
+    if (e >= s_start[ng] && e < n) grp_ent[e] = -1;
 }
 
 // ------------------------------------------------------------------------------------------------ expert rows
@@ -2201,12 +2203,19 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
         }
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }
-    if (n_tokens > 1 && !(gate_up_by_entries(a) && down_by_entries(a))) {
+    if (n_tokens > 1) {
         if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
-        a.grp_ptr = w.grp_ptr;
-        a.grp_start = w.grp_start;
-        a.grp_ent = w.grp_ent;
-        a.n_groups = w.n_groups;
+        if (gate_up_by_entries(a) && down_by_entries(a)) {
+            // The entry-by-entry kernels take no groups, only the ORDER of the entries: those of one expert side by side,
+            // so that they run at the same time on the same XCD (an entry's row block b always lands on XCD b % 8) and
+            // the expert's rows come from DRAM once and from that XCD's L2 for the other tokens.
+            a.grp_ent = w.grp_ent;
+        } else {
+            a.grp_ptr = w.grp_ptr;
+            a.grp_start = w.grp_start;
+            a.grp_ent = w.grp_ent;
+            a.n_groups = w.n_groups;
+        }
     }
     if ((rc = maya_moe_gate_up(&a, stream))) return rc;
     if (down_rounds_h(a)) {
