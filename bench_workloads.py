@@ -224,9 +224,8 @@ def batch8_mixed(K, W):
         distinct.append(int(torch.unique(ids).numel()))
     stream = torch.cuda.Stream()
 
-    def step(i):
-        sh = dense[i % n_sh].forward(x)
-        layer.forward(table, logits[i % n_sets], x, add=sh)
+    def step(i):   # (the shared expert's launches run beside the routed experts' on the library's second stream)
+        layer.forward(table, logits[i % n_sets], x, shared=dense[i % n_sh])
 
     dt = timed_graph(step, K, W, stream)
     d_avg = float(np.mean([distinct[(W + i) % n_sets] for i in range(K)]))

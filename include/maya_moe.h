@@ -302,6 +302,26 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
                                  float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* The routed layer and the expert EVERY token takes (a shared expert), side by side:
+ *   out[t] = shared->add[t] + shared_expert(x[t]) + sum_j weights[t][j] * expert_{ids[t][j]}(x[t]).
+ * The reference runs the shared expert's down rows as extra blocks of the routed experts' gate/up launch
+ * (include/strata/kernels/glm_fast.hpp:496-501, src/kernels/cuda/glm_fast.cu:4841-4849) so that they cost no time of
+ * their own; here the shared expert's launches (quantize x, gate/up, quantize h, down + add) go to a second stream that
+ * the library keeps a device (default priority), forked from `stream` by an event when the call starts and joined back
+ * before the routed down launch, which adds the routed experts to the shared expert's output.  Every result is the bits
+ * of maya_moe_gate_up / maya_moe_down on `shared` followed by maya_moe_layer_decode_routed with add = shared->out.
+ *   shared: the stage arguments of the shared expert as maya_moe_gate_up / maya_moe_down take them - k = 1, n_tokens
+ *   entries, plan_ptr all its blob, plan_w all 1, its groups (one group of n_tokens entries), its own x / h / hq (NULL
+ *   where the down kernel rounds h itself) / part buffers, `add` the layer's residual or NULL, `out` its own
+ *   [n_tokens][n_embd] buffer (not the layer's out).
+ * The fork and the join are event records and waits, so the call may be captured in a HIP graph (maya_init() first).
+ * Calls on one device are serialised on the host by a lock; whatever fails, `stream` has joined the second stream again
+ * when the call returns. */
+int maya_moe_layer_decode_shared(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                                 const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
+                                 float limit, const maya_moe_args* shared, int32_t* ids, float* weights, float* out,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* The same layer for callers that cannot allocate or own a workspace (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): the workspace is a file-scope device array of MAYA_STATIC_SCRATCH_BYTES inside the
  * library, one copy a device, held until the process ends.  No counterpart in the reference (its callers own every buffer,

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -32,6 +33,11 @@ struct DeviceState {
     int lds_limit = 65536;
     int n_cu = 0;
     void* static_scratch = nullptr;   // this device's copy of the file-scope scratch array (maya_moe_layer_decode_static)
+    // maya_moe_layer_decode_shared: the stream the shared expert's launches run on beside the caller's, and the two events
+    // that fork it from the caller's stream and join it back (default priority; one call at a time a device: side_mu)
+    hipStream_t side = nullptr;
+    hipEvent_t side_fork = nullptr, side_join = nullptr;
+    std::mutex side_mu;
 };
 // the current device's state, initialised on first use (gfx950 only); MAYA_OK or a status
 int current_state(DeviceState** out);

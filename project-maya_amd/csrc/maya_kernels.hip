@@ -79,6 +79,10 @@ int current_state(DeviceState** out) {
             e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));   // (this device is the current one)
             if (e != hipSuccess || sp == nullptr) return hip_fail(e == hipSuccess ? hipErrorInvalidSymbol : e, "address of the static scratch");
             s.static_scratch = sp;
+            if ((e = hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking)) != hipSuccess) return hip_fail(e, "the shared expert's stream");
+            if ((e = hipEventCreateWithFlags(&s.side_fork, hipEventDisableTiming)) != hipSuccess ||
+                (e = hipEventCreateWithFlags(&s.side_join, hipEventDisableTiming)) != hipSuccess)
+                return hip_fail(e, "the shared expert's events");
             s.cb.iq2s = d;
             s.cb.iq1s = d + 1024;
             s.lds_limit = (int) p.sharedMemPerBlock;
@@ -2154,9 +2158,14 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
     return maya_moe_layer_decode_routed(l, expert_table, n_expert, k, nullptr, logits, x, x_dtype, n_tokens, limit, add, ids, weights,
                                         out, workspace, workspace_bytes, stream);
 }
-int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
-                                 const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
-                                 int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+}  // extern "C"
+
+// The layer's launches.  `join`: an event the down launch waits for (the shared expert's output, which `add` then points
+// at), *joined set once the stream waits for it.
+static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                             const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                             int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream,
+                             hipEvent_t join, bool* joined) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     if (!l) return fail(MAYA_E_ARG, "layer_decode: null layout");
@@ -2224,7 +2233,55 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
     } else {
         if ((rc = maya_quant_act(l->down_type, w.h, MAYA_DT_F32, 0, n_tokens * k, l->n_ff, w.hq, stream))) return rc;
     }
+    if (join) {
+        MAYA_HIP(hipStreamWaitEvent(as_stream(stream), join, 0));
+        *joined = true;
+    }
     return maya_moe_down(&a, stream);
+}
+
+extern "C" {
+
+int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                                 const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                                 int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    return layer_decode_core(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out, workspace,
+                             workspace_bytes, stream, nullptr, nullptr);
+}
+
+int maya_moe_layer_decode_shared(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                                 const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const maya_moe_args* shared,
+                                 int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!l || !shared || !x) return fail(MAYA_E_ARG, "layer_decode_shared: null pointer");
+    if (const int rc = check_layout(shared->layout)) return rc;
+    if (shared->k != 1 || shared->n_tokens != n_tokens || shared->layout.n_embd != l->n_embd)
+        return fail(MAYA_E_SHAPE, "layer_decode_shared: the shared expert's arguments hold %d tokens x %d slots of %lld values, the layer %d tokens of %lld",
+                    shared->n_tokens, shared->k, (long long) shared->layout.n_embd, n_tokens, (long long) l->n_embd);
+    if (!shared->x.q || !shared->x.d || !shared->h || !shared->out || !shared->plan_ptr || !shared->plan_w)
+        return fail(MAYA_E_ARG, "layer_decode_shared: the shared expert's arguments lack a buffer (x, h, out, plan)");
+    if (shared->out == out) return fail(MAYA_E_ARG, "layer_decode_shared: the shared expert's out is the layer's out");
+    // one call at a time a device: the side stream and its two events are the device's
+    std::lock_guard<std::mutex> lock(st->side_mu);
+    hipStream_t s = as_stream(stream);
+    MAYA_HIP(hipEventRecord(st->side_fork, s));
+    MAYA_HIP(hipStreamWaitEvent(st->side, st->side_fork, 0));
+    // the shared expert beside the routed experts' head and gate/up launches: quantize x, gate/up, quantize h, down + add
+    int rc = maya_quant_act(shared->layout.gate_type, x, x_dtype, 0, n_tokens, shared->layout.n_embd, shared->x, st->side);
+    if (!rc) rc = maya_moe_gate_up(shared, st->side);
+    if (!rc && shared->hq.q)   // (no hq: a down kernel that rounds h itself, as in maya_moe_down)
+        rc = maya_quant_act(shared->layout.down_type, shared->h, MAYA_DT_F32, 0, n_tokens, shared->layout.n_ff, shared->hq, st->side);
+    if (!rc) rc = maya_moe_down(shared, st->side);
+    // (whatever happened, the side stream joins the caller's again: a capture must not end with it forked)
+    bool joined = false;
+    hipError_t e = hipEventRecord(st->side_join, st->side);
+    if (e == hipSuccess && !rc)
+        rc = layer_decode_core(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, shared->out, ids, weights, out,
+                               workspace, workspace_bytes, stream, st->side_join, &joined);
+    if (e == hipSuccess && !joined) e = hipStreamWaitEvent(s, st->side_join, 0);
+    if (e != hipSuccess && !rc) rc = hip_fail(e, "layer_decode_shared: joining the shared expert's stream");
+    return rc;
 }
 
 int maya_moe_layer_decode_static(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,

@@ -21,6 +21,7 @@ EXPORTS = [
     "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
     "maya_moe_tab_update",
     "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv", "maya_moe_layer_decode_static",
+    "maya_moe_layer_decode_shared",
 ]
 
 
@@ -112,6 +113,8 @@ def load():
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
     L.maya_moe_layer_decode_routed.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32, vp, vp, vp,
                                                vp, vp, sz, vp]
+    L.maya_moe_layer_decode_shared.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32,
+                                               C.POINTER(Args), vp, vp, vp, vp, sz, vp]
     L.maya_moe_route_sigmoid.argtypes = [vp, vp, i32, i32, i32, f32, i32, vp, vp, vp]
     L.maya_moe_route_plan.argtypes = [C.POINTER(Router), vp, i32, i32, i32, vp, vp, vp, vp, vp]
     _lib = L
@@ -341,9 +344,11 @@ class MoeLayer:
         self.weights = torch.empty((max_tokens, k), dtype=torch.float32, device=device)
         self.out = torch.empty((max_tokens, n_embd), dtype=torch.float32, device=device)
 
-    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None, routed=None):
+    def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None, routed=None, shared=None,
+                shared_limit=float("inf")):
         """router: None (the softmax router) or a Router (kind, norm, bias pointer, w_scale); routed = (ids, weights)
-        [nt, k] tensors: the tokens are already routed (logits is then ignored)."""
+        [nt, k] tensors: the tokens are already routed (logits is then ignored); shared: a DenseExpert over the same
+        tokens that runs beside the routed experts (maya_moe_layer_decode_shared) - out = add + shared(x) + routed(x)."""
         nt = x.shape[0]
         assert nt <= self.max_tokens and x.is_contiguous()
         if routed is not None:
@@ -352,6 +357,16 @@ class MoeLayer:
             logits = None
         else:
             assert logits.is_contiguous()
+        if shared is not None:
+            assert shared.n == nt and shared.n_embd == self.n_embd
+            a = shared.args
+            a.limit, a.add = shared_limit, (add.data_ptr() if add is not None else None)
+            check(load().maya_moe_layer_decode_shared(C.byref(self.layout), _p(expert_table), self.n_expert, self.k,
+                                                      C.byref(router) if router is not None else None, _p(logits), _p(x), dtype_id(x),
+                                                      nt, limit, C.byref(a), _p(self.ids), _p(self.weights), _p(self.out), _p(self.ws),
+                                                      self.ws_bytes, _stream(stream)))
+            a.add = None
+            return self.out[:nt]
         if router is not None:
             check(load().maya_moe_layer_decode_routed(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, C.byref(router),
                                                       _p(logits), _p(x), dtype_id(x), nt, limit, _p(add), _p(self.ids),
