@@ -61,9 +61,12 @@ __device__ __forceinline__ float pos_q4k_value(const PosQ4K& p, const u32x4 hdr,
 
 // ---- gate/up: a workgroup of NW waves = the 2 * 32 NW positions of a (gate row, up row) pair of n_embd = 1024 NW values;
 // grid (n_ff / ROWS, entries); entry e = token e / k, slot e % k.  Rows in batches of 8, one row ahead in registers.
-template <int NW, int ROWS, int MINW>
+// AHEAD (8 rows): all of a lane's rows are requested up front - the launches of a few entries, whose workgroups do not fill
+// the chip and would otherwise run at the memory's latency a row.
+template <int NW, int ROWS, int MINW, bool AHEAD = false>
 __global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe_args a) {
     static_assert(ROWS % 8 == 0, "rows come in batches of 8");
+    static_assert(!AHEAD || ROWS == 8, "every row up front: one batch");
     constexpr int NU = 32 * NW;
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
@@ -84,17 +87,30 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe
     const __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob + a.layout.gate_off, (uint32_t) (a.layout.down_off - a.layout.gate_off));
     u32x4 hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) r0 * rb, 0);
     u32x4 qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) r0 * rb, 0);
+    u32x4 ha[AHEAD ? ROWS : 1], qa[AHEAD ? ROWS : 1];
+    if constexpr (AHEAD) {
+        ha[0] = hn, qa[0] = qn;
+#pragma unroll
+        for (int i = 1; i < ROWS; ++i) {
+            ha[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) (r0 + i) * rb, 0);
+            qa[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) (r0 + i) * rb, 0);
+        }
+    }
     float acc[8];
 #pragma unroll 1
     for (int r = 0; r < ROWS; r += 8) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const u32x4 hc = hn, qc = qn;
-            if (r + i + 1 < ROWS) {
-                hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) (r0 + r + i + 1) * rb, 0);
-                qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) (r0 + r + i + 1) * rb, 0);
+            if constexpr (AHEAD) {
+                acc[i] = pos_q4k_value(p, ha[i], qa[i]);
+            } else {
+                const u32x4 hc = hn, qc = qn;
+                if (r + i + 1 < ROWS) {
+                    hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) (r0 + r + i + 1) * rb, 0);
+                    qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) (r0 + r + i + 1) * rb, 0);
+                }
+                acc[i] = pos_q4k_value(p, hc, qc);
             }
-            acc[i] = pos_q4k_value(p, hc, qc);
             asm volatile("" : "+v"(acc[i]));
         }
         const float v = reduce8_half(acc, lane);
@@ -116,9 +132,12 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe
 // ---- down + combine, n_ff = 32 NU <= 2048 (NU positions a row on the first NU lanes of one wave; NU a multiple of 8, the
 // lanes past it idle): wave w = slot w of token blockIdx.y, rows in batches of 8; grid (n_embd / ROWS, tokens).  Without a
 // rounded h (hq.q == NULL) a wave rounds its slot's h to Q8_K itself.
-template <int ROWS, int MINW, int NU = 64>
+// AHEAD: all ROWS rows of the wave are requested before anything else is done (one or two slots on one token: a few
+// hundred waves on the whole chip, each with one row in flight, run at the memory's latency a row).
+template <int ROWS, int MINW, int NU = 64, bool AHEAD = false>
 __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a) {
     static_assert(ROWS % 8 == 0, "rows come in batches of 8");
+    static_assert(!AHEAD || ROWS == 8, "every row up front: one batch");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
@@ -143,6 +162,14 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
         const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) n_embd * rb);
         u32x4 hn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) r0 * rb, 0);
         u32x4 qn = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) r0 * rb, 0);
+        u32x4 ha[AHEAD ? ROWS : 1], qa[AHEAD ? ROWS : 1];
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int i = 1; i < ROWS; ++i) {
+                ha[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_hdr, (uint32_t) (r0 + i) * rb, 0);
+                qa[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, p.o_q, (uint32_t) (r0 + i) * rb, 0);
+            }
+        }
         if (a.hq.q) {
             pos_q4k_codes(p, pos, a.hq.q + (size_t) ent * (32 * NU), a.hq.d + (size_t) ent * NU, a.hq.bsums + (size_t) ent * (2 * NU));
         } else {
@@ -178,6 +205,17 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
             p.dx = 0.0f;
         }
         float acc[8];
+        if constexpr (AHEAD) {
+            ha[0] = hn, qa[0] = qn;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc[i] = pos_q4k_value(p, ha[i], qa[i]);
+                asm volatile("" : "+v"(acc[i]));
+            }
+            float v = reduce8_half(acc, lane);
+            v += __shfl_xor(v, 32, kWave);
+            if ((lane & 35) == 0) part[wave][(lane >> 2) & 7] = v;
+        } else
 #pragma unroll 1
         for (int r = 0; r < ROWS; r += 8) {
 #pragma unroll

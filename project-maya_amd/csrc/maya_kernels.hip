@@ -1495,12 +1495,12 @@ bool down_q4k_pos_ok(const maya_moe_args& a) {
            (l.down_off & 15) == 0;
 }
 int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
-    // 16 rows a workgroup, 8 when the call has so few entries that 16 would leave compute units idle
+    // 16 rows a workgroup, 8 - all requested up front - when the call has so few entries that 16 would leave compute units idle
     const bool small = (long long) (a.layout.n_ff / 16) * a.n_tokens * a.k < 512;
     const int rows = small ? 8 : 16;
     const dim3 grid((unsigned) (a.layout.n_ff / rows), (unsigned) (a.n_tokens * a.k));
 #define MAYA_Q4(NWV)                                                                                              \
-    if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 8>), grid, dim3(64 * NWV), 0, s, a);          \
+    if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 4, true>), grid, dim3(64 * NWV), 0, s, a);    \
     else hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a);
     switch (a.layout.n_embd / 1024) {
         case 2: MAYA_Q4(2) break;
@@ -1528,7 +1528,12 @@ int launch_down_q4k_pos(const maya_moe_args& a, hipStream_t s) {
     else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_q4k_pos_kernel<R, 8, 48>), grid, block, 0, s, a);     \
     else hipLaunchKernelGGL((down_q4k_pos_kernel<R, 8>), grid, block, 0, s, a);
     if (rows == 32) { MAYA_ROWS(32) }
-    else if (rows == 8) { MAYA_ROWS(8) }
+    else if (rows == 8) {
+        // every row of a wave requested up front (128 registers)
+        if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_q4k_pos_kernel<8, 4, 32, true>), grid, block, 0, s, a);
+        else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_q4k_pos_kernel<8, 4, 48, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((down_q4k_pos_kernel<8, 4, 64, true>), grid, block, 0, s, a);
+    }
     else { MAYA_ROWS(16) }
 #undef MAYA_ROWS
     MAYA_LAUNCHED("down_q4k_pos_kernel");
