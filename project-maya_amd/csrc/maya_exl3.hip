@@ -195,16 +195,16 @@ __device__ __forceinline__ h2 as_h2(uint32_t v) {
 template <int K2>
 __device__ __forceinline__ void tile_values(uint32_t wa, uint32_t wb, int sh, h2& w01, h2& w23) {
     const uint32_t c = __builtin_amdgcn_alignbit(wa, wb, (uint32_t) sh);   // (wa : wb) >> sh, 0 <= sh < 32
-    uint32_t hb[4];
+    uint32_t prod[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t st = __builtin_amdgcn_ubfe(c, Taps<K2>::below(i), 16);
-        const uint32_t prod = st * 0x83DCD12Du;
-        hb[i] = __builtin_amdgcn_sad_u8(prod, 0u, 0x6400u);   // the bits of FP16(1024 + byte sum)
-    }
+    for (int i = 0; i < 4; ++i) prod[i] = __builtin_amdgcn_ubfe(c, Taps<K2>::below(i), 16) * 0x83DCD12Du;
+    // 0x6400 + the byte sum (at most 1020: no carry out of the half) = the bits of FP16(1024 + byte sum); the pair's second
+    // sum lands in the upper half directly (v_sad_hi_u8: (sum << 16) + the third operand), so the pair needs no packing
+    const uint32_t p01 = __builtin_amdgcn_sad_hi_u8(prod[1], 0u, __builtin_amdgcn_sad_u8(prod[0], 0u, 0x64006400u));
+    const uint32_t p23 = __builtin_amdgcn_sad_hi_u8(prod[3], 0u, __builtin_amdgcn_sad_u8(prod[2], 0u, 0x64006400u));
     const h2 kinv = as_h2(0x1eee1eeeu), kbias = as_h2(0xc931c931u);
-    w01 = __builtin_elementwise_fma(as_h2(hb[0] | (hb[1] << 16)), kinv, kbias);
-    w23 = __builtin_elementwise_fma(as_h2(hb[2] | (hb[3] << 16)), kinv, kbias);
+    w01 = __builtin_elementwise_fma(as_h2(p01), kinv, kbias);
+    w23 = __builtin_elementwise_fma(as_h2(p23), kinv, kbias);
 }
 template <int K2, int NT>
 __device__ __forceinline__ void walk_tiles_fast(const uint32_t* __restrict__ trellis, int k, int ld, int tc, int lane,
