@@ -117,6 +117,13 @@ __device__ __forceinline__ int ex_entry_of(const maya_exl3_args& a, const ExGrou
 
 // xr = FP16(H(x * suh)) of one activation into LDS; every wave of the workgroup takes blocks of 128 values (`tmp` is not
 // used: the transform runs in registers)
+// PAIRED (the compile-time walk): inside every 16 rows the word of rows 2q, 2q + 1 and the word of rows 2q + 8, 2q + 9 -
+// a lane's four rows - sit side by side (words 2q, 2q + 1), so the walk reads them in one 8-byte LDS read
+__device__ __forceinline__ int paired_pos(int i) {
+    const int w = (i >> 1) & 7;
+    return (i & ~15) | ((w < 4 ? 2 * w : 2 * (w - 4) + 1) << 1) | (i & 1);
+}
+template <bool PAIRED>
 __device__ __forceinline__ void rotate_in(const float* __restrict__ x, const uint16_t* __restrict__ suh, int k, float* tmp,
                                           __half* xr) {
     (void) tmp;
@@ -125,8 +132,8 @@ __device__ __forceinline__ void rotate_in(const float* __restrict__ x, const uin
         const int i0 = b * 128 + lane;
         float v0 = __fmul_rn(x[i0], f16_bits_to_f32(suh[i0])), v1 = __fmul_rn(x[i0 + 64], f16_bits_to_f32(suh[i0 + 64]));
         had128_wave(v0, v1, lane);
-        xr[i0] = __float2half_rn(v0);
-        xr[i0 + 64] = __float2half_rn(v1);
+        xr[PAIRED ? paired_pos(i0) : i0] = __float2half_rn(v0);
+        xr[PAIRED ? paired_pos(i0 + 64) : i0 + 64] = __float2half_rn(v1);
     }
     __syncthreads();
 }
@@ -233,8 +240,8 @@ __device__ __forceinline__ void walk_tiles_fast(const uint32_t* __restrict__ tre
         ra[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, oa, t_off + (uint32_t) i * step, 0);
         rb[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, ob, t_off + (uint32_t) i * step, 0);
     }
-    const uint32_t* xw = (const uint32_t*) xr;   // pairs of FP16 activations
-    const int xs = xr_stride >> 1;
+    const uint2* xw = (const uint2*) xr;   // the lane's two pairs of FP16 activations of a row tile (rotate_in<true>'s order)
+    const int xs = xr_stride >> 2;
 #pragma unroll 1
     for (int ks = 0; ks < nks; ks += kAhead) {
 #pragma unroll
@@ -245,11 +252,12 @@ __device__ __forceinline__ void walk_tiles_fast(const uint32_t* __restrict__ tre
             rb[i] = __builtin_amdgcn_raw_buffer_load_b32(rs, ob, nxt, 0);
             h2 w01, w23;
             tile_values<K2>(ca, cb, sh, w01, w23);
-            const int rw = (ks + i) * 8 + q;   // the word of rows 2q, 2q + 1 of this row tile
+            const int rw = (ks + i) * 4 + q;   // rows 2q, 2q + 1 | 2q + 8, 2q + 9 of this row tile
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                acc[t] = __builtin_amdgcn_fdot2(w01, as_h2(xw[t * xs + rw]), acc[t], false);
-                acc[t] = __builtin_amdgcn_fdot2(w23, as_h2(xw[t * xs + rw + 4]), acc[t], false);
+                const uint2 xv = xw[t * xs + rw];
+                acc[t] = __builtin_amdgcn_fdot2(w01, as_h2(xv.x), acc[t], false);
+                acc[t] = __builtin_amdgcn_fdot2(w23, as_h2(xv.y), acc[t], false);
             }
         }
     }
@@ -300,7 +308,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gate_up_kernel(maya_exl3_args
         for (int t = 0; t < NTC; ++t) {
             const float* x = a.x + (size_t) (ents[t] / a.k) * xs;
             for (int role = 0; role < 2; ++role)
-                rotate_in(x, (const uint16_t*) (blob + a.layout.suh[role]), k, tmp, xr + ((size_t) t * 2 + role) * k);
+                rotate_in<(K2 > 0)>(x, (const uint16_t*) (blob + a.layout.suh[role]), k, tmp, xr + ((size_t) t * 2 + role) * k);
         }
         float raw[2][NTC];
 #pragma unroll
@@ -374,7 +382,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_gu_split_kernel(maya_exl3_arg
         for (int t = 0; t < NTC; ++t) ents[t] = ex_entry_of(a, gr, c0 + t);
         __syncthreads();
         for (int t = 0; t < NTC; ++t)
-            rotate_in(a.x + (size_t) (ents[t] / a.k) * xs + (size_t) ks * kb, suh, kb, tmp, xr + (size_t) t * kb);
+            rotate_in<true>(a.x + (size_t) (ents[t] / a.k) * xs + (size_t) ks * kb, suh, kb, tmp, xr + (size_t) t * kb);
         float acc[NTC];
 #pragma unroll
         for (int t = 0; t < NTC; ++t) acc[t] = 0.0f;
@@ -437,7 +445,7 @@ __global__ __launch_bounds__(kExThreads) void exl3_down_kernel(maya_exl3_args a)
         for (int t = 0; t < NTC; ++t) ents[t] = ex_entry_of(a, gr, c0 + t);
         __syncthreads();
         for (int t = 0; t < NTC; ++t)
-            rotate_in(a.h + (size_t) ents[t] * k, (const uint16_t*) (blob + a.layout.suh[2]), k, tmp, xr + (size_t) t * k);
+            rotate_in<(K2 > 0)>(a.h + (size_t) ents[t] * k, (const uint16_t*) (blob + a.layout.suh[2]), k, tmp, xr + (size_t) t * k);
         float acc[NTC];
 #pragma unroll
         for (int t = 0; t < NTC; ++t) acc[t] = 0.0f;
