@@ -238,6 +238,17 @@ int maya_moe_plan(const int32_t* ids, int n_entries, const uint64_t* expert_tabl
 int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, int32_t* grp_start, int32_t* grp_ent,
                    int32_t* n_groups, void* stream);
 
+/* A window's routing, plan and groups in ONE launch (the softmax router, up to 256 experts, n_tokens * k <= 256): what
+ * maya_moe_route_plan followed by maya_moe_group writes, bit for bit - one workgroup routes the tokens a wave each and
+ * groups their plans itself (glmf::moe_route + moe_win_group_kernel, include/strata/kernels/glm_fast.hpp:424-458,
+ * src/kernels/cuda/glm_fast.cu:7545-7625).  maya_moe_route_window_ok: 1 when the arguments are covered;
+ * maya_moe_layer_decode* and maya_exl3_layer_decode take this launch for windows of up to four tokens (the workgroup
+ * routes four tokens at a time: beyond that the separate launches, a workgroup a token, are faster). */
+int maya_moe_route_window_ok(const struct maya_router* router, int n_tokens, int n_expert, int k);
+int maya_moe_route_window(const struct maya_router* router, const float* logits, int n_tokens, int n_expert, int k,
+                          const uint64_t* expert_table, int32_t* ids, float* weights, uint64_t* plan_ptr, uint64_t* grp_ptr,
+                          int32_t* grp_start, int32_t* grp_ent, int32_t* n_groups, void* stream);
+
 /* ---- the expert rows.
  * maya_moe_gate_up: h[e][r] = swiglu(gate_r . x[token(e)], up_r . x[token(e)]) for every entry:
  *   glmf::moe_gate_up (include/strata/kernels/glm_fast.hpp:496-498), iq::gate_up (src/ds4/ds4_iq.cuh:88-89),

@@ -775,7 +775,13 @@ int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_tab
     const Exl3Ws w = exl3_carve(*l, n_tokens, k, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "exl3 layer: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
     int rc;
-    if (logits) {   // route and plan in one launch; null: ids / weights are given
+    bool grouped = false;
+    if (logits && n_tokens > 1 && n_tokens <= 4 && maya_moe_route_window_ok(nullptr, n_tokens, n_expert, k)) {   // a window of up to four tokens (one pass of the routing workgroup): route, plan and group in one launch
+        if ((rc = maya_moe_route_window(nullptr, logits, n_tokens, n_expert, k, expert_table, ids, weights, w.plan_ptr, w.grp_ptr, w.grp_start,
+                                        w.grp_ent, w.n_groups, stream)))
+            return rc;
+        grouped = true;
+    } else if (logits) {   // route and plan in one launch; null: ids / weights are given
         if ((rc = maya_moe_route_plan(nullptr, logits, n_tokens, n_expert, k, expert_table, ids, weights, w.plan_ptr, stream))) return rc;
     } else if ((rc = maya_moe_plan(ids, n_tokens * k, expert_table, n_expert, w.plan_ptr, stream))) return rc;
     maya_exl3_args a{};
@@ -785,7 +791,7 @@ int maya_exl3_layer_decode(const maya_exl3_layout* l, const uint64_t* expert_tab
     a.plan_ptr = w.plan_ptr;
     a.plan_w = weights;
     if (n_tokens > 1) {
-        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
+        if (!grouped && (rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
         a.grp_ptr = w.grp_ptr;
         a.grp_start = w.grp_start;
         a.grp_ent = w.grp_ent;

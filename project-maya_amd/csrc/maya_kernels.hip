@@ -501,14 +501,15 @@ __device__ __forceinline__ int wave_max_i32(int v) {
 //    values as signed integers and -1 marks "taken" or "no such expert"; a round is a 4-way maximum a lane, the wave
 //    maximum, and the first lane (lowest expert: lower register first, then lower lane) that holds it.
 //  * renormalisation: the k weights summed in slot order in double, one division a lane.
-__device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm) {
-    const int lane = threadIdx.x;
-    double ex[4];
+// (the token's exponentials already 4 a lane in ex; the wave's lane i < k returns slot i: its expert and weight.  `tab`:
+// the residency table's entries of the lane's four experts, NULL when no plan is wanted; the slot's blob address then
+// comes back in my_ptr - read from the chosen expert's lane, no second trip to memory.)
+__device__ __forceinline__ void route_narrow_regs(int n_expert, int k, const double (&ex)[4], const uint64_t* tab, int& my_id,
+                                                  float& my_weight, uint64_t& my_ptr) {
+    const int lane = threadIdx.x & 63;
     int lo[4], hi[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        const int e = 64 * r + lane;
-        ex[r] = e < n_expert ? sm.ex[e] : 0.0;   // (+0.0 past the end: adding it changes nothing)
         lo[r] = __double2loint(ex[r]);
         hi[r] = __double2hiint(ex[r]);
     }
@@ -533,7 +534,8 @@ __device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm)
     int key[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) key[r] = 64 * r + lane < n_expert ? __float_as_int((float) (ex[r] * (double) inv)) : -1;
-    int my_id = 0, my_w = 0;
+    int id = 0, my_w = 0;
+    uint64_t ptr = 0ull;
     for (int i = 0; i < k; ++i) {
         const int top = wave_max_i32(max(max(key[0], key[1]), max(key[2], key[3])));
         unsigned long long b = __ballot(key[0] == top);
@@ -541,17 +543,39 @@ __device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm)
         if (b == 0ull) b = __ballot(key[1] == top), r = 1;
         if (b == 0ull) b = __ballot(key[2] == top), r = 2;
         if (b == 0ull) b = __ballot(key[3] == top), r = 3;
-        const int at = __builtin_ctzll(b);
+        const int at = __builtin_amdgcn_readfirstlane(__builtin_ctzll(b));
 #pragma unroll
         for (int q = 0; q < 4; ++q) key[q] = (q == r && lane == at) ? -1 : key[q];
-        if (lane == i) my_id = 64 * r + at, my_w = top;
+        if (lane == i) id = 64 * r + at, my_w = top;
+        if (tab) {
+            const uint64_t tq = r == 0 ? tab[0] : r == 1 ? tab[1] : r == 2 ? tab[2] : tab[3];
+            const uint32_t plo = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) tq, at);
+            const uint32_t phi = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) (tq >> 32), at);
+            if (lane == i) ptr = ((uint64_t) phi << 32) | plo;
+        }
     }
     double s = 0.0;
     for (int i = 0; i < k; ++i) s += (double) __int_as_float(__builtin_amdgcn_readlane(my_w, i));
     const double sc = fmax(s, 6.103515625e-05);
+    my_id = id;
+    my_weight = (float) ((double) __int_as_float(my_w) / sc);
+    my_ptr = ptr;
+}
+__device__ __forceinline__ void route_narrow(int n_expert, int k, RouterLds& sm) {
+    const int lane = threadIdx.x;
+    double ex[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int e = 64 * r + lane;
+        ex[r] = e < n_expert ? sm.ex[e] : 0.0;   // (+0.0 past the end: adding it changes nothing)
+    }
+    int id;
+    float w;
+    uint64_t ptr;
+    route_narrow_regs(n_expert, k, ex, nullptr, id, w, ptr);
     if (lane < k) {
-        sm.id[lane] = my_id;
-        sm.w[lane] = (float) ((double) __int_as_float(my_w) / sc);
+        sm.id[lane] = id;
+        sm.w[lane] = w;
     }
 }
 
@@ -822,61 +846,126 @@ __global__ void plan_kernel(const int32_t* __restrict__ ids, int n, const uint64
 // grouping produces, src/kernels/cuda/glm_fast.cu:7545-7590).  n <= 256 entries: one workgroup, entry e's thread finds the
 // first entry with its blob (its group's leader); leaders are ranked by a prefix count; members are ranked inside their
 // group the same way.  Entries with a null blob belong to no group.
-__global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__ plan, int n,
-                                                    uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
-                                                    int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups) {
-    __shared__ uint64_t s_ptr[256];
-    __shared__ int s_leader[256];   // the first entry with the same blob, -1 for a null blob
-    __shared__ int s_gidx[256];     // leader entry -> group index
-    __shared__ int s_count[256];    // group -> entries
-    __shared__ int s_start[257];
-    __shared__ int s_ng;
+struct GroupLds {
+    uint64_t ptr[256];
+    int leader[256];   // the first entry with the same blob, -1 for a null blob
+    int gidx[256];     // leader entry -> group index
+    int count[256];    // group -> entries
+    int start[257];
+    int ng;
+};
+// 256 threads, g.ptr[0 .. n) filled (and a barrier passed); thread e = entry e
+__device__ __forceinline__ void group_entries(GroupLds& g, int n, uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
+                                              int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups) {
     const int e = threadIdx.x;
-    s_ptr[e] = e < n ? plan[e] : 0ull;
-    s_count[e] = 0;
-    __syncthreads();
+    g.count[e] = 0;
     int leader = -1;
-    if (e < n && s_ptr[e] != 0ull) {
+    if (e < n && g.ptr[e] != 0ull) {
         leader = e;
         for (int f = 0; f < e; ++f)
-            if (s_ptr[f] == s_ptr[e]) {
+            if (g.ptr[f] == g.ptr[e]) {
                 leader = f;
                 break;
             }
     }
-    s_leader[e] = leader;
+    g.leader[e] = leader;
     __syncthreads();
     if (leader == e) {
-        int g = 0;
-        for (int f = 0; f < e; ++f) g += s_leader[f] == f;
-        s_gidx[e] = g;
+        int gi = 0;
+        for (int f = 0; f < e; ++f) gi += g.leader[f] == f;
+        g.gidx[e] = gi;
     }
     __syncthreads();
-    int rank = 0, g = -1;
+    int rank = 0, gi = -1;
     if (leader >= 0) {
-        g = s_gidx[leader];
-        for (int f = 0; f < e; ++f) rank += s_leader[f] == leader;
-        atomicAdd(&s_count[g], 1);
-        if (leader == e) grp_ptr[g] = s_ptr[e];
+        gi = g.gidx[leader];
+        for (int f = 0; f < e; ++f) rank += g.leader[f] == leader;
+        atomicAdd(&g.count[gi], 1);
+        if (leader == e) grp_ptr[gi] = g.ptr[e];
     }
     __syncthreads();
     if (e == 0) {
         int ng = 0, acc = 0;
-        for (int f = 0; f < n; ++f) ng += s_leader[f] == f;
+        for (int f = 0; f < n; ++f) ng += g.leader[f] == f;
         for (int i = 0; i < ng; ++i) {
-            s_start[i] = acc;
-            acc += s_count[i];
+            g.start[i] = acc;
+            acc += g.count[i];
         }
-        s_start[ng] = acc;
+        g.start[ng] = acc;
         *n_groups = ng;
-        s_ng = ng;
+        g.ng = ng;
     }
     __syncthreads();
-    const int ng = s_ng;
-    if (e <= ng) grp_start[e] = s_start[e];
-    if (g >= 0) grp_ent[s_start[g] + rank] = e;
+    const int ng = g.ng;
+    if (e <= ng) grp_start[e] = g.start[e];
+    if (gi >= 0) grp_ent[g.start[gi] + rank] = e;
     // (past the grouped entries: -1, so that grp_ent read as a list of length n says where it ends)
-    if (e >= s_start[ng] && e < n) grp_ent[e] = -1;
+    if (e >= g.start[ng] && e < n) grp_ent[e] = -1;
+}
+__global__ __launch_bounds__(256) void group_kernel(const uint64_t* __restrict__ plan, int n,
+                                                    uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
+                                                    int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups) {
+    __shared__ GroupLds g;
+    const int e = threadIdx.x;
+    g.ptr[e] = e < n ? plan[e] : 0ull;
+    __syncthreads();
+    group_entries(g, n, grp_ptr, grp_start, grp_ent, n_groups);
+}
+
+// A window's head in ONE launch (2 ... 16 tokens, the softmax router, up to 256 experts), grid (1 + n_embd / 256, tokens):
+// workgroup (0, 0) routes every token - a wave a token, the token's experts 4 a lane, nothing but registers: the
+// maximum, the exponentials, then route_narrow_regs - writes ids / weights / plan and groups the plan itself
+// (group_kernel's arithmetic), so a window needs no grouping launch; the workgroups (b >= 1, t) round x like
+// layer_head_kernel's.  x NULL: routing only, grid (1, 1).
+template <int DT>
+__global__ __launch_bounds__(256) void window_head_kernel(const float* __restrict__ logits, int n_expert, int k, int n_tokens,
+                                                          const uint64_t* __restrict__ table, int32_t* __restrict__ ids,
+                                                          float* __restrict__ weights, uint64_t* __restrict__ plan,
+                                                          uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
+                                                          int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups,
+                                                          const void* __restrict__ x, int64_t n_embd, maya_act xq) {
+    __shared__ GroupLds g;
+    __shared__ int qs[264];
+    if (blockIdx.x == 0) {
+        if (blockIdx.y != 0) return;
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        for (int t = wave; t < n_tokens; t += 4) {
+            const float* l = logits + (size_t) t * n_expert;
+            float lv[4];
+            uint64_t tab[4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int e = 64 * r + lane;
+                lv[r] = e < n_expert ? l[e] : -INFINITY;
+                tab[r] = e < n_expert ? table[e] : 0ull;
+                mx = fmaxf(mx, lv[r]);
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+            double ex[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) ex[r] = 64 * r + lane < n_expert ? exp((double) lv[r] - (double) mx) : 0.0;
+            int id;
+            float w;
+            uint64_t ptr;
+            route_narrow_regs(n_expert, k, ex, tab, id, w, ptr);
+            if (lane < k) {
+                ids[(size_t) t * k + lane] = id;
+                weights[(size_t) t * k + lane] = w;
+                plan[(size_t) t * k + lane] = ptr;
+                g.ptr[t * k + lane] = ptr;
+            }
+        }
+        const int n = n_tokens * k;
+        if ((int) threadIdx.x >= n) g.ptr[threadIdx.x] = 0ull;
+        __syncthreads();
+        group_entries(g, n, grp_ptr, grp_start, grp_ent, n_groups);
+    } else {
+        const int t = blockIdx.y, b = blockIdx.x - 1, j = threadIdx.x;
+        const float xv = load_x<DT>(x, (int64_t) t * n_embd + (int64_t) b * 256 + j);
+        quant_q8k_block(xv, j, true, qs, xq, (size_t) t * n_embd + (size_t) b * 256);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ expert rows
@@ -1869,6 +1958,25 @@ int maya_moe_route_plan(const maya_router* router, const float* logits, int n_to
     return MAYA_OK;
 }
 
+int maya_moe_route_window_ok(const maya_router* router, int n_tokens, int n_expert, int k) {
+    return (!router || router->kind == MAYA_ROUTER_SOFTMAX) && n_tokens >= 1 && n_tokens <= MAYA_MAX_TOKENS && n_expert >= 1 && n_expert <= 256 &&
+           k >= 1 && k <= MAYA_MAX_K && k <= n_expert && n_tokens * k <= 256;
+}
+int maya_moe_route_window(const maya_router* router, const float* logits, int n_tokens, int n_expert, int k, const uint64_t* expert_table,
+                          int32_t* ids, float* weights, uint64_t* plan_ptr, uint64_t* grp_ptr, int32_t* grp_start, int32_t* grp_ent,
+                          int32_t* n_groups, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!logits || !expert_table || !ids || !weights || !plan_ptr || !grp_ptr || !grp_start || !grp_ent || !n_groups)
+        return fail(MAYA_E_ARG, "route_window: null pointer");
+    if (!maya_moe_route_window_ok(router, n_tokens, n_expert, k))
+        return fail(MAYA_E_UNSUPPORTED, "route_window: the softmax router, up to 256 experts and 256 entries (tokens %d experts %d k %d)", n_tokens, n_expert, k);
+    hipLaunchKernelGGL(window_head_kernel<MAYA_DT_F32>, dim3(1, 1), dim3(256), 0, as_stream(stream), logits, n_expert, k, n_tokens, expert_table, ids,
+                       weights, plan_ptr, grp_ptr, grp_start, grp_ent, n_groups, nullptr, (int64_t) 0, maya_act{nullptr, nullptr, nullptr});
+    MAYA_LAUNCHED("window_head_kernel");
+    return MAYA_OK;
+}
+
 int maya_moe_route_tiered(const maya_router* router, const float* logits, int n_tokens, int layer, int n_expert, int k,
                           const maya_residency* r, int promote_min, int32_t* ids, float* weights, uint64_t* plan_ptr, void* stream) {
     DeviceState* st;
@@ -2118,6 +2226,11 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
     return MAYA_OK;
 }
 
+// Windows of up to this many tokens take window_head_kernel: its one workgroup routes four tokens at a time, so four tokens
+// cost one router's time and save the grouping launch (configs[4], 4 tokens: 172.9 -> 171.3 us), eight cost two and lose
+// more than the launch saves (configs[2], 8 tokens: 256.0 -> 261.8 us, A/B on one box).
+constexpr int kWindowHeadTokens = 4;
+
 // workspace carve-up of maya_moe_layer_decode (every region 256-byte aligned)
 struct LayerWs {
     uint64_t *plan_ptr, *grp_ptr;
@@ -2197,7 +2310,20 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
     a.part = w.part;
     a.add = add;
     a.out = out;
-    if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
+    bool grouped = false;
+    if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
+        n_tokens <= kWindowHeadTokens && maya_moe_route_window_ok(router, n_tokens, n_expert, k)) {
+        // a window, one launch: route every token, plan, group, Q8_K of x
+        const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
+        hipStream_t s = as_stream(stream);
+        switch (x_dtype) {
+            case MAYA_DT_F32: hipLaunchKernelGGL(window_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, n_tokens, expert_table, ids, weights, w.plan_ptr, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, x, (int64_t) l->n_embd, w.x); break;
+            case MAYA_DT_BF16: hipLaunchKernelGGL(window_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, n_tokens, expert_table, ids, weights, w.plan_ptr, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, x, (int64_t) l->n_embd, w.x); break;
+            default: hipLaunchKernelGGL(window_head_kernel<MAYA_DT_F16>, grid, dim3(256), 0, s, logits, n_expert, k, n_tokens, expert_table, ids, weights, w.plan_ptr, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, x, (int64_t) l->n_embd, w.x); break;
+        }
+        MAYA_LAUNCHED("window_head_kernel");
+        grouped = true;
+    } else if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2) {
         // one launch: route, plan, Q8_K of x
         const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
         hipStream_t s = as_stream(stream);
@@ -2218,7 +2344,7 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
         if ((rc = maya_quant_act(l->gate_type, x, x_dtype, 0, n_tokens, l->n_embd, w.x, stream))) return rc;
     }
     if (n_tokens > 1) {
-        if ((rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
+        if (!grouped && (rc = maya_moe_group(w.plan_ptr, n_tokens * k, w.grp_ptr, w.grp_start, w.grp_ent, w.n_groups, stream))) return rc;
         if (gate_up_by_entries(a) && down_by_entries(a)) {
             // The entry-by-entry kernels take no groups, only the ORDER of the entries: those of one expert side by side,
             // so that they run at the same time on the same XCD (an entry's row block b always lands on XCD b % 8) and

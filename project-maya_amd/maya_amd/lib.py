@@ -21,7 +21,7 @@ EXPORTS = [
     "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
     "maya_moe_tab_update",
     "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv", "maya_moe_layer_decode_static",
-    "maya_moe_layer_decode_shared",
+    "maya_moe_layer_decode_shared", "maya_moe_route_window_ok", "maya_moe_route_window",
 ]
 
 
@@ -117,6 +117,8 @@ def load():
                                                C.POINTER(Args), vp, vp, vp, vp, sz, vp]
     L.maya_moe_route_sigmoid.argtypes = [vp, vp, i32, i32, i32, f32, i32, vp, vp, vp]
     L.maya_moe_route_plan.argtypes = [C.POINTER(Router), vp, i32, i32, i32, vp, vp, vp, vp, vp]
+    L.maya_moe_route_window_ok.argtypes = [C.POINTER(Router), i32, i32, i32]
+    L.maya_moe_route_window.argtypes = [C.POINTER(Router), vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 
@@ -238,6 +240,23 @@ def route_plan(logits, k, expert_table, router=None, stream=None):
     check(load().maya_moe_route_plan(None if router is None else C.byref(router), _p(logits), nt, ne, k, _p(expert_table), _p(ids),
                                      _p(w), _p(pl), _stream(stream)))
     return ids, w, pl
+
+
+def route_window(logits, k, expert_table, stream=None):
+    """A window's ids, weights, plan and groups in one launch (maya_moe_route_window: the softmax router, up to 256
+    experts): what route_plan followed by group returns."""
+    nt, ne = logits.shape
+    dev, n = logits.device, nt * k
+    ids = torch.empty((nt, k), dtype=torch.int32, device=dev)
+    w = torch.empty((nt, k), dtype=torch.float32, device=dev)
+    pl = torch.empty(n, dtype=torch.int64, device=dev)
+    grp_ptr = torch.zeros(n, dtype=torch.int64, device=dev)
+    grp_start = torch.zeros(n + 1, dtype=torch.int32, device=dev)
+    grp_ent = torch.zeros(n, dtype=torch.int32, device=dev)
+    n_groups = torch.zeros(1, dtype=torch.int32, device=dev)
+    check(load().maya_moe_route_window(None, _p(logits), nt, ne, k, _p(expert_table), _p(ids), _p(w), _p(pl), _p(grp_ptr), _p(grp_start),
+                                       _p(grp_ent), _p(n_groups), _stream(stream)))
+    return ids, w, pl, (grp_ptr, grp_start, grp_ent, n_groups)
 
 
 class Tiers:

@@ -184,3 +184,58 @@ def test_sigmoid_router_refuses_non_finite_rows(lib, oracle, ne):
     ids, w = _check_sigmoid(lib, oracle, logits, bias, k, 1.0, 2)
     assert np.all(ids == -1) and np.all(w == 0.0)
 
+
+
+def _window_logits(rng, nt, ne):
+    """Rows that press the router's rules: random, all equal, a many-way tie at the top, one dominant expert, many equal
+    values, one expert with every other probability exactly 0."""
+    logits = rng.standard_normal((nt, ne)).astype(np.float32)
+    for t in range(nt):
+        kind = t % 6
+        if kind == 1:
+            logits[t, :] = 0.25
+        elif kind == 2:
+            logits[t, rng.choice(ne, min(12, ne), replace=False)] = 4.0
+        elif kind == 3:
+            logits[t, rng.integers(ne)] = 60.0
+        elif kind == 4:
+            logits[t] = np.round(logits[t] * 2) / 2
+        elif kind == 5:
+            logits[t, :] = -1e30
+            logits[t, ne - 1] = 0.0
+    return logits
+
+
+@pytest.mark.parametrize("nt,ne,k", ((2, 256, 8), (3, 160, 6), (4, 256, 8), (5, 64, 8), (8, 256, 8), (16, 256, 16), (16, 8, 1),
+                                     (7, 200, 10), (12, 65, 3), (1, 256, 8)))
+def test_window_routing_in_one_launch(lib, oracle, nt, ne, k):
+    """maya_moe_route_window = maya_moe_route_plan + maya_moe_group, bit for bit (ids, weights, plan, groups), with experts
+    that are not resident and tokens that share experts; ids also against the CPU checker."""
+    rng = np.random.default_rng(1000 + 31 * nt + ne + k)
+    logits = _window_logits(rng, nt, ne)
+    table = torch.from_numpy((rng.integers(1, 1 << 40, ne) * 16).astype(np.int64)).cuda()
+    table[rng.choice(ne, max(1, ne // 8), replace=False)] = 0      # not resident: null plan entries, no group
+    if ne >= 4:
+        table[2] = table[3]                                        # two experts behind one blob: one group
+    ld = torch.from_numpy(logits).cuda()
+    assert lib.load().maya_moe_route_window_ok(None, nt, ne, k) == 1
+    ids, w, pl, (gp, gs, ge, ng) = lib.route_window(ld, k, table)
+    ids2, w2, pl2 = lib.route_plan(ld, k, table)
+    gp2, gs2, ge2, ng2 = lib.group(pl2)
+    torch.cuda.synchronize()
+    assert torch.equal(ids, ids2) and torch.equal(w, w2) and torch.equal(pl, pl2)
+    n = int(ng.item())
+    assert n == int(ng2.item())
+    assert torch.equal(gp[:n], gp2[:n]) and torch.equal(gs[:n + 1], gs2[:n + 1]) and torch.equal(ge, ge2)
+    wi, _ = oracle.router_topk(logits, k)
+    assert np.array_equal(ids.cpu().numpy(), wi)
+
+
+def test_window_routing_refuses_what_it_does_not_cover(lib):
+    L = lib.load()
+    assert L.maya_moe_route_window_ok(None, 4, 512, 8) == 0        # more than 256 experts
+    assert L.maya_moe_route_window_ok(None, 16, 256, 16) == 1
+    assert L.maya_moe_route_window_ok(None, 17, 256, 8) == 0
+    r = lib.Router(lib.ROUTER_SIGMOID, 1, None, 1.0)
+    import ctypes as C
+    assert L.maya_moe_route_window_ok(C.byref(r), 4, 256, 8) == 0   # the sigmoid router keeps its own launches
