@@ -14,6 +14,7 @@
 
 namespace maya {
 
+
 typedef const __attribute__((address_space(1))) uint8_t* gptr8;
 typedef const __attribute__((address_space(1))) uint16_t* gptr16;
 typedef const __attribute__((address_space(1))) uint32_t __attribute__((aligned(2))) * gptr32_a2;
@@ -102,6 +103,25 @@ __device__ __forceinline__ void stage_iq2s_tables(int* lds, const Codebooks& cb,
 }
 
 constexpr int kFastLdsWords = 2048 + 512;
+
+// The position-mapped kernels' form of the second table: per sign byte the two v_perm_b32 selectors that pick, for the
+// eight values it covers, each activation code from y (bit clear) or from the negated copy -y (bit set): selector byte i
+// of a word = i + 4 * bit i.  LDS: [0, 2048) words the codebook, [2048, 2560) the selectors.
+__device__ __forceinline__ void stage_iq2s_tables_sel(int* lds, const Codebooks& cb, int nthreads) {
+    const int* src = (const int*) cb.iq2s;
+    for (int i = threadIdx.x; i < 2048; i += nthreads) lds[i] = src[i];
+    for (int j = threadIdx.x; j < 256; j += nthreads) {
+        const int i = j;
+        uint32_t lo = 0x03020100u, hi = 0x03020100u;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            if (i & (1 << b)) lo |= 4u << (8 * b);
+            if (i & (16 << b)) hi |= 4u << (8 * b);
+        }
+        lds[2048 + 2 * j] = (int) lo;
+        lds[2048 + 2 * j + 1] = (int) hi;
+    }
+}
 
 // the lane's slice of an activation row: units sub + LPR j
 template <int KU, int LPR>
@@ -251,6 +271,31 @@ __global__ __launch_bounds__(512) void down_iq2s_1tok_kernel(maya_moe_args a, Co
 // stay in 8 registers), walks down the rows with a ring of prefetched rows, and every 8 rows a butterfly over the
 // lanes turns 8 per-lane values into per-row sums.  Loads of a wave are contiguous 512-byte / 128-byte runs.
 
+// The value of lane (lane ^ MASK), without address arithmetic: a DPP operand for masks 1, 2 (quad permutes) and 8 (a
+// rotation by 8 inside a row of 16 lanes), ds_swizzle for 4 and 16 (an LDS-crossbar exchange inside 32 lanes whose
+// pattern is an immediate), the gfx950 half-wave swap for 32.  (__shfl_xor costs four vector instructions of index
+// arithmetic per call before its ds_bpermute.)
+template <int MASK>
+__device__ __forceinline__ float xor_lane(float v) {
+    const int i = __float_as_int(v);
+    if constexpr (MASK == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0xB1, 0xf, 0xf, true));        // quad_perm [1,0,3,2]
+    else if constexpr (MASK == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x128, 0xf, 0xf, true));  // row_ror:8
+    else if constexpr (MASK == 4) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x101F));                    // swap 4
+    else if constexpr (MASK == 16) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x401F));                   // swap 16
+    else {
+        static_assert(MASK == 32, "masks inside a wave");
+        const auto r = __builtin_amdgcn_permlane32_swap(i, i, false, false);   // r[0] = (lower, lower), r[1] = (upper, upper)
+        return __int_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+    }
+}
+// v + the value of lane ^ 32 (both halves get lower + upper, the order __shfl_xor's form adds them in)
+__device__ __forceinline__ float add_other_half(float v) {
+    const int i = __float_as_int(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(i, i, false, false);
+    return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
 // acc[i] = this lane's value for row i of the batch.  On return every lane holds, in acc[0], the sum over its
 // 32-lane half of the values of row (lane >> 2) & 7.
 __device__ __forceinline__ float reduce8_half(float (&acc)[8], int lane) {
@@ -259,17 +304,17 @@ __device__ __forceinline__ float reduce8_half(float (&acc)[8], int lane) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float send = b4 ? acc[i] : acc[i + 4], keep = b4 ? acc[i + 4] : acc[i];
-        v4[i] = keep + __shfl_xor(send, 16, kWave);
+        v4[i] = keep + xor_lane<16>(send);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const float send = b3 ? v4[i] : v4[i + 2], keep = b3 ? v4[i + 2] : v4[i];
-        v2[i] = keep + __shfl_xor(send, 8, kWave);
+        v2[i] = keep + xor_lane<8>(send);
     }
     const float send = b2 ? v2[0] : v2[1], keep = b2 ? v2[1] : v2[0];
-    float v = keep + __shfl_xor(send, 4, kWave);
-    v += __shfl_xor(v, 2, kWave);
-    v += __shfl_xor(v, 1, kWave);
+    float v = keep + xor_lane<4>(send);
+    v += xor_lane<2>(v);
+    v += xor_lane<1>(v);
     return v;
 }
 
@@ -311,27 +356,26 @@ __device__ __forceinline__ RawIQ2S quad_row(const QuadIQ2S& q) {
     r.d = (R & 1) ? (d >> 16) : (d & 0xffffu);
     return r;
 }
-// One sub-block against the lane's activation codes y and their negation yn: with m the negative values' mask,
-//   sum s_i g_i y_i = dot4(g ^ m, y) + dot4(m, -y)      (g ^ 0xff = -g - 1, m = -1 there)
-// so each 16-value half needs one accumulator and no subtraction.  dy8 = the activation scale / 8.
-__device__ __forceinline__ float unit_value(const RawIQ2S& r, const uint2* grid, const uint2* stab, const int (&y)[8],
+// One sub-block against the lane's activation codes y and their negation yn.  The signs go onto the activation, not
+// the weight: v_perm_b32 over the pair (-y word, y word) with the sign byte's selector takes -y_i where value i is
+// negative, and the codebook word meets it in one dot4 - two instructions per four weights, no xor, no mask term.
+// dy8 = the activation scale / 8.
+__device__ __forceinline__ float unit_value(const RawIQ2S& r, const uint2* grid, const uint2* ssel, const int (&y)[8],
                                             const int (&yn)[8], float dy8) {
     int t0 = 0, t1 = 0;
 #pragma unroll
     for (int l = 0; l < 4; ++l) {
         const uint32_t idx = ((r.i4 >> (8 * l)) & 255u) | ((r.hs << (8 - 2 * l)) & 0x300u);
         const uint2 g = grid[idx];
-        const uint2 m = stab[(r.sg4 >> (8 * l)) & 255u];
+        const uint2 sl = ssel[(r.sg4 >> (8 * l)) & 255u];
+        const int ya = (int) __builtin_amdgcn_perm((uint32_t) yn[2 * l], (uint32_t) y[2 * l], sl.x);
+        const int yb = (int) __builtin_amdgcn_perm((uint32_t) yn[2 * l + 1], (uint32_t) y[2 * l + 1], sl.y);
         if (l < 2) {
-            t0 = dot4((int) (g.x ^ m.x), y[2 * l], t0);
-            t0 = dot4((int) m.x, yn[2 * l], t0);
-            t0 = dot4((int) (g.y ^ m.y), y[2 * l + 1], t0);
-            t0 = dot4((int) m.y, yn[2 * l + 1], t0);
+            t0 = dot4((int) g.x, ya, t0);
+            t0 = dot4((int) g.y, yb, t0);
         } else {
-            t1 = dot4((int) (g.x ^ m.x), y[2 * l], t1);
-            t1 = dot4((int) m.x, yn[2 * l], t1);
-            t1 = dot4((int) (g.y ^ m.y), y[2 * l + 1], t1);
-            t1 = dot4((int) m.y, yn[2 * l + 1], t1);
+            t1 = dot4((int) g.x, ya, t1);
+            t1 = dot4((int) g.y, yb, t1);
         }
     }
     const int s0 = 2 * (int) ((r.hs >> 8) & 15u) + 1, s1 = 2 * (int) ((r.hs >> 12) & 15u) + 1;
@@ -370,7 +414,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     if (e < 0) return;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
-    stage_iq2s_tables(lds, cb, 64 * NW);
+    stage_iq2s_tables_sel(lds, cb, 64 * NW);
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
@@ -428,6 +472,101 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     }
 }
 
+// ---- gate/up, one token, as a stream of tiles: the same arithmetic as gate_up_iq2s_pos_kernel (a row is the same
+// sequence of operations, so its bits are the same), but the workgroups stay: gridDim.x workgroups - as many as the chip
+// holds at once - walk the (entry, 8-row block) tiles t = blockIdx.x, blockIdx.x + gridDim.x, ... and request the next
+// tile's first rows while they compute this one's.  A workgroup pays the cold start (arguments, plan, tables, first
+// weights: three memory round trips one after the other) once instead of once per 16 rows, and no second round of
+// workgroups starts behind the first.  The plan's blob addresses ride in a register, entry i on lane i.
+template <int NW, int MINW>
+__global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(maya_moe_args a, Codebooks cb) {
+    constexpr int NU = 32 * NW;  // sub-blocks a row
+    __shared__ int lds[kFastLdsWords];
+    __shared__ float part[2][2 * NW][8];
+    const uint2* grid = (const uint2*) lds;
+    const uint2* stab = (const uint2*) (lds + 2048);
+    const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
+    const bool is_up = t >= NU;
+    const int u = is_up ? t - NU : t;
+    const int n_ent = a.k;   // one token: entry = plan slot
+    // everything the first tile needs is requested side by side: no load waits on another
+    const int skipv = a.skip ? *a.skip : 0;
+    int y[8];
+    {
+        const int4* q = (const int4*) a.x.q;
+        const int4 ya = q[2 * u], yb = q[2 * u + 1];
+        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+    }
+    const float dy8 = a.x.d[u] * 0.125f;
+    stage_iq2s_tables_sel(lds, cb, 64 * NW);
+    if (skipv) return;
+    int yn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
+    constexpr uint32_t qb = NU / 8 * 82 * 4;  // bytes of a quad of rows
+    const int n_ff = a.layout.n_ff;
+    const int tiles_per_entry = n_ff >> 3, n_tiles = n_ent * tiles_per_entry;
+    const uint32_t gu_bytes = (uint32_t) (a.layout.down_off - a.layout.gate_off);
+    const QuadOffs qo = quad_offs<NU>(is_up ? (uint32_t) (a.layout.up_off - a.layout.gate_off) : 0u, u);
+    // the resource of a tile's expert (an absent expert: an empty resource, whose loads read as zero and touch nothing);
+    // the entry is the same for the whole workgroup, so its blob address is a scalar load
+    int tile = blockIdx.x;
+    if (tile >= n_tiles) return;
+    int e = tile / tiles_per_entry, rb = tile - e * tiles_per_entry;
+    uint64_t blob = a.plan_ptr[e];
+    __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob ? blob + a.layout.gate_off : 0ull, blob ? gu_bytes : 0u);
+    QuadIQ2S ring = load_quad(rs, qo, (uint32_t) (2 * rb) * qb);
+    __syncthreads();
+    float acc[8];
+    int buf = 0;
+    // The ring is consumed in place: a register pair of the quad is requested again, for the quad after, as soon as its
+    // last row is done, so a lane never holds a second copy of a quad (12 registers saved: 8 waves a SIMD).
+#define MAYA_TROW(B, R)                                                          \
+    acc[B + R] = unit_value(quad_row<R>(ring), grid, stab, y, yn, dy8);          \
+    asm volatile("" : "+v"(acc[B + R]));                                         \
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+    for (;;) {
+        const uint32_t o1 = (uint32_t) (2 * rb + 1) * qb;
+        MAYA_TROW(0, 0) MAYA_TROW(0, 1)
+        ring.is01 = __builtin_amdgcn_raw_buffer_load_b128(rs, qo.is, o1, 0);
+        MAYA_TROW(0, 2) MAYA_TROW(0, 3)
+        ring.is23 = __builtin_amdgcn_raw_buffer_load_b128(rs, qo.is + 16u, o1, 0);
+        ring.hs = __builtin_amdgcn_raw_buffer_load_b64(rs, qo.hs, o1, 0);
+        ring.d = __builtin_amdgcn_raw_buffer_load_b64(rs, qo.d, o1, 0);
+        // the next tile (past the end: the empty resource)
+        const int nt = tile + (int) gridDim.x;
+        const bool more = nt < n_tiles;
+        const int ne = more ? nt / tiles_per_entry : 0, nrb = nt - ne * tiles_per_entry;
+        const uint64_t pblob = a.plan_ptr[ne];
+        const uint64_t nblob = more ? pblob : 0ull;
+        const __amdgpu_buffer_rsrc_t nrs = weight_rsrc(nblob ? nblob + a.layout.gate_off : 0ull, nblob ? gu_bytes : 0u);
+        const uint32_t o2 = (uint32_t) (2 * nrb) * qb;
+        MAYA_TROW(4, 0) MAYA_TROW(4, 1)
+        ring.is01 = __builtin_amdgcn_raw_buffer_load_b128(nrs, qo.is, o2, 0);
+        MAYA_TROW(4, 2) MAYA_TROW(4, 3)
+        ring.is23 = __builtin_amdgcn_raw_buffer_load_b128(nrs, qo.is + 16u, o2, 0);
+        ring.hs = __builtin_amdgcn_raw_buffer_load_b64(nrs, qo.hs, o2, 0);
+        ring.d = __builtin_amdgcn_raw_buffer_load_b64(nrs, qo.d, o2, 0);
+        const float v = reduce8_half(acc, lane);
+        if ((lane & 3) == 0) part[buf][hw][(lane >> 2) & 7] = v;
+        const bool present = blob != 0ull;
+        __syncthreads();
+        if (t < 8) {
+            float g = part[buf][0][t], up = part[buf][NW][t];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                g += part[buf][w][t];
+                up += part[buf][NW + w][t];
+            }
+            if (present) a.h[(size_t) e * n_ff + 8 * rb + t] = swiglu(g, up, a.limit);
+        }
+        if (!more) break;
+        tile = nt, e = ne, rb = nrb, rs = nrs, blob = nblob, buf ^= 1;
+    }
+#undef MAYA_TROW
+}
+
 // ---- down + combine, one token, n_ff = 32 NU <= 2048 (NU sub-blocks a row on the first NU lanes of one wave; NU a
 // multiple of 8, the lanes past it idle): wave w = plan slot w, rows in batches of 8; grid (n_embd / ROWS).  The slots' rows
 // meet in LDS and are summed in slot order.
@@ -475,7 +614,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
             v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
         }
     }
-    stage_iq2s_tables(lds, cb, 512);
+    stage_iq2s_tables_sel(lds, cb, 512);
     if (threadIdx.x < 8) {
         s_on[threadIdx.x] = (int) threadIdx.x < a.k && c_ptr != 0ull;
         s_w[threadIdx.x] = c_w;
@@ -537,7 +676,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
                 for (int i = 4; i < 8; ++i) acc[i] = 0.0f;   // an odd number of quads: the last batch's second half is empty
             }
             float v = reduce8_half(acc, lane);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             const int rr = r + ((lane >> 2) & 7);
             if ((lane & 35) == 0 && (ROWS % 8 == 0 || rr < ROWS)) part[wave][rr] = v;
         }

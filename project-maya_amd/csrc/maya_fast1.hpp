@@ -220,7 +220,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq1s_pos_kernel(maya_moe_args 
                 quad1_values<4>(cur, grid, y, sy, dy8, acc);
             }
             float v = reduce8_half(acc, lane);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
         }
     }
@@ -449,7 +449,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq1m_pos_kernel(maya_moe_args 
                 quadm_values<4>(cur, grid, y, sy8, sh, dy8, acc);
             }
             float v = reduce8_half(acc, lane);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
         }
     }

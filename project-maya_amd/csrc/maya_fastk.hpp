@@ -213,7 +213,7 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
                 asm volatile("" : "+v"(acc[i]));
             }
             float v = reduce8_half(acc, lane);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             if ((lane & 35) == 0) part[wave][(lane >> 2) & 7] = v;
         } else
 #pragma unroll 1
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(512, MINW) void down_q4k_pos_kernel(maya_moe_args a
                 asm volatile("" : "+v"(acc[i]));
             }
             float v = reduce8_half(acc, lane);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             if ((lane & 35) == 0) part[wave][r + ((lane >> 2) & 7)] = v;
         }
     }

@@ -138,7 +138,7 @@ __global__ __launch_bounds__(512) void down_q80_pos_kernel(maya_moe_args a, int 
                 q80_values<NT>(qa, qb, db, y, dx, acc, rr * NT);
             }
             float v = reduce8_half(acc, lane0);
-            v += __shfl_xor(v, 32, kWave);
+            v = add_other_half(v);
             if ((lane0 & 35) == 0) {
                 const int i = (lane0 >> 2) & 7, rr = i / NT, tk = i % NT;
                 if (ents[tk] >= 0 && r0 + r + rr < n_embd) a.part[(size_t) ents[tk] * n_embd + r0 + r + rr] = v;

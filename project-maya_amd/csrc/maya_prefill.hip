@@ -412,7 +412,7 @@ typedef _Float16 pf_v2h __attribute__((ext_vector_type(2)));
 // sub-block's 32 values of activation row ln (A operand, from LDS) and of weight row ln (B operand, decoded in
 // registers), and 16 outputs: weight row ln against the rows 8 b + 4 kh + r (b, r = 0..3) of the 32.  These
 // instructions take 32 cycles, and the vector ALU issues about four instructions under each of them; the 16-cycle
-// 16x16 forms leave it no slot (measured: project-maya_amd/csrc/maya_probe.hip, section 5), which is what bounds a
+// 16x16 forms leave it no slot (measured with a microbenchmark of matrix instructions followed by vector instructions), which is what bounds a
 // kernel that has as many vector instructions as this one.
 template <bool GU, int NM>
 __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b1, uint8_t* b2, int ex, int row0, int nrows) {

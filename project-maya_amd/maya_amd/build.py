@@ -1,5 +1,4 @@
-"""Compiles the HIP sources into project-maya_amd/libmaya_moe.so for gfx950 (hipcc cross-compiles without a GPU), and the
-stand-alone microbenchmark program project-maya_amd/maya_probe beside it."""
+"""Compiles the HIP sources into project-maya_amd/libmaya_moe.so for gfx950 (hipcc cross-compiles without a GPU)."""
 import os
 import subprocess
 import sys
@@ -7,7 +6,6 @@ import sys
 PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmaya_moe.so")
-PROBE = os.path.join(PKG, "maya_probe")
 SOURCES = ["maya_kernels.hip", "maya_exl3.hip", "maya_prefill.hip"]
 # -packed-fp32-ops off: the compiler then forms no v_pk_*_f32 from scalar float code
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-ffp-contract=off",
@@ -26,7 +24,6 @@ def _run(cmd, verbose):
 def build(verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     _run([hipcc] + FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES], verbose)
-    _run([hipcc] + [f for f in FLAGS if f not in ("-shared", "-fPIC")] + ["-o", PROBE, os.path.join(CSRC, "maya_probe.hip")], verbose)
     return LIB
 
 
