@@ -14,7 +14,6 @@
 
 namespace maya {
 
-
 typedef const __attribute__((address_space(1))) uint8_t* gptr8;
 typedef const __attribute__((address_space(1))) uint16_t* gptr16;
 typedef const __attribute__((address_space(1))) uint32_t __attribute__((aligned(2))) * gptr32_a2;

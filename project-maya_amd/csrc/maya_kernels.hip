@@ -471,8 +471,8 @@ __global__ __launch_bounds__(256) void quant_i8x32_kernel(const void* __restrict
 struct alignas(16) RouterLds {
     double ex[MAYA_MAX_EXPERTS];
     float p[MAYA_MAX_EXPERTS];
-    float rv[4];
-    int ri[4];
+    float rv[8];
+    int ri[8];
     double sum;
     float w[MAYA_MAX_K];
     int id[MAYA_MAX_K];
@@ -617,20 +617,24 @@ __device__ __forceinline__ void topk_by_keys(const unsigned long long* key, int 
     }
 }
 
-// 256 threads; on return sm.id / sm.w hold the token's k experts and renormalised weights
+// NTH threads (256, or a workgroup of 512 with up to 256 experts); on return sm.id / sm.w hold the token's k experts and
+// renormalised weights
+template <int NTH = 256>
 __device__ __forceinline__ void route_token(const float* __restrict__ l, int n_expert, int k, RouterLds& sm) {
     const int tid = threadIdx.x;
     float mx = -INFINITY;
-    for (int e = tid; e < n_expert; e += 256) mx = fmaxf(mx, l[e]);
+    for (int e = tid; e < n_expert; e += NTH) mx = fmaxf(mx, l[e]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
     if ((tid & 63) == 0) sm.rv[tid >> 6] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(sm.rv[0], sm.rv[1]), fmaxf(sm.rv[2], sm.rv[3]));
+    mx = sm.rv[0];
+#pragma unroll
+    for (int w = 1; w < NTH / 64; ++w) mx = fmaxf(mx, sm.rv[w]);   // (the maximum is exact in any order)
     __syncthreads();
-    for (int e = tid; e < n_expert; e += 256) sm.ex[e] = exp((double) l[e] - (double) mx);
+    for (int e = tid; e < n_expert; e += NTH) sm.ex[e] = exp((double) l[e] - (double) mx);
     __syncthreads();
-    if (n_expert <= 256) {
+    if (n_expert <= 256 || NTH != 256) {   // (wider workgroups are only given up to 256 experts)
         if (tid < 64) route_narrow(n_expert, k, sm);
         __syncthreads();
         return;
@@ -733,12 +737,13 @@ __device__ __forceinline__ void sigmoid_narrow(int n_expert, int k, const Router
     }
     if (lane < k) sm.id[lane] = my_id;
 }
-// 256 threads; on return sm.id / sm.w hold the token's k experts and weights
+// NTH threads (as route_token); on return sm.id / sm.w hold the token's k experts and weights
+template <int NTH = 256>
 __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l, int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
     const int tid = threadIdx.x;
     float* sel = (float*) sm.ex;
     int bad = 0;
-    for (int e = tid; e < n_expert; e += 256) {
+    for (int e = tid; e < n_expert; e += NTH) {
         const float le = l[e];
         const float p = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-le)));
         const float sc = r.bias ? __fadd_rn(p, r.bias[e]) : p;
@@ -749,7 +754,7 @@ __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l,
     // a row with a non-finite logit or score is refused: no routes (the engine's routers,
     // src/kernels/cuda/glm_batch.cu:2077-2092, glm_fast.cu:4040); it is still ranked below, its picks unused
     bad = __syncthreads_or(bad);
-    if (n_expert <= 256) {
+    if (n_expert <= 256 || NTH != 256) {
         if (tid < 64) sigmoid_narrow(n_expert, k, r, sm);
     } else {
         // (the scores' ordered bits, offset to unsigned, above the complemented index; the keys take the scores' place)
@@ -780,9 +785,10 @@ __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ l,
     }
     __syncthreads();
 }
+template <int NTH = 256>
 __device__ __forceinline__ void route_any(const float* __restrict__ l, int n_expert, int k, const RouterSpec& r, RouterLds& sm) {
-    if (r.kind == MAYA_ROUTER_SIGMOID) route_token_sigmoid(l, n_expert, k, r, sm);
-    else route_token(l, n_expert, k, sm);
+    if (r.kind == MAYA_ROUTER_SIGMOID) route_token_sigmoid<NTH>(l, n_expert, k, r, sm);
+    else route_token<NTH>(l, n_expert, k, sm);
 }
 
 __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec r,

@@ -7,9 +7,12 @@ PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libmaya_moe.so")
 SOURCES = ["maya_kernels.hip", "maya_exl3.hip", "maya_prefill.hip"]
-# -packed-fp32-ops off: the compiler then forms no v_pk_*_f32 from scalar float code
+# -packed-fp32-ops off: the compiler then forms no v_pk_*_f32 from scalar float code.  amdgpu-kernarg-preload-count: the
+# first 16 dwords of a kernel's arguments arrive in scalar registers with the dispatch instead of by a load (one memory
+# round trip less at the start of every kernel: the decode layer 37.55 -> 37.15 us).
 FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-ffp-contract=off",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-kernarg-preload-count=16",
+         "-Wall", "-Wno-unused-function"]
 
 
 def _run(cmd, verbose):
