@@ -7,7 +7,8 @@ state, fused dequant gate/up GLU mat-vec over the 8 routed IQ2_S experts, Q8_K r
 combine.  All 256 experts (3.6 GB) are resident in HBM; consecutive steps route to disjoint expert sets (32 sets of 8),
 so no step re-reads weights that an earlier step left in the on-die caches.  The K steps are one HIP graph (the
 reference's timing method, tests/hip/expert_kernel_bench.cpp:136-172): untimed replays until two in a row agree within
-1 %, then 7 timed replays bracketed by device synchronisations, the median.
+1 %, then 7 timed samples - each the graph replayed back to back (at least 256 steps and 10 ms of GPU work) between two
+HIP events on the launch stream - the median; the figure does not move with --steps.
 
 value = algorithmic HBM bytes of a step (weights of the 8 routed experts + logits + x + out) / time per step, GB/s.
 roofline = the dominant kernel (gate/up: two thirds of the bytes): its algorithmic bytes / its average launch duration
@@ -254,8 +255,10 @@ def decode_iq2s(args, np, torch, lib, L, info):
                                "rotate over the steps",
                    "n_embd": N_EMBD, "n_ff": N_FF, "n_expert": N_EXPERT, "top_k": TOP_K, "tokens": 1,
                    "weight_bytes_per_step": w_bytes, "algorithmic_bytes_per_step": bytes_step,
-                   "timed_as": ("eager launches" if args.no_graph else "one HIP graph of the K steps") +
-                               ", median of %d replays after the clocks settled" % bw.ROUNDS, "device": info},
+                   "timed_as": ("eager launches, median of %d rounds" % bw.ROUNDS if args.no_graph else
+                                "one HIP graph of the K steps, replayed back to back (>= 256 steps and >= 10 ms a sample) between "
+                                "two HIP events on the launch stream, median of %d samples after the clocks settled" % bw.ROUNDS),
+                   "device": info},
         "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_pos_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
                      "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_s * 1e6, 3),
@@ -273,17 +276,64 @@ def decode_iq2s(args, np, torch, lib, L, info):
 
 
 def parity_of(np, torch, r):
-    """The CPU path's expert on a workload's own bytes (workloads that hand back a `_parity` record)."""
+    """The CPU path on a workload's own bytes (workloads hand back a `_parity` record): one expert, or the rows of the
+    sampled tokens of one step - router ids of every token exact, each sampled row's relative L2 against the checker's layer
+    on the routed experts' blobs pulled to the host.  Returns (worst relative L2, bar, ids exact or None)."""
     import oracle_py
     p = r.pop("_parity", None)
     if p is None:
-        return None
-    blob = p["blob"].cpu().numpy()
-    gr = oracle_py.row_bytes(p["type"], p["n_embd"])
-    up_off, down_off = gr * p["n_ff"], 2 * gr * p["n_ff"]
-    want = oracle_py.expert(p["type"], p["type"], blob, blob[up_off:], blob[down_off:], p["n_embd"], p["n_ff"],
-                            p["x"].to(torch.float32).cpu().numpy())
-    return rel_l2(np, p["out"].cpu().numpy(), want)
+        return None, PARITY_BAR, None
+    if p["kind"] == "expert":
+        blob = p["blob"].cpu().numpy()
+        gr = oracle_py.row_bytes(p["type"], p["n_embd"])
+        up_off, down_off = gr * p["n_ff"], 2 * gr * p["n_ff"]
+        want = oracle_py.expert(p["type"], p["type"], blob, blob[up_off:], blob[down_off:], p["n_embd"], p["n_ff"],
+                                p["x"].to(torch.float32).cpu().numpy())
+        return rel_l2(np, p["out"].cpu().numpy(), want), PARITY_BAR, None
+    tests = os.path.join(ROOT, "tests")   # the parity helpers of the tests: the checker's layer on the host
+    if tests not in sys.path:
+        sys.path.insert(0, tests)
+    import gpu_util
+    ids, w = oracle_py.router_topk(p["logits"], p["k"])
+    ids_ok = bool(np.array_equal(ids, p["ids"]))
+    toks = p["tokens"]
+
+    class Blobs:   # an expert's blob comes to the host when the checker asks for it
+        def __init__(self):
+            self.have = {}
+
+        def __getitem__(self, e):
+            if e not in self.have:
+                self.have[e] = p["blob_of"](e)
+            return self.have[e]
+
+    blobs = Blobs()
+    worst = 0.0
+    if p["kind"] == "layer":
+        sh = None
+        if p.get("shared"):
+            st, sblob, sl = p["shared"]
+            sh = (st, sblob(), sl)
+        for t in toks:
+            _, _, want = gpu_util.oracle_layer(oracle_py, p["gate_type"], p["down_type"], blobs, p["k"], p["n_embd"], p["n_ff"],
+                                               p["logits"][t:t + 1], p["x"][t:t + 1])
+            want = want[0]
+            if sh is not None:
+                st, sb, sl = sh
+                want = want + oracle_py.expert(st, st, sb, sb[sl.up_off:], sb[sl.down_off:], p["n_embd"], p["n_ff"], p["x"][t:t + 1])[0]
+            worst = max(worst, rel_l2(np, p["out"][t], want))
+    else:
+        from maya_amd import exl3
+        experts = {}
+        for t in toks:
+            for e in ids[t]:
+                if int(e) not in experts:
+                    experts[int(e)] = gpu_util.HostExpert(exl3, oracle_py, p["layout"], blobs[int(e)])
+        for t in toks:
+            parts = [experts[int(e)].part(experts[int(e)].h(p["x"][t], 0.0)) for e in ids[t]]
+            want = oracle_py.combine(np.stack(parts), np.ascontiguousarray(w[t], dtype=np.float32))
+            worst = max(worst, rel_l2(np, p["out"][t], want))
+    return worst, p.get("tol", PARITY_BAR), ids_ok
 
 
 def main():
@@ -327,15 +377,15 @@ def main():
             sys.exit("bench.py: unknown workload %r" % args.workload)
         r = workloads.WORKLOADS[args.workload](args.steps, args.warmup)
         r["config"]["device"] = info
-        err = None if args.no_cpu else parity_of(np, torch, r)
+        err, bar, ids_ok = (None, PARITY_BAR, None) if args.no_cpu else parity_of(np, torch, r)
         r.pop("_parity", None)
         line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
                 "warmup": args.warmup, "ms_per_step": round(r["ms_per_step"], 6), "higher_is_better": True, "scaling": "weak",
                 "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"], "roofline": r["roofline"],
-                "cpu_baseline": None, "parity_rel_l2_vs_cpu_path": err}
+                "cpu_baseline": None, "parity_rel_l2_vs_cpu_path": err, "parity_bar": bar, "parity_ids_exact": ids_ok}
         print(json.dumps(line))
-        if err is not None and not err <= PARITY_BAR:
-            print("bench.py: parity failed: relative L2 %g against the CPU path" % err, file=sys.stderr)
+        if (err is not None and not err <= bar) or ids_ok is False:
+            print("bench.py: parity failed: relative L2 %s against the CPU path (bar %g), ids exact %s" % (err, bar, ids_ok), file=sys.stderr)
             sys.exit(3)
         return
 
@@ -345,6 +395,7 @@ def main():
         # gives the same numbers alone
         ksteps = max(4, min(16, args.steps))
         r = workloads.prefill_q4k(ksteps, 2)
+        r.pop("_parity", None)
         line["prefill"] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "ms_per_chunk": round(r["ms_per_step"], 4),
                            "steps": ksteps, "pct_of_int8_peak": round(100.0 * r["value"] * 1e12 / workloads.INT8_PEAK, 2),
                            "pct_of_hbm_peak": r["config"]["pct_of_hbm_peak"], "weight_gbps": r["config"]["weight_gbps"],

@@ -52,3 +52,50 @@ def oracle_layer(oracle, gate_type, down_type, blobs, k, n_embd, n_ff, logits, x
         if parts:
             out[t] = oracle.combine(np.stack(parts), np.array(ws, dtype=np.float32))
     return ids, w, out
+
+
+# ---- the EXL3 layer on the host (the checker decodes each matrix once an expert)
+
+def swiglu(g, u, limit):
+    g = g.astype(np.float32)
+    u = u.astype(np.float32)
+    if limit > 0 and np.isfinite(limit):
+        g = np.minimum(g, np.float32(limit))
+        u = np.clip(u, -np.float32(limit), np.float32(limit))
+    return (g / (np.float32(1) + np.exp(-g)) * u).astype(np.float32)
+
+
+class HostExpert:
+    def __init__(self, ex, oracle, l, blob):
+        self.m = []
+        for r in range(3):
+            k, n = ex.matrix_of(l, r)
+            tr, suh, svh = ex.parts_of(l, blob, r)
+            self.m.append((oracle.exl3_inner(tr, k, n, l.k2[r], l.cb), suh, svh))
+        self.oracle = oracle
+
+    def h(self, x, limit):
+        g = self.oracle.exl3_mv(*self.m[0], x)
+        u = self.oracle.exl3_mv(*self.m[1], x)
+        return swiglu(g, u, limit)
+
+    def part(self, h):
+        return self.oracle.exl3_mv(*self.m[2], h)
+
+
+def host_layer(oracle, experts, ids, w, x, limit, skip=()):
+    nt, k = ids.shape
+    hs = np.zeros((nt * k, experts[0].m[0][0].shape[1]), dtype=np.float32)
+    out = np.zeros((nt, x.shape[1]), dtype=np.float32)
+    for t in range(nt):
+        parts, ws = [], []
+        for i in range(k):
+            e = int(ids[t, i])
+            if e in skip:
+                continue
+            hs[t * k + i] = experts[e].h(x[t], limit)
+            parts.append(experts[e].part(hs[t * k + i]))
+            ws.append(w[t, i])
+        if parts:
+            out[t] = oracle.combine(np.stack(parts), np.array(ws, dtype=np.float32))
+    return out, hs

@@ -10,7 +10,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 torch = pytest.importorskip("torch")
-from gpu_util import rel_l2  # noqa: E402
+from gpu_util import HostExpert, host_layer, swiglu, rel_l2  # noqa: E402
 from test_oracle_exl3 import read_exh1, FILES  # noqa: E402
 
 TOL = 1e-3
@@ -49,51 +49,6 @@ def test_unsupported_k2_is_refused(ex):
     assert ex.supported(6, 2) and ex.supported(3, 2) and not ex.supported(3, 0) and not ex.supported(18, 2)
     with pytest.raises(MayaError):
         ex.reconstruct_inner(torch.zeros(64, dtype=torch.int32, device="cuda"), 16, 16, 9, 0)
-
-
-def swiglu(g, u, limit):
-    g = g.astype(np.float32)
-    u = u.astype(np.float32)
-    if limit > 0 and np.isfinite(limit):
-        g = np.minimum(g, np.float32(limit))
-        u = np.clip(u, -np.float32(limit), np.float32(limit))
-    return (g / (np.float32(1) + np.exp(-g)) * u).astype(np.float32)
-
-
-class HostExpert:
-    def __init__(self, ex, oracle, l, blob):
-        self.m = []
-        for r in range(3):
-            k, n = ex.matrix_of(l, r)
-            tr, suh, svh = ex.parts_of(l, blob, r)
-            self.m.append((oracle.exl3_inner(tr, k, n, l.k2[r], l.cb), suh, svh))
-        self.oracle = oracle
-
-    def h(self, x, limit):
-        g = self.oracle.exl3_mv(*self.m[0], x)
-        u = self.oracle.exl3_mv(*self.m[1], x)
-        return swiglu(g, u, limit)
-
-    def part(self, h):
-        return self.oracle.exl3_mv(*self.m[2], h)
-
-
-def host_layer(oracle, experts, ids, w, x, limit, skip=()):
-    nt, k = ids.shape
-    hs = np.zeros((nt * k, experts[0].m[0][0].shape[1]), dtype=np.float32)
-    out = np.zeros((nt, x.shape[1]), dtype=np.float32)
-    for t in range(nt):
-        parts, ws = [], []
-        for i in range(k):
-            e = int(ids[t, i])
-            if e in skip:
-                continue
-            hs[t * k + i] = experts[e].h(x[t], limit)
-            parts.append(experts[e].part(hs[t * k + i]))
-            ws.append(w[t, i])
-        if parts:
-            out[t] = oracle.combine(np.stack(parts), np.array(ws, dtype=np.float32))
-    return out, hs
 
 
 CASES = [
