@@ -359,10 +359,10 @@ def _prefill(K, W, gt, dt, what, types):
                          "algorithmic_ops_per_launch": ops_gu, "avg_launch_us": round(sec_gu * 1e6, 1)}}
 
 
-def exl3_verify(K, W, k2=6):
-    """configs[4]: 160 EXL3 experts (3 bits a weight: k2 = 6, mul1 codebook), top-8, hidden 6144, intermediate 1536, a
-    4-token verify window; 8 logit sets rotate.  (k2 = 8, 10: the same layer at 4 and 5 bits a weight.)"""
-    E, FF, NE, TK, T = 6144, 1536, 160, 8, 4
+def exl3_pool(E, FF, NE, k2):
+    """NE EXL3 experts (mul1 codebook, k2 / 2 bits a weight) on the device: random trellis words (every pattern is a valid
+    encoding, tests/exl3_test.cu:112-116), sign vectors suh and scaled sign vectors svh.  Returns the layout, a blob's bytes,
+    the pool, its [NE, stride] view and the address table."""
     l, bb = exl3.make_layout(E, FF, k2, exl3.CB_MUL1)
     stride = (bb + 255) & ~255
     pool = random_blocks(NE * stride, 256, {}, 13)
@@ -377,6 +377,14 @@ def exl3_verify(K, W, k2=6):
         view[:, l.suh[r]:l.suh[r] + 2 * k] = suh.view(torch.uint8).view(NE, -1)
         view[:, l.svh[r]:l.svh[r] + 2 * n] = svh.view(torch.uint8).view(NE, -1)
     table = torch.tensor([pool.data_ptr() + e * stride for e in range(NE)], dtype=torch.int64, device="cuda")
+    return l, bb, pool, view, table
+
+
+def exl3_verify(K, W, k2=6):
+    """configs[4]: 160 EXL3 experts (3 bits a weight: k2 = 6, mul1 codebook), top-8, hidden 6144, intermediate 1536, a
+    4-token verify window; 8 logit sets rotate.  (k2 = 8, 10: the same layer at 4 and 5 bits a weight.)"""
+    E, FF, NE, TK, T = 6144, 1536, 160, 8, 4
+    l, bb, pool, view, table = exl3_pool(E, FF, NE, k2)
     layer = exl3.Exl3Layer(l, NE, TK, max_tokens=T)
     rng = np.random.default_rng(15)
     n_sets = 8

@@ -46,6 +46,7 @@ extern "C" {
 #define MAYA_E_SHAPE 2       /* a size outside what the kernels assume (not whole blocks, too many tokens, ...) */
 #define MAYA_E_ARG 3         /* a null pointer or a workspace that is too small */
 #define MAYA_E_NOGPU 4       /* no gfx950 device / the library's device code is not loadable */
+#define MAYA_E_BUSY 5        /* maya_moe_layer_decode_shared: the device's side stream is inside another stream's capture */
 
 #define MAYA_MAX_K 16          /* experts per token */
 #define MAYA_MAX_TOKENS 16     /* tokens of one decode / verify-window call */
@@ -326,8 +327,12 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
  *   where the down kernel rounds h itself) / part buffers, `add` the layer's residual or NULL, `out` its own
  *   [n_tokens][n_embd] buffer (not the layer's out).
  * The fork and the join are event records and waits, so the call may be captured in a HIP graph (maya_init() first).
- * Calls on one device are serialised on the host by a lock; whatever fails, `stream` has joined the second stream again
- * when the call returns. */
+ * Every refusal of the stages (status > 0) is found before the fork: such a call has launched nothing on either stream.
+ * Calls on one device are serialised on the host by a lock.  The device has ONE such second stream: while `stream` is being
+ * captured that second stream belongs to the capture until hipStreamEndCapture, and a call from any other stream (eager,
+ * or inside another capture) in between is refused with MAYA_E_BUSY and launches nothing - the open capture is not
+ * disturbed and may call again.  After a HIP error (status < 0) `stream` has joined the second stream again when the
+ * call returns. */
 int maya_moe_layer_decode_shared(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
                                  const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
                                  float limit, const maya_moe_args* shared, int32_t* ids, float* weights, float* out,

@@ -1726,6 +1726,61 @@ int launch_down_q80_pos(const maya_moe_args& a, hipStream_t s) {
 }
 
 // whether the gate/up (down) call is served entry by entry (no use for the groups of a window)
+// the shapes the IQ2_S streaming kernels take (what try_gate_up_iq2s_1tok / try_down_iq2s_1tok launch on)
+static bool gate_up_iq2s_fast_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (l.packing == MAYA_PACK_STREAM) return l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 && l.n_embd >= 2048 && l.n_embd <= 8192;
+    return fast_1tok(a) && l.n_embd % 1024 == 0 && l.n_embd <= 8192 && l.n_ff % 32 == 0;
+}
+static bool down_iq2s_fast_ok(const maya_moe_args& a) {
+    const maya_moe_layout& l = a.layout;
+    if (a.k > 8) return false;
+    if (l.packing == MAYA_PACK_STREAM) return down_pos_nff_ok(l.n_ff) && l.n_embd % 16 == 0;
+    return fast_1tok(a) && l.n_ff % 1024 == 0 && l.n_ff <= 4096 && l.n_embd % 14 == 0;
+}
+// Everything maya_moe_gate_up / maya_moe_down / maya_quant_act refuse (status > 0), asked without launching anything:
+// the calls themselves ask first, and a caller that forks a stream before them (maya_moe_layer_decode_shared) asks before
+// the fork, so that its own "> 0: nothing launched" holds.
+static int gate_up_refusal(const maya_moe_args* a, const DeviceState& st) {
+    if (const int rc = check_args(a)) return rc;
+    if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
+    const int tg = a->layout.gate_type, tu = a->layout.up_type;
+    const bool pair = (tg == tu) || (tg == kIQ2_S && tu == kIQ1_M) || (tg == kIQ1_M && tu == kIQ2_S) || (tg == kIQ2_S && tu == kQ4_K) ||
+                      (tg == kIQ1_S && tu == kIQ1_M) || (tg == kIQ1_M && tu == kIQ1_S);
+    if (!pair) return fail(MAYA_E_UNSUPPORTED, "gate_up: no kernel for gate type %d with up type %d", tg, tu);
+    const bool pos = (tg == kIQ2_S && tu == kIQ2_S && gate_up_iq2s_fast_ok(*a)) || gate_up_q4k_pos_ok(*a) || gate_up_iq1s_pos_ok(*a) ||
+                     gate_up_q80_pos_ok(*a);
+    if (!pos) {   // the general kernel: its activation tile and codebooks must fit the device's LDS
+        const int nt = a->grp_ptr ? (a->n_tokens >= 4 ? 4 : a->n_tokens >= 2 ? 2 : 1) : 1;
+        const int cbw = codebook_words(tg) + (codebook_words(tg) == codebook_words(tu) ? 0 : codebook_words(tu));
+        const size_t lds = (size_t) cbw * 4 + act_lds_bytes(a->layout.n_embd, nt);
+        if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "gate/up needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    }
+    return MAYA_OK;
+}
+static int quant_act_refusal(int act_type, const void* x, int x_dtype, int rows, int64_t k, const maya_act& out) {
+    if (!type_ok(act_type)) return fail(MAYA_E_UNSUPPORTED, "quant_act: weight type %d", act_type);
+    if (x_dtype < 0 || x_dtype > 2) return fail(MAYA_E_UNSUPPORTED, "quant_act: dtype %d", x_dtype);
+    if (!x || !out.q || !out.d || !out.bsums) return fail(MAYA_E_ARG, "quant_act: null pointer");
+    if (rows <= 0 || rows > 65535 || k <= 0 || k % 256) return fail(MAYA_E_SHAPE, "quant_act: rows %d k %lld", rows, (long long) k);
+    return MAYA_OK;
+}
+
+static bool down_self_rounding(const maya_moe_args& a) { return !a.hq.q && !a.hq.d && !a.hq.bsums && a.h && a.out && down_rounds_h(a); }
+static int down_refusal(const maya_moe_args* a, const DeviceState& st) {
+    if (const int rc = check_args(a)) return rc;
+    if (down_self_rounding(*a)) return MAYA_OK;
+    if (!a->hq.q || !a->hq.d || !a->hq.bsums || !a->part || !a->out) return fail(MAYA_E_ARG, "down: null activation, part or out");
+    const bool pos = (a->layout.down_type == kIQ2_S && down_iq2s_fast_ok(*a)) || down_q4k_pos_ok(*a) || down_iq1s_pos_ok(*a) ||
+                     down_q80_pos_ok(*a);
+    if (!pos) {
+        const int nt = a->grp_ptr ? (a->n_tokens >= 4 ? 4 : a->n_tokens >= 2 ? 2 : 1) : 1;
+        const size_t lds = (size_t) codebook_words(a->layout.down_type) * 4 + act_lds_bytes(a->layout.n_ff, nt);
+        if (lds > (size_t) st.lds_limit) return fail(MAYA_E_SHAPE, "down needs %zu bytes of LDS, the device gives %d", lds, st.lds_limit);
+    }
+    return MAYA_OK;
+}
+
 bool gate_up_by_entries(const maya_moe_args& a) {
     const maya_moe_layout& l = a.layout;
     if (gate_up_q4k_pos_ok(a) || gate_up_iq1s_pos_ok(a)) return true;
@@ -1903,10 +1958,7 @@ int maya_quant_act(int act_type, const void* x, int x_dtype, int64_t x_stride, i
                    void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (!type_ok(act_type)) return fail(MAYA_E_UNSUPPORTED, "quant_act: weight type %d", act_type);
-    if (x_dtype < 0 || x_dtype > 2) return fail(MAYA_E_UNSUPPORTED, "quant_act: dtype %d", x_dtype);
-    if (!x || !out.q || !out.d || !out.bsums) return fail(MAYA_E_ARG, "quant_act: null pointer");
-    if (rows <= 0 || rows > 65535 || k <= 0 || k % 256) return fail(MAYA_E_SHAPE, "quant_act: rows %d k %lld", rows, (long long) k);
+    if (const int rc = quant_act_refusal(act_type, x, x_dtype, rows, k, out)) return rc;
     if (x_stride == 0) x_stride = k;
     const dim3 grid((unsigned) (k / 256), (unsigned) rows);
     hipStream_t s = as_stream(stream);
@@ -2091,8 +2143,7 @@ int maya_moe_group(const uint64_t* plan_ptr, int n_entries, uint64_t* grp_ptr, i
 int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (const int rc = check_args(a)) return rc;
-    if (!a->x.q || !a->x.d || !a->x.bsums || !a->h) return fail(MAYA_E_ARG, "gate_up: null activation or h");
+    if (const int rc = gate_up_refusal(a, *st)) return rc;
     hipStream_t s = as_stream(stream);
     const int tg = a->layout.gate_type, tu = a->layout.up_type;
     if (tg == kIQ2_S && tu == kIQ2_S) {
@@ -2122,8 +2173,8 @@ int maya_moe_down_rounds_h(const maya_moe_args* a) { return a && down_rounds_h(*
 int maya_moe_down(const maya_moe_args* a, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
-    if (const int rc = check_args(a)) return rc;
-    if (!a->hq.q && !a->hq.d && !a->hq.bsums && a->h && a->out && down_rounds_h(*a)) {
+    if (const int rc = down_refusal(a, *st)) return rc;
+    if (down_self_rounding(*a)) {
         int rc = 0;   // the kernel rounds h itself
         if (a->layout.down_type == kQ4_K) return launch_down_q4k_pos(*a, as_stream(stream));
         if (a->layout.down_type == kIQ1_S || a->layout.down_type == kIQ1_M) return launch_down_iq1s_pos(*a, *st, as_stream(stream));
@@ -2315,24 +2366,24 @@ int maya_moe_layer_decode(const maya_moe_layout* l, const uint64_t* expert_table
 
 // The layer's launches.  `join`: an event the down launch waits for (the shared expert's output, which `add` then points
 // at), *joined set once the stream waits for it.
-static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
-                             const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
-                             int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream,
-                             hipEvent_t join, bool* joined) {
-    DeviceState* st;
-    if (const int rc = current_state(&st)) return rc;
+// The routed layer's refusals (status > 0) and its stage arguments over the carved workspace, without launching anything.
+static int layer_setup(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                       const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,
+                       float* weights, float* out, void* workspace, size_t workspace_bytes, const DeviceState& st, RouterSpec& rs,
+                       LayerWs& w, maya_moe_args& a) {
     if (!l) return fail(MAYA_E_ARG, "layer_decode: null layout");
-    RouterSpec rs;
     if (!router_spec(router, rs)) return fail(MAYA_E_UNSUPPORTED, "layer_decode: router kind %d / normalisation %d", router->kind, router->norm);
     if (const int rc = check_layout(*l)) return rc;
     if (!expert_table || !x || !ids || !weights || !out || !workspace) return fail(MAYA_E_ARG, "layer_decode: null pointer");
     if (n_tokens < 1 || n_tokens > MAYA_MAX_TOKENS || k < 1 || k > MAYA_MAX_K)
         return fail(MAYA_E_SHAPE, "layer_decode: n_tokens %d / k %d", n_tokens, k);
     if (((uintptr_t) workspace & 255) != 0) return fail(MAYA_E_ARG, "layer_decode: workspace not 256-byte aligned");
-    const LayerWs w = carve(*l, n_tokens, k, (uint8_t*) workspace);
+    w = carve(*l, n_tokens, k, (uint8_t*) workspace);
     if (workspace_bytes < w.bytes) return fail(MAYA_E_ARG, "layer_decode: workspace %zu < %zu bytes", workspace_bytes, w.bytes);
-    int rc;
-    maya_moe_args a{};
+    if (logits && k > n_expert) return fail(MAYA_E_SHAPE, "layer_decode: k %d > n_expert %d", k, n_expert);
+    if (logits && n_expert > MAYA_MAX_EXPERTS) return fail(MAYA_E_SHAPE, "layer_decode: %d experts, the routers take %d", n_expert, MAYA_MAX_EXPERTS);
+    if (const int rc = quant_act_refusal(l->gate_type, x, x_dtype, n_tokens, l->n_embd, w.x)) return rc;
+    a = maya_moe_args{};
     a.layout = *l;
     a.n_tokens = n_tokens;
     a.k = k;
@@ -2345,6 +2396,31 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
     a.part = w.part;
     a.add = add;
     a.out = out;
+    // (the stage calls' own refusals, on the arguments they will get: grouped beyond one token unless both stages take
+    // the entries one by one)
+    maya_moe_args probe = a;
+    if (n_tokens > 1) {
+        probe.grp_ent = w.grp_ent;
+        if (!(gate_up_by_entries(a) && down_by_entries(a))) probe.grp_ptr = w.grp_ptr, probe.grp_start = w.grp_start, probe.n_groups = w.n_groups;
+    }
+    if (const int rc = gate_up_refusal(&probe, st)) return rc;
+    if (down_rounds_h(probe)) probe.hq = maya_act{nullptr, nullptr, nullptr}, probe.part = nullptr;
+    return down_refusal(&probe, st);
+}
+
+static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                             const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                             int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream,
+                             hipEvent_t join, bool* joined) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    RouterSpec rs;
+    LayerWs w;
+    maya_moe_args a;
+    if (const int rc0 = layer_setup(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out,
+                                    workspace, workspace_bytes, *st, rs, w, a))
+        return rc0;
+    int rc;
     bool grouped = false;
     if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
         n_tokens <= kWindowHeadTokens && maya_moe_route_window_ok(router, n_tokens, n_expert, k)) {
@@ -2362,7 +2438,6 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
         // one launch: route, plan, Q8_K of x
         const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
         hipStream_t s = as_stream(stream);
-        if (k > n_expert) return fail(MAYA_E_SHAPE, "layer_decode: k %d > n_expert %d", k, n_expert);
         switch (x_dtype) {
             case MAYA_DT_F32: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_F32>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x); break;
             case MAYA_DT_BF16: hipLaunchKernelGGL(layer_head_kernel<MAYA_DT_BF16>, grid, dim3(256), 0, s, logits, n_expert, k, rs, expert_table, ids, weights, w.plan_ptr, x, (int64_t) l->n_embd, w.x); break;
@@ -2428,9 +2503,34 @@ int maya_moe_layer_decode_shared(const maya_moe_layout* l, const uint64_t* exper
     if (!shared->x.q || !shared->x.d || !shared->h || !shared->out || !shared->plan_ptr || !shared->plan_w)
         return fail(MAYA_E_ARG, "layer_decode_shared: the shared expert's arguments lack a buffer (x, h, out, plan)");
     if (shared->out == out) return fail(MAYA_E_ARG, "layer_decode_shared: the shared expert's out is the layer's out");
+    // Everything the stage calls below could refuse is asked BEFORE the fork, so that a status > 0 means nothing was launched
+    // on either stream.
+    if (const int rc = quant_act_refusal(shared->layout.gate_type, x, x_dtype, n_tokens, shared->layout.n_embd, shared->x)) return rc;
+    if (const int rc = gate_up_refusal(shared, *st)) return rc;
+    if (shared->hq.q)
+        if (const int rc = quant_act_refusal(shared->layout.down_type, shared->h, MAYA_DT_F32, n_tokens, shared->layout.n_ff, shared->hq)) return rc;
+    if (const int rc = down_refusal(shared, *st)) return rc;
+    {
+        RouterSpec rs;
+        LayerWs w;
+        maya_moe_args a;
+        if (const int rc = layer_setup(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, shared->out, ids, weights,
+                                       out, workspace, workspace_bytes, *st, rs, w, a))
+            return rc;
+    }
     // one call at a time a device: the side stream and its two events are the device's
     std::lock_guard<std::mutex> lock(st->side_mu);
     hipStream_t s = as_stream(stream);
+    {   // A side stream that an earlier call left inside a capture that has not ended belongs to that capture's graph until
+        // hipStreamEndCapture: work forked onto it from another stream (eager, or another capture) would land in the wrong
+        // graph or break the open capture.  The same capture calling again (a graph of several layers) is fine.
+        hipStreamCaptureStatus side_st = hipStreamCaptureStatusNone, mine_st = hipStreamCaptureStatusNone;
+        unsigned long long side_id = 0, mine_id = 0;
+        MAYA_HIP(hipStreamGetCaptureInfo(st->side, &side_st, &side_id));
+        MAYA_HIP(hipStreamGetCaptureInfo(s, &mine_st, &mine_id));
+        if (side_st != hipStreamCaptureStatusNone && !(mine_st == hipStreamCaptureStatusActive && mine_id == side_id))
+            return fail(MAYA_E_BUSY, "layer_decode_shared: the device's side stream is inside another stream's capture; end that capture first");
+    }
     MAYA_HIP(hipEventRecord(st->side_fork, s));
     MAYA_HIP(hipStreamWaitEvent(st->side, st->side_fork, 0));
     // the shared expert beside the routed experts' head and gate/up launches: quantize x, gate/up, quantize h, down + add

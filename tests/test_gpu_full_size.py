@@ -112,3 +112,28 @@ def test_prompt_chunk_512_tokens_256_q4k_experts(lib, oracle):
         assert rel_l2(out[t], want[0]) <= TOL, (t, rel_l2(out[t], want[0]))
         dec = one.forward(table, ld[t:t + 1].contiguous(), xd[t:t + 1].contiguous()).cpu().numpy()
         assert rel_l2(out[t], dec[0]) <= 1e-5, (t, rel_l2(out[t], dec[0]))
+
+
+def test_exl3_verify_window_160_experts(oracle):
+    """configs[4]: 160 EXL3 experts (3 bits a weight, mul1), hidden 6144, intermediate 1536, top-8, a 4-token window:
+    every token's ids, and the rows of sampled tokens against the checker's decode of the routed experts' own bytes."""
+    from maya_amd import exl3
+    from gpu_util import HostExpert
+    E4, FF4, NE4, T = 6144, 1536, 160, 4
+    l, bb, pool, view, table = workloads.exl3_pool(E4, FF4, NE4, 6)
+    layer = exl3.Exl3Layer(l, NE4, TK, max_tokens=T)
+    rng = np.random.default_rng(401)
+    logits = rng.standard_normal((T, NE4)).astype(np.float32)
+    x = rng.standard_normal((T, E4)).astype(np.float16).astype(np.float32)   # FP16 activations, handed over as F32
+    out = layer.forward(table, torch.from_numpy(logits).cuda(), torch.from_numpy(x).cuda()).cpu().numpy()
+    ids, w = oracle.router_topk(logits, TK)
+    assert np.array_equal(layer.ids[:T].cpu().numpy(), ids)
+    assert np.max(np.abs(layer.weights[:T].cpu().numpy() - w)) < 1e-5
+    experts = {}
+    for t in (0, 3):
+        for e in ids[t]:
+            if int(e) not in experts:
+                experts[int(e)] = HostExpert(exl3, oracle, l, view[int(e), :bb].cpu().numpy())
+        parts = [experts[int(e)].part(experts[int(e)].h(x[t], 0.0)) for e in ids[t]]
+        want = oracle.combine(np.stack(parts), np.ascontiguousarray(w[t], dtype=np.float32))
+        assert rel_l2(out[t], want) <= TOL, (t, rel_l2(out[t], want))

@@ -160,11 +160,15 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
     got = out.cpu().numpy()
     part_h = part.cpu().numpy()
     entry_row = want["entry_row"]
+    explained_ties = 0
     for t in range(n_tokens):
         err = rel_l2(got[t], want["out"][t])
         if err <= 1e-3:
             continue
+        # never at the real intermediate width (the n_ff = 2048 case above holds every token to 1e-3), and at most one
+        # token a toy case
         assert n_ff < 2048 and err <= 3e-3, (t, err)
+        explained_ties += 1
         sel = [j for j in range(k) if entry_row[t * k + j] >= 0]
         parts = []
         for j in sel:
@@ -174,6 +178,8 @@ def test_stages_and_layer_match_checker(pf, oracle, case):
             assert rel_l2(part_h[r], parts[-1]) <= 1e-5, (t, r)
         explained = oracle.combine(np.stack(parts), np.array([want["w"][t, j] for j in sel], dtype=np.float32))
         assert rel_l2(got[t], explained) <= 1e-5, (t, err)
+    print("tokens past 1e-3 explained by a Q8_K tie of h: %d of %d" % (explained_ties, n_tokens))
+    assert explained_ties <= 1, explained_ties
     assert torch.equal(out16, out.to(torch.bfloat16))
 
     # the one-call layer gives the same bits as the stages

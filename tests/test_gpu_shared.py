@@ -132,14 +132,57 @@ def test_refusals_leave_the_stream_usable(lib):
                                         float("inf"), C.byref(a), w["layer"].ids.data_ptr(), w["layer"].weights.data_ptr(),
                                         w["layer"].out.data_ptr(), w["layer"].ws.data_ptr(), w["layer"].ws_bytes, None)
     assert rc != 0 and b"tokens" in L.maya_last_error()
-    # a routed layer the kernels refuse AFTER the shared expert was launched (k above the number of experts): the call
-    # fails, the streams are joined, and the next call works
+    # a routed layer that is refused (k above the number of experts): asked before the fork, so the status is > 0, nothing
+    # was launched on either stream, and the next call works
     rc = L.maya_moe_layer_decode_shared(C.byref(w["layer"].layout), w["table"].data_ptr(), 1, TK, None, logits.data_ptr(), x.data_ptr(), 0, T,
                                         float("inf"), C.byref(w["dense"].args), w["layer"].ids.data_ptr(), w["layer"].weights.data_ptr(),
                                         w["layer"].out.data_ptr(), w["layer"].ws.data_ptr(), w["layer"].ws_bytes, None)
-    assert rc != 0
+    assert rc > 0 and b"n_expert" in L.maya_last_error()
     torch.cuda.synchronize()
     got = w["layer"].forward(w["table"], logits, x, shared=w["dense"]).clone()
     want = two_calls(w, logits, x, None, float("inf"))
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+def test_another_stream_is_refused_while_the_side_stream_is_inside_a_capture(lib):
+    """The device's one side stream belongs to an open capture until that capture ends: a call from another stream in between
+    gets MAYA_E_BUSY and launches nothing, the capture stays valid (the same capture may call again), and its graph replays
+    with the right bits."""
+    import ctypes as C
+    gt, dt, st, E, FF, NE, TK, T = IQ2_S, Q4_K, Q8_0, 4096, 2048, 16, 4, 2
+    w = build(lib, gt, dt, st, E, FF, NE, TK, T, 570)
+    logits, x, _ = inputs(E, NE, T, 571)
+    L = lib.load()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(s1):
+        w["layer"].forward(w["table"], logits, x, shared=w["dense"], stream=s1)
+    s1.synchronize()
+    out2 = torch.zeros_like(w["layer"].out)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s1):
+        w["layer"].forward(w["table"], logits, x, shared=w["dense"], stream=torch.cuda.current_stream())
+        rc = L.maya_moe_layer_decode_shared(C.byref(w["layer"].layout), w["table"].data_ptr(), NE, TK, None, logits.data_ptr(), x.data_ptr(),
+                                            0, T, float("inf"), C.byref(w["dense"].args), w["layer"].ids.data_ptr(),
+                                            w["layer"].weights.data_ptr(), out2.data_ptr(), w["layer"].ws.data_ptr(), w["layer"].ws_bytes,
+                                            C.c_void_p(s2.cuda_stream))
+        busy_msg = L.maya_last_error()
+        w["layer"].forward(w["table"], logits, x, shared=w["dense"], stream=torch.cuda.current_stream())   # the same capture again
+    assert rc == 5 and b"capture" in busy_msg
+    s2.synchronize()
+    assert not out2.any()   # nothing ran for the refused call
+    l2, x2, _ = inputs(E, NE, T, 572)
+    logits.copy_(l2)
+    x.copy_(x2)
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    got = w["layer"].out[:T].clone()
+    want = two_calls(w, logits, x, None, float("inf"))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    # after the capture has ended the other stream is served
+    with torch.cuda.stream(s2):
+        got2 = w["layer"].forward(w["table"], logits, x, shared=w["dense"], stream=s2).clone()
+    s2.synchronize()
+    assert torch.equal(got2, want)

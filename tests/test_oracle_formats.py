@@ -228,6 +228,55 @@ def test_float_and_double_selection_agree(oracle):
     assert np.array_equal(a, b)
 
 
+def test_softmax_router_against_an_independent_statement(oracle):
+    """The softmax router's ids and weights against numpy: softmax in double, the k largest by a stable descending sort
+    (the lower index wins a tie), the chosen probabilities renormalised by max(sum, 2^-14) - the reference's host form
+    (src/kernels/router_top10_parity.cpp:36-60).  Random rows, rows of quantised logits (many exact ties), all-equal rows."""
+    rng = np.random.default_rng(81)
+    k, ne = 8, 256
+    rows = [rng.standard_normal((400, ne)), np.round(rng.standard_normal((150, ne)) * 2.0) / 2.0, np.zeros((3, ne)),
+            np.full((2, ne), -3.25)]
+    logits = np.concatenate(rows).astype(np.float32)
+    ids, w = oracle.router_topk(logits, k)
+    for t in range(logits.shape[0]):
+        x = logits[t].astype(np.float64)
+        p = np.exp(x - x.max())
+        p /= p.sum()
+        pf = p.astype(np.float32)   # (the device selects on the probabilities rounded to float: ties there go to the lower index too)
+        order = np.argsort(-pf, kind="stable")[:k]
+        assert np.array_equal(ids[t], order), t
+        want = p[order] / max(p[order].sum(), 2.0 ** -14)
+        assert np.max(np.abs(w[t] - want) / want) < 1e-5, t
+    # closed forms: all-equal logits -> ids 0 .. k-1, every weight 1 / k
+    assert np.array_equal(ids[-1], np.arange(k)) and np.allclose(w[-1], 1.0 / k, rtol=1e-6)
+    # a wrong reading must differ: no renormalisation leaves the weights' sum below 1
+    assert abs(float(w[0].sum()) - 1.0) < 1e-5
+
+
+def test_combine_is_the_slot_order_rounded_sum(oracle):
+    """mo_combine against its statement (src/kernels/cuda/native_moe.cu:36-52): sum = parts[0] * w[0]; sum += parts[i] * w[i]
+    in slot order, every product and every sum rounded to float - bit for bit; a reversed order or a fused multiply-add
+    gives different bits on random data."""
+    rng = np.random.default_rng(82)
+    parts = rng.standard_normal((8, 4096)).astype(np.float32)
+    w = rng.random(8).astype(np.float32)
+    got = oracle.combine(parts, w)
+    want = (parts[0] * w[0]).astype(np.float32)
+    for i in range(1, 8):
+        want = (want + (parts[i] * w[i]).astype(np.float32)).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    rev = (parts[7] * w[7]).astype(np.float32)
+    for i in range(6, -1, -1):
+        rev = (rev + (parts[i] * w[i]).astype(np.float32)).astype(np.float32)
+    assert not np.array_equal(rev.view(np.uint32), want.view(np.uint32))
+    fused = (parts[0].astype(np.float64) * w[0]).astype(np.float32)
+    for i in range(1, 8):
+        fused = (fused.astype(np.float64) + parts[i].astype(np.float64) * float(w[i])).astype(np.float32)
+    assert not np.array_equal(fused.view(np.uint32), want.view(np.uint32))
+    # one slot: the product alone
+    assert np.array_equal(oracle.combine(parts[:1], w[:1]).view(np.uint32), (parts[0] * w[0]).astype(np.float32).view(np.uint32))
+
+
 # ---- the sigmoid router: the device arithmetic against the reference's host form (router_sigmoid_parity.cpp:36-86) restated
 # here in double with a stable sort, on that test's own case shapes, to its bars (ids equal, weights 1e-5; :137-143)
 
