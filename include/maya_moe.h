@@ -162,6 +162,8 @@ int maya_dequant_rows_packed(int ggml_type, int packing, const void* w, size_t r
  * (quantize_oracle_q8_0, src/kernels/cpu/expert.cpp:92-130): FP16 d = amax / 127, q = nearest-even(x * (127 / amax)); the
  * reference's GPU quantize_q8_0 (include/strata/kernels/quantize_act.hpp:28-31; rint of the double quotient x / d) gives
  * the same scale and differs by one code on the rare value next to a rounding boundary.
+ * The contract covers finite inputs: a block that holds a NaN, an infinity or a value whose scaled magnitude passes 2^31 is
+ * outside it (the x86 path saturates such lanes to -128, this library clamps them to +-127 and turns NaN into 0).
  * x: rows x k of x_dtype, x_stride elements apart (0: k). */
 int maya_quant_act(int act_type, const void* x, int x_dtype, int64_t x_stride, int rows, int64_t k, maya_act out,
                    void* stream);
@@ -403,7 +405,10 @@ int maya_moe_prefill_down(const maya_moe_layout* l, const uint64_t* expert_table
 /* out[t] = sum_j weights[t][j] * part[entry_row[t k + j]] in slot order (+ add[t]), stored as out_dtype */
 int maya_moe_prefill_combine(const maya_prefill_plan* plan, const float* weights, const float* part, int n_tokens, int k,
                              int64_t n_embd, const float* add, void* out, int out_dtype, void* stream);
-/* route -> plan -> quantize -> gate/up -> down -> combine of one chunk, all on `stream` */
+/* route -> plan -> quantize -> gate/up -> down -> combine of one chunk, all on `stream`.  A chunk holds at most 8192 tokens
+ * and at most 65535 entries (n_tokens * k: the entries are a grid dimension of the quantizers); a larger call is refused
+ * with MAYA_E_SHAPE before anything is launched - 8192 tokens at k = 8 is one entry too many, 8191 fit.  The stage calls
+ * (maya_moe_prefill_plan / _quant / _gate_up / _down) share the entry limit. */
 size_t maya_moe_prefill_workspace_bytes(const maya_moe_layout* l, int n_tokens, int k, int n_expert);
 int maya_moe_prefill_layer(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const float* logits,
                            const void* x, int x_dtype, int n_tokens, float limit, const float* add, int32_t* ids,

@@ -74,15 +74,26 @@ int current_state(DeviceState** out) {
             hipError_t e = hipMalloc((void**) &d, sizeof(uint64_t) * (1024 + 2048));
             if (e == hipSuccess) e = hipMemcpy(d, host, sizeof(uint64_t) * (1024 + 2048), hipMemcpyHostToDevice);
             delete[] host;
-            if (e != hipSuccess) return hip_fail(e, "codebook upload");
+            // (a step that fails gives back what the steps before it made: the next call starts over)
+            auto undo = [&](hipError_t err, const char* what) {
+                if (s.side_join) (void) hipEventDestroy(s.side_join);
+                if (s.side_fork) (void) hipEventDestroy(s.side_fork);
+                if (s.side) (void) hipStreamDestroy(s.side);
+                s.side_join = s.side_fork = nullptr;
+                s.side = nullptr;
+                s.static_scratch = nullptr;
+                if (d) (void) hipFree(d);
+                return hip_fail(err, what);
+            };
+            if (e != hipSuccess) return undo(e, "codebook upload");
             void* sp = nullptr;
             e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));   // (this device is the current one)
-            if (e != hipSuccess || sp == nullptr) return hip_fail(e == hipSuccess ? hipErrorInvalidSymbol : e, "address of the static scratch");
+            if (e != hipSuccess || sp == nullptr) return undo(e == hipSuccess ? hipErrorInvalidSymbol : e, "address of the static scratch");
             s.static_scratch = sp;
-            if ((e = hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking)) != hipSuccess) return hip_fail(e, "the shared expert's stream");
+            if ((e = hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking)) != hipSuccess) return undo(e, "the shared expert's stream");
             if ((e = hipEventCreateWithFlags(&s.side_fork, hipEventDisableTiming)) != hipSuccess ||
                 (e = hipEventCreateWithFlags(&s.side_join, hipEventDisableTiming)) != hipSuccess)
-                return hip_fail(e, "the shared expert's events");
+                return undo(e, "the shared expert's events");
             s.cb.iq2s = d;
             s.cb.iq1s = d + 1024;
             s.lds_limit = (int) p.sharedMemPerBlock;

@@ -303,3 +303,17 @@ def test_unsupported_and_bad_arguments(pf):
                     torch.zeros((4096, 256), dtype=torch.float32, device="cuda"))
     torch.cuda.synchronize()
     assert bool((big.ids == -7).all())
+    # the advertised 8192 tokens at k = 8 are one entry past the 65535 a call takes: refused with MAYA_E_SHAPE, nothing
+    # launched; 8191 tokens fit the limit
+    import ctypes as C
+    lay = lib.layout(Q4_K, Q4_K, 256, 256)[0]
+    ids8 = torch.full((8192, 8), -7, dtype=torch.int32, device="cuda")
+    w8 = torch.zeros((8192, 8), dtype=torch.float32, device="cuda")
+    out8 = torch.zeros((8192, 256), dtype=torch.float32, device="cuda")
+    ws = torch.zeros(int(L.maya_moe_prefill_workspace_bytes(C.byref(lay), 8191, 8, 16)) + 256, dtype=torch.uint8, device="cuda")
+    tab16 = torch.arange(1, 17, dtype=torch.int64, device="cuda") * 4096
+    rc = L.maya_moe_prefill_layer(C.byref(lay), lib._p(tab16), 16, 8, lib._p(torch.zeros((8192, 16), device="cuda")),
+                                  lib._p(torch.zeros((8192, 256), device="cuda")), 0, 8192, 0.0, None, lib._p(ids8), lib._p(w8), lib._p(out8), 0,
+                                  lib._p(ws), ws.numel(), None)
+    torch.cuda.synchronize()
+    assert rc == 2 and b"65535" in L.maya_last_error() and bool((ids8 == -7).all())

@@ -56,3 +56,44 @@ def test_static_layer_equals_the_workspace_layer_twice_in_a_row():
     torch.cuda.synchronize()
     assert rc == 2 and b"static" in L.maya_last_error()
     assert int(ids[0, 0]) == -7 and bool(torch.isnan(out).all())
+
+
+def test_static_layer_is_capturable_and_leaves_device_memory_alone():
+    """Nothing is allocated: the call is captured into a HIP graph (a capture fails when anything under it allocates device
+    memory or copies synchronously), the device's free memory is the same before and after, and the replayed graph gives the
+    eager call's bits."""
+    from maya_amd import lib
+    L = lib.load()
+    lib.check(L.maya_init())
+    L.maya_moe_layer_decode_static.argtypes = [C.POINTER(lib.Layout), C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                               C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    rng = np.random.default_rng(2027)
+    gt, dt, n_embd, n_ff, ne, k, nt = 22, 22, 4096, 2048, 12, 8, 2
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 950)
+    gguf, _ = lib.layout(gt, dt, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf)
+    layer = lib.MoeLayer(gt, dt, n_embd, n_ff, ne, k, max_tokens=nt, packing=1)
+    logits = dev(rng.standard_normal((nt, ne)).astype(np.float32))
+    x = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    rc, ids, w, out = _static(lib, L, layer, store.table, logits, x)   # (eager first: every kernel's code is on the device)
+    assert rc == 0, L.maya_last_error().decode()
+    torch.cuda.synchronize()
+    want = out.clone()
+    ids2 = torch.full_like(ids, -7)
+    w2 = torch.zeros_like(w)
+    out2 = torch.full_like(out, float("nan"))
+    s = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        rc = L.maya_moe_layer_decode_static(C.byref(layer.layout), lib._p(store.table), ne, k, None, lib._p(logits), lib._p(x), lib.dtype_id(x), nt,
+                                            float("inf"), None, lib._p(ids2), lib._p(w2), lib._p(out2), lib._stream())
+    assert rc == 0, L.maya_last_error().decode()
+    for _ in range(2):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ids2, ids) and torch.equal(w2, w) and torch.equal(out2.view(torch.int32), want.view(torch.int32))
+        out2.fill_(float("nan"))
+        torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] >= free_before - (4 << 20)   # (the graph's own launch records, nothing else)
