@@ -32,6 +32,7 @@ extern "C" {
 /* ggml type ids of the weight formats (src/ds4/ds4_iq.cuh:27-31) */
 #define MAYA_TYPE_Q8_0 8
 #define MAYA_TYPE_Q4_K 12
+#define MAYA_TYPE_IQ2_XXS 16 /* general kernels only: no stream packing of its own, no prefill GEMM */
 #define MAYA_TYPE_IQ1_S 19
 #define MAYA_TYPE_IQ2_S 22
 #define MAYA_TYPE_IQ1_M 29

@@ -72,7 +72,7 @@ uint16_t mo_f32_to_bf16(float f) {
 
 /* ------------------------------------------------------------------------------------------------- codebooks */
 
-static uint64_t g_iq2s[1024], g_iq1s[2048];
+static uint64_t g_iq2s[1024], g_iq1s[2048], g_iq2xxs[256];
 static int g_grids_ready = 0;
 
 static void grids_init(void) {
@@ -91,6 +91,11 @@ static void grids_init(void) {
                 for (int j = 0; j < 8; ++j) v |= (uint64_t) m1[(maya_iq1s_packed[i] >> (2 * j)) & 3] << (8 * j);
                 g_iq1s[i] = v;
             }
+            for (int i = 0; i < 256; ++i) {
+                uint64_t v = 0;
+                for (int j = 0; j < 8; ++j) v |= (uint64_t) m2[(maya_iq2xxs_packed[i] >> (2 * j)) & 3] << (8 * j);
+                g_iq2xxs[i] = v;
+            }
             g_grids_ready = 1;
         }
     }
@@ -103,6 +108,13 @@ const uint64_t* mo_iq1s_grid(void) {
     grids_init();
     return g_iq1s;
 }
+const uint64_t* mo_iq2xxs_grid(void) {
+    grids_init();
+    return g_iq2xxs;
+}
+/* ksigns_iq2xs (third_party/ggml/ggml-common.h:513): seven sign bits and, in bit 7, their parity - an even number of
+ * negative values in every group of 8 */
+static inline uint8_t ksigns7(uint32_t i) { return (uint8_t) (i | ((uint32_t) (__builtin_popcount(i) & 1) << 7)); }
 
 uint32_t mo_crc32(const void* p, size_t n) {
     const uint8_t* b = (const uint8_t*) p;
@@ -124,6 +136,7 @@ int mo_block_bytes(int type) {
         case MO_IQ1_S: return 50;
         case MO_IQ2_S: return 82;
         case MO_IQ1_M: return 56;
+        case MO_IQ2_XXS: return 66;
         default: return 0;
     }
 }
@@ -199,6 +212,25 @@ static void dq_iq2_s(const uint8_t* blk, float* out) {
         }
     }
 }
+/* src/kernels/cuda/iq_kernels.cu:661-672 (dq_iq2_xxs); block third_party/ggml/ggml-common.h:380-384: d, then 8 bytes a
+ * 32-value sub-block - four codebook indices, then four 7-bit sign indices and a 4-bit scale in one word */
+static void dq_iq2_xxs(const uint8_t* blk, float* out) {
+    const uint64_t* grid = mo_iq2xxs_grid();
+    const float d = mo_f16_to_f32(rd16(blk));
+    for (int ib = 0; ib < 8; ++ib) {
+        const uint8_t* q = blk + 2 + 8 * ib;
+        const uint32_t aux = rd32(q + 4);
+        const float dl = d * (0.5f + (float) (aux >> 28)) * 0.25f;
+        for (int il = 0; il < 4; ++il) {
+            const uint64_t g = grid[q[il]];
+            const uint8_t sg = ksigns7((aux >> (7 * il)) & 127u);
+            for (int j = 0; j < 8; ++j) {
+                const float v = dl * (float) ((g >> (8 * j)) & 255u);
+                out[32 * ib + 8 * il + j] = (sg >> j) & 1 ? -v : v;
+            }
+        }
+    }
+}
 /* src/kernels/cuda/iq_kernels.cu:825-837 (dq_iq1_s): d*(2s+1) * (grid + delta), delta = -+0.125 by qh bit 15 */
 static void dq_iq1_s(const uint8_t* blk, float* out) {
     const uint64_t* grid = mo_iq1s_grid();
@@ -244,6 +276,7 @@ int mo_dequant_row(int type, const uint8_t* row, int64_t k, float* out) {
             case MO_IQ2_S: dq_iq2_s(blk, o); break;
             case MO_IQ1_S: dq_iq1_s(blk, o); break;
             case MO_IQ1_M: dq_iq1_m(blk, o); break;
+            case MO_IQ2_XXS: dq_iq2_xxs(blk, o); break;
             default: return 1;
         }
     }
@@ -383,6 +416,37 @@ static float dot_iq2_s(const uint8_t* row, int nb, const mo_q8k* y) {
     return 0.125f * hsum8(accf);
 }
 
+/* IQ2_XXS x Q8_K (iq_avx2.cpp:130-141 Fmt32<16>::decode, 225-250 row_dot): as IQ2_S with one scale a 32-value chunk */
+static float dot_iq2_xxs(const uint8_t* row, int nb, const mo_q8k* y) {
+    const uint64_t* grid = mo_iq2xxs_grid();
+    float accf[8] = {0};
+    for (int i = 0; i < nb; ++i) {
+        const uint8_t* blk = row + (size_t) i * 66;
+        int32_t acci[8] = {0};
+        for (int c = 0; c < 8; ++c) {
+            const uint8_t* q = blk + 2 + 8 * c;
+            const uint32_t aux = rd32(q + 4);
+            const int sc = 2 * (int) (aux >> 28) + 1;
+            for (int l = 0; l < 4; ++l) {
+                const uint64_t g = grid[q[l]];
+                const uint8_t sg = ksigns7((aux >> (7 * l)) & 127u);
+                const int8_t* q8 = y[i].qs + 32 * c + 8 * l;
+                for (int hf = 0; hf < 2; ++hf) { /* lane n = 2l + hf */
+                    int s = 0;
+                    for (int j = 4 * hf; j < 4 * hf + 4; ++j) {
+                        const int m = (int) ((g >> (8 * j)) & 255u);
+                        s += m * ((sg >> j) & 1 ? -(int) q8[j] : (int) q8[j]);
+                    }
+                    acci[2 * l + hf] += s * sc;
+                }
+            }
+        }
+        const float dd = mo_f16_to_f32(rd16(blk)) * y[i].d;
+        for (int n = 0; n < 8; ++n) accf[n] = fmaf(dd, (float) acci[n], accf[n]);
+    }
+    return 0.125f * hsum8(accf);
+}
+
 /* Q4_K x Q8_K (iq_avx2.cpp:319-394 k_scales + row_dot_k<12>) */
 static float dot_q4_K(const uint8_t* row, int nb, const mo_q8k* y) {
     float accf[8] = {0}, accm[4] = {0};
@@ -500,6 +564,7 @@ float mo_vec_dot(int type, const uint8_t* row, int64_t k, const void* act) {
         case MO_IQ2_S: return dot_iq2_s(row, (int) (k / 256), (const mo_q8k*) act);
         case MO_IQ1_S: return dot_iq1_s(row, (int) (k / 256), (const mo_q8k*) act);
         case MO_IQ1_M: return dot_iq1_m(row, (int) (k / 256), (const mo_q8k*) act);
+        case MO_IQ2_XXS: return dot_iq2_xxs(row, (int) (k / 256), (const mo_q8k*) act);
         default: return NAN;
     }
 }

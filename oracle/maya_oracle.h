@@ -15,6 +15,10 @@
  *   IQ2_S dequant .................... structure check |w| = d(2ls+1)/8 * {8,25,43}; integer decode identical to the
  *                                       reference build's Fmt32<22>::decode through the row dots below; codebook CRC
  *   IQ1_M dequant .................... integer decode pinned through the reference build's iq256_rows(29,...)
+ *   IQ2_XXS dequant .................. an independent numpy decode from the block layout (ggml-common.h:380-384) over every
+ *                                       codebook index x sign index x scale, bit for bit; codebook CRC and the reference tree's
+ *                                       table; the sign table's rule (bit 7 = parity of the low seven) checked against
+ *                                       ksigns_iq2xs when the grids are generated; integer decode through the row dots below
  *   IQ1_S dequant .................... an independent numpy decode written from the block layout and dq_iq1_s's formula
  *                                       (ggml-common.h:425-430, src/kernels/cuda/iq_kernels.cu:825-837), bit for bit over every
  *                                       grid index x 3-bit scale x delta sign and on random blocks; the same values, bit for bit,
@@ -34,7 +38,7 @@
  *                                       against it (one code apart on < 2e-4 of N(0,1) values)
  *   Q8_0 x Q8_0 row dot .............. the float64 dot of both operands dequantized independently with numpy, 1e-6 of the terms'
  *                                       magnitude; block-permutation and negation invariants (exact where they must be)
- *   row dots IQ2_S / Q4_K / IQ1_M .... reference build: strata::kernels::cpu::iq256_rows / iq256_gu_rows, BIT-EXACT
+ *   row dots IQ2_S/Q4_K/IQ1_M/IQ2_XXS  reference build: strata::kernels::cpu::iq256_rows / iq256_gu_rows, BIT-EXACT
  *                                       (this file restates the 8 int32 lanes and the float steps in their order)
  *   IQ2_S expert in device arithmetic  reference build: strata::ds4::par::gate_up_ref / down_ref, bit-exact
  *   SwiGLU ........................... closed form; exp_portable (ds4_par_exp.h:60-85) bit-exact against the reference build
@@ -101,6 +105,7 @@ uint16_t mo_f32_to_bf16(float f); /* round to nearest even */
 /* ---- codebooks expanded from iq_grids.h (third_party/ggml/ggml-common.h:758, 1135) */
 const uint64_t* mo_iq2s_grid(void); /* 1024 entries */
 const uint64_t* mo_iq1s_grid(void); /* 2048 entries */
+const uint64_t* mo_iq2xxs_grid(void); /* 256 entries */
 uint32_t mo_crc32(const void* p, size_t n);
 
 /* ---- format geometry (src/ds4/ds4_iq.cuh:47-52) */

@@ -48,6 +48,7 @@ def lib():
         L.mo_bf16_to_f32.argtypes = [C.c_uint16]
         L.mo_iq2s_grid.restype = C.POINTER(C.c_uint64)
         L.mo_iq1s_grid.restype = C.POINTER(C.c_uint64)
+        L.mo_iq2xxs_grid.restype = C.POINTER(C.c_uint64)
         L.mo_crc32.restype = C.c_uint32
         L.mo_crc32.argtypes = [C.c_void_p, C.c_size_t]
         L.mo_block_bytes.argtypes = [C.c_int]

@@ -16,7 +16,7 @@
 
 namespace maya {
 
-constexpr int kQ8_0 = 8, kQ4_K = 12, kIQ1_S = 19, kIQ2_S = 22, kIQ1_M = 29;
+constexpr int kQ8_0 = 8, kQ4_K = 12, kIQ2_XXS = 16, kIQ1_S = 19, kIQ2_S = 22, kIQ1_M = 29;
 constexpr int kWave = 64;
 
 // ------------------------------------------------------------------------------------------------ scalars
@@ -49,6 +49,7 @@ __device__ __forceinline__ float group_sum(float v) {
 struct Codebooks {
     const uint64_t* iq2s;  // 1024 x 8 magnitudes
     const uint64_t* iq1s;  // 2048 x 8 values -1 / 0 / +1
+    const uint64_t* iq2xxs;  // 256 x 8 magnitudes
 };
 
 // four sign bits -> 0x01 in the bytes of the set bits (bit i -> byte i); the 16 partial products land on distinct bits
@@ -180,6 +181,29 @@ template <> struct Fmt<kIQ2_S> {
         const uint32_t hs = ((const uint16_t*) (quad + 32 * (size_t) nu))[un * 4 + rq];
         d = f16_bits_to_f32(((const uint16_t*) (quad + 40 * (size_t) nu))[(un >> 3) * 4 + rq]) * 0.125f;
         decode_fields(is.x, is.y, hs & 255u, hs >> 8, grid, u);
+    }
+};
+
+// IQ2_XXS: 66 bytes a 256-value block - d, then 8 bytes a 32-value sub-block: four codebook indices (256 entries), then one
+// word of four 7-bit sign indices and a 4-bit scale for all 32 values.  A sign index is seven sign bits; the eighth is
+// their parity (ksigns_iq2xs, third_party/ggml/ggml-common.h:513: an even number of negative values a group of 8).
+template <> struct Fmt<kIQ2_XXS> {
+    static constexpr bool kBiased = false;
+    static constexpr int kBytes = 66, kValues = 256, kUnit = 32, kLdsWords = 512;  // codebook: 256 x u64
+    static constexpr bool kMin = false;
+    __device__ static __forceinline__ float scale(const uint8_t* blk) { return f16_bits_to_f32(ld16(blk)) * 0.125f; }
+    __device__ static __forceinline__ uint32_t signs8(uint32_t seven) { return seven | ((uint32_t) (__popc(seven) & 1) << 7); }
+    // third_party/ggml/ggml-common.h:380-384; decode: src/kernels/cuda/iq_kernels.cu:661-672
+    __device__ static __forceinline__ void decode(const uint8_t* blk, int ib, const uint2* grid, Unit32& u) {
+        const uint32_t w0 = ld32_a2(blk + 2 + 8 * ib), aux = ld32_a2(blk + 6 + 8 * ib);
+#pragma unroll
+        for (int l = 0; l < 4; ++l) {
+            const uint2 g = grid[(w0 >> (8 * l)) & 255u];
+            const uint32_t sb = signs8((aux >> (7 * l)) & 127u);
+            u.q[2 * l] = (int) neg_bytes(g.x, spread4(sb & 15u));
+            u.q[2 * l + 1] = (int) neg_bytes(g.y, spread4(sb >> 4));
+        }
+        u.s0 = u.s1 = 2 * (int) (aux >> 28) + 1;
     }
 };
 

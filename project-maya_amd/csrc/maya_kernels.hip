@@ -59,7 +59,7 @@ int current_state(DeviceState** out) {
             if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
                 return fail(MAYA_E_NOGPU, "device %d is %s; this library holds gfx950 code only", dev, p.gcnArchName);
             static const uint8_t m2[4] = {8, 25, 43, 0}, m1[4] = {0xff, 0x00, 0x01, 0};
-            uint64_t* host = new uint64_t[1024 + 2048];
+            uint64_t* host = new uint64_t[1024 + 2048 + 256];
             for (int i = 0; i < 1024; ++i) {
                 uint64_t v = 0;
                 for (int j = 0; j < 8; ++j) v |= (uint64_t) m2[(maya_iq2s_packed[i] >> (2 * j)) & 3] << (8 * j);
@@ -70,9 +70,14 @@ int current_state(DeviceState** out) {
                 for (int j = 0; j < 8; ++j) v |= (uint64_t) m1[(maya_iq1s_packed[i] >> (2 * j)) & 3] << (8 * j);
                 host[1024 + i] = v;
             }
+            for (int i = 0; i < 256; ++i) {
+                uint64_t v = 0;
+                for (int j = 0; j < 8; ++j) v |= (uint64_t) m2[(maya_iq2xxs_packed[i] >> (2 * j)) & 3] << (8 * j);
+                host[1024 + 2048 + i] = v;
+            }
             uint64_t* d = nullptr;
-            hipError_t e = hipMalloc((void**) &d, sizeof(uint64_t) * (1024 + 2048));
-            if (e == hipSuccess) e = hipMemcpy(d, host, sizeof(uint64_t) * (1024 + 2048), hipMemcpyHostToDevice);
+            hipError_t e = hipMalloc((void**) &d, sizeof(uint64_t) * (1024 + 2048 + 256));
+            if (e == hipSuccess) e = hipMemcpy(d, host, sizeof(uint64_t) * (1024 + 2048 + 256), hipMemcpyHostToDevice);
             delete[] host;
             // (a step that fails gives back what the steps before it made: the next call starts over)
             auto undo = [&](hipError_t err, const char* what) {
@@ -96,6 +101,7 @@ int current_state(DeviceState** out) {
                 return undo(e, "the shared expert's events");
             s.cb.iq2s = d;
             s.cb.iq1s = d + 1024;
+            s.cb.iq2xxs = d + 1024 + 2048;
             s.lds_limit = (int) p.sharedMemPerBlock;
             s.n_cu = p.multiProcessorCount;
             s.ready = true;
@@ -159,6 +165,15 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
         const uint64_t g = cb.iq2s[idx];
         const int ls = (sc >> (4 * (il >> 1))) & 15;
         const float dl = __fmul_rn(__fmul_rn(f16_bits_to_f32(dbits), __fadd_rn(0.5f, (float) ls)), 0.25f);
+        const float mag = __fmul_rn(dl, (float) (uint32_t) ((g >> (8 * j)) & 255u));
+        r = (sg >> j) & 1 ? -mag : mag;
+    } else if constexpr (TYPE == kIQ2_XXS) {
+        const int i = (int) (v & 255), ib = i >> 5, il = (i >> 3) & 3, j = i & 7;
+        const uint8_t* blk = rp + (size_t) (v >> 8) * 66;
+        const uint32_t aux = ld32_a2(blk + 6 + 8 * ib);
+        const uint64_t g = cb.iq2xxs[blk[2 + 8 * ib + il]];
+        const uint32_t sg = Fmt<kIQ2_XXS>::signs8((aux >> (7 * il)) & 127u);
+        const float dl = __fmul_rn(__fmul_rn(f16_bits_to_f32(ld16(blk)), __fadd_rn(0.5f, (float) (aux >> 28))), 0.25f);
         const float mag = __fmul_rn(dl, (float) (uint32_t) ((g >> (8 * j)) & 255u));
         r = (sg >> j) & 1 ? -mag : mag;
     } else if constexpr (TYPE == kIQ1_S) {
@@ -1087,6 +1102,7 @@ __device__ __forceinline__ void row_dot(const uint8_t* __restrict__ row, int k, 
 template <int TYPE> __device__ __forceinline__ const uint64_t* codebook_of(const Codebooks& cb) {
     if constexpr (TYPE == kIQ2_S) return cb.iq2s;
     else if constexpr (TYPE == kIQ1_S || TYPE == kIQ1_M) return cb.iq1s;
+    else if constexpr (TYPE == kIQ2_XXS) return cb.iq2xxs;
     else return nullptr;
 }
 
@@ -1359,7 +1375,7 @@ namespace maya {
 
 // ------------------------------------------------------------------------------------------------ host launchers
 
-bool type_ok(int t) { return t == kQ8_0 || t == kQ4_K || t == kIQ1_S || t == kIQ2_S || t == kIQ1_M; }
+bool type_ok(int t) { return t == kQ8_0 || t == kQ4_K || t == kIQ2_XXS || t == kIQ1_S || t == kIQ2_S || t == kIQ1_M; }
 bool q8k_act(int t) { return t != kQ8_0; }
 int block_bytes(int t) {
     switch (t) {
@@ -1368,11 +1384,12 @@ int block_bytes(int t) {
         case kIQ1_S: return 50;
         case kIQ2_S: return 82;
         case kIQ1_M: return 56;
+        case kIQ2_XXS: return 66;
         default: return 0;
     }
 }
 int block_values(int t) { return t == kQ8_0 ? 32 : (type_ok(t) ? 256 : 0); }
-int codebook_words(int t) { return t == kIQ2_S ? 2048 : (t == kIQ1_S || t == kIQ1_M) ? 4096 : 0; }
+int codebook_words(int t) { return t == kIQ2_S ? 2048 : (t == kIQ1_S || t == kIQ1_M) ? 4096 : t == kIQ2_XXS ? 512 : 0; }
 size_t act_lds_bytes(int k, int nt) { return (size_t) nt * ((size_t) k + (size_t) (k / 32) * 8); }
 
 int check_layout(const maya_moe_layout& l) {
@@ -1959,6 +1976,7 @@ int maya_dequant_rows_packed(int t, int packing, const void* w, size_t row_strid
         case kQ4_K: hipLaunchKernelGGL(dequant_kernel<kQ4_K>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
         case kIQ2_S: hipLaunchKernelGGL(dequant_kernel<kIQ2_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
         case kIQ1_S: hipLaunchKernelGGL(dequant_kernel<kIQ1_S>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
+        case kIQ2_XXS: hipLaunchKernelGGL(dequant_kernel<kIQ2_XXS>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
         default: hipLaunchKernelGGL(dequant_kernel<kIQ1_M>, grid, dim3(256), 0, s, wb, row_stride, k, out, st->cb, packing); break;
     }
     MAYA_LAUNCHED("dequant_kernel");
@@ -2170,6 +2188,7 @@ int maya_moe_gate_up(const maya_moe_args* a, void* stream) {
     MAYA_GU(kQ8_0, kQ8_0)
     MAYA_GU(kIQ1_S, kIQ1_S)
     MAYA_GU(kIQ1_M, kIQ1_M)
+    MAYA_GU(kIQ2_XXS, kIQ2_XXS)
     MAYA_GU(kIQ2_S, kIQ1_M)
     MAYA_GU(kIQ1_M, kIQ2_S)
     MAYA_GU(kIQ2_S, kQ4_K)
@@ -2212,6 +2231,7 @@ int maya_moe_down(const maya_moe_args* a, void* stream) {
         case kQ4_K: rc = launch_down_t<kQ4_K>(*a, *st, s); break;
         case kQ8_0: rc = launch_down_t<kQ8_0>(*a, *st, s); break;
         case kIQ1_S: rc = launch_down_t<kIQ1_S>(*a, *st, s); break;
+        case kIQ2_XXS: rc = launch_down_t<kIQ2_XXS>(*a, *st, s); break;
         default: rc = launch_down_t<kIQ1_M>(*a, *st, s); break;
     }
     if (rc) return rc;
@@ -2297,7 +2317,7 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
         fast[i] = mv_pos_ok(jobs[i]);
         if (fast[i]) launch_mv_pos(jobs[i], as_stream(stream));
     }
-    static const int kTypes[] = {kQ8_0, kQ4_K, kIQ1_S, kIQ2_S, kIQ1_M};
+    static const int kTypes[] = {kQ8_0, kQ4_K, kIQ2_XXS, kIQ1_S, kIQ2_S, kIQ1_M};
     for (const int t : kTypes) {
         MvBatch b{};
         int n = 0, max_in = 0, max_out = 0, max_col = 0;
@@ -2316,6 +2336,7 @@ int maya_mv(const maya_mv_job* jobs, int n_jobs, void* stream) {
             case kQ4_K: rc = launch_mv_t<kQ4_K>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
             case kIQ1_S: rc = launch_mv_t<kIQ1_S>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
             case kIQ2_S: rc = launch_mv_t<kIQ2_S>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
+            case kIQ2_XXS: rc = launch_mv_t<kIQ2_XXS>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
             default: rc = launch_mv_t<kIQ1_M>(b, n, max_in, max_out, max_col, *st, as_stream(stream)); break;
         }
         if (rc) return rc;

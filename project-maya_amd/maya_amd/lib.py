@@ -8,7 +8,7 @@ import torch
 PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(PKG, "libmaya_moe.so")
 
-Q8_0, Q4_K, IQ1_S, IQ2_S, IQ1_M = 8, 12, 19, 22, 29
+Q8_0, Q4_K, IQ2_XXS, IQ1_S, IQ2_S, IQ1_M = 8, 12, 16, 19, 22, 29
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 MAX_TOKENS, MAX_K = 16, 16
 PACK_GGUF, PACK_STREAM = 0, 1

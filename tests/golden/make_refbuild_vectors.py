@@ -106,6 +106,29 @@ def main():
     out.update(exl3_tr=tr, exl3_w=wv.astype(np.float16), exl3_suh=suh, exl3_svh=svh, exl3_x=xv, exl3_y=yv)
 
     path = os.path.join(HERE, "refbuild_vectors.npz")
+    # IQ2_XXS rows (a generator of its own, so that the vectors above keep their values)
+    rng16 = np.random.default_rng(20261216)
+    for t in (16,):
+        kk, n = 768, 12
+        w = synth.constructed_rows(t, n, kk, rng16)
+        xs = rng16.standard_normal((2, kk)).astype(np.float32)
+        xs[1] *= 21.0
+        acts = [oracle_py.quant_q8k(v) for v in xs]
+        actp = (C.c_void_p * 2)(*[a.ctypes.data for a in acts])
+        outs = [np.zeros(n, dtype=np.float32) for _ in range(2)]
+        outp = (C.c_void_p * 2)(*[o.ctypes.data for o in outs])
+        R.ref_iq256_rows(t, w.ctypes.data, oracle_py.row_bytes(t, kk), kk, actp, 2, outp, 0, n)
+        out["rows%d_w" % t] = w
+        out["rows%d_act" % t] = np.stack(acts)
+        out["rows%d_y" % t] = np.stack(outs)
+        blob = np.concatenate([synth.constructed_rows(t, n, kk, rng16, d_scale=4.0), synth.constructed_rows(t, n, kk, rng16)])
+        rb = oracle_py.row_bytes(t, kk)
+        gouts = [np.zeros(n, dtype=np.float32) for _ in range(2)]
+        goutp = (C.c_void_p * 2)(*[o.ctypes.data for o in gouts])
+        R.ref_iq256_gu_rows(t, blob.ctypes.data, rb, n * rb, kk, actp, 2, goutp, 0, n)
+        out["gu%d_w" % t] = blob
+        out["gu%d_h" % t] = np.stack(gouts)
+
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
 

@@ -5,12 +5,13 @@ tests/hip/expert_kernel_bench.cpp:68-77).  numpy only; no device code here.
 """
 import numpy as np
 
-Q8_0, Q4_K, IQ1_S, IQ2_S, IQ1_M = 8, 12, 19, 22, 29
-BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, IQ1_S: 50, IQ2_S: 82, IQ1_M: 56}
-BLOCK_VALUES = {Q8_0: 32, Q4_K: 256, IQ1_S: 256, IQ2_S: 256, IQ1_M: 256}
+Q8_0, Q4_K, IQ2_XXS, IQ1_S, IQ2_S, IQ1_M = 8, 12, 16, 19, 22, 29
+BLOCK_BYTES = {Q8_0: 34, Q4_K: 144, IQ2_XXS: 66, IQ1_S: 50, IQ2_S: 82, IQ1_M: 56}
+BLOCK_VALUES = {Q8_0: 32, Q4_K: 256, IQ2_XXS: 256, IQ1_S: 256, IQ2_S: 256, IQ1_M: 256}
 # the block scale's range a type (tools/iq_fixture.py:40-60 gives IQ2_S [2e-3, 6e-3]); chosen so that rows of
 # thousands of values have O(1) sums
-D_RANGE = {Q8_0: (1e-4, 4e-4), Q4_K: (2e-4, 6e-4), IQ1_S: (4e-3, 1.2e-2), IQ2_S: (2e-3, 6e-3), IQ1_M: (4e-3, 1.2e-2)}
+D_RANGE = {Q8_0: (1e-4, 4e-4), Q4_K: (2e-4, 6e-4), IQ2_XXS: (2e-3, 6e-3), IQ1_S: (4e-3, 1.2e-2), IQ2_S: (2e-3, 6e-3),
+           IQ1_M: (4e-3, 1.2e-2)}
 
 
 def row_bytes(t, k):

@@ -39,7 +39,7 @@ def test_every_declared_function_is_exported(maya):
 def test_sizes_and_support_tables(maya, oracle):
     L = maya.load()
     for t, bytes_, vals in ((maya.Q8_0, 34, 32), (maya.Q4_K, 144, 256), (maya.IQ2_S, 82, 256), (maya.IQ1_S, 50, 256),
-                            (maya.IQ1_M, 56, 256)):
+                            (maya.IQ1_M, 56, 256), (maya.IQ2_XXS, 66, 256)):
         assert L.maya_moe_supported(t) == 1
         assert L.maya_moe_block_bytes(t) == bytes_ and L.maya_moe_block_values(t) == vals
         assert maya.row_bytes(t, 4096) == oracle.row_bytes(t, 4096) == 4096 // vals * bytes_

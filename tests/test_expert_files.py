@@ -100,7 +100,7 @@ def test_layers_and_blobs(tmp_path):
         # the library's own sizes for the same formats
         for t, k in ((L.gate_type, n_embd), (L.down_type, n_ff)):
             assert ef.row_bytes(t, k) == lib.row_bytes(t, k)
-        if L.up_type in (8, 12, 19, 22, 29):
+        if L.up_type in (8, 12, 16, 19, 22, 29):
             lay, nbytes = lib.layout(L.gate_type, L.down_type, n_embd, n_ff, L.up_type)
             assert nbytes == L.blob_bytes and lay.up_off - lay.gate_off == L.part_bytes[0] and lay.down_off - lay.up_off == L.part_bytes[1]
         blobs = ef.layer_blobs(g, L)

@@ -26,7 +26,7 @@ def test_q8k_blocks(oracle, vec):
     assert np.array_equal(bs, qs.astype(np.int32).reshape(-1, 16, 16).sum(axis=2))
 
 
-@pytest.mark.parametrize("t", (22, 12, 29))
+@pytest.mark.parametrize("t", (22, 12, 29, 16))
 def test_contract_rows_and_gate_up(oracle, vec, t):
     k, n = 768, 12
     acts = vec["rows%d_act" % t]

@@ -73,6 +73,11 @@ CASES = [
     (29, 29, 7168, 2048, 9, 8, 3),
     (29, 19, 6144, 2048, 4, 2, 2),
     (12, 29, 8192, 2048, 4, 3, 2),
+    # IQ2_XXS (the general kernels): one token, a window, mixed with IQ2_S either side
+    (16, 16, 1024, 512, 8, 4, 1),
+    (16, 16, 7168, 2048, 9, 8, 3),
+    (16, 22, 4096, 2048, 6, 4, 2),
+    (22, 16, 2048, 1024, 4, 2, 5),
     # other expert shapes on the position-mapped kernels: rows of 2048 / 3072 / 5120 values, n_ff 1024 / 1536 (the down
     # rows then leave lanes of their wave idle)
     (22, 22, 5120, 1536, 6, 4, 1),

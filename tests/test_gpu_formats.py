@@ -7,7 +7,7 @@ import synth
 
 pytestmark = pytest.mark.gpu
 
-TYPES = (8, 12, 19, 22, 29)
+TYPES = (8, 12, 16, 19, 22, 29)
 
 
 @pytest.fixture(scope="module")
@@ -35,7 +35,7 @@ def test_dequant_bit_exact(lib, oracle, t, misalign):
 def test_dequant_subnormal_scales(lib, oracle):
     """FP16 block scales in the subnormal range and at the extremes decode to the same bits."""
     rng = np.random.default_rng(3)
-    for t in (12, 22, 8, 19):
+    for t in (12, 22, 8, 19, 16):
         w = synth.constructed_rows(t, 2, 512, rng).reshape(-1, synth.BLOCK_BYTES[t])
         specials = np.array([0x0001, 0x03FF, 0x0400, 0x7BFF, 0x8001, 0x0000, 0x83FF, 0x3C00], dtype=np.uint16)
         for b in range(w.shape[0]):
@@ -103,7 +103,7 @@ def test_i8x32_quant_byte_exact(lib, oracle):
         assert np.array_equal(q[r], wq) and np.array_equal(d[r].view(np.uint32), wd.view(np.uint32))
 
 
-@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8), (19, 19), (19, 22), (29, 29)))
+@pytest.mark.parametrize("gt,dt", ((22, 22), (22, 12), (12, 22), (29, 8), (8, 8), (19, 19), (19, 22), (29, 29), (16, 16), (22, 16)))
 def test_stream_packing_round_trip_and_values(lib, oracle, gt, dt):
     """maya_moe_repack regroups bytes only: unpack(repack(blob)) == blob, and the packed rows dequantize to the same bits."""
     n_embd, n_ff = 1024, 512

@@ -40,6 +40,8 @@ CASES = [
     (22, 2048, 777, 5, 1.0, True),
     (22, 7168, 256, 16, 0.25, False),
     (29, 1024, 96, 4, 1.0, True),
+    (16, 1024, 130, 3, 1.0, True),
+    (16, 7168, 64, 1, 0.5, False),
     (22, 16384, 40, 4, 1.0, False),     # long rows: the activations of 4 columns do not fit LDS at once
 ]
 
@@ -80,7 +82,7 @@ def test_mv_against_the_oracle_rows(lib, oracle, t, n_in, n_out, ncol, alpha, wi
 
 def test_mv_jobs_of_several_types_in_one_call(lib, oracle):
     rng = np.random.default_rng(5)
-    specs = [(8, 1024, 200, 2), (12, 2048, 128, 1), (22, 1024, 64, 4), (12, 512, 333, 3), (29, 768, 50, 1), (19, 512, 20, 2)]
+    specs = [(8, 1024, 200, 2), (12, 2048, 128, 1), (22, 1024, 64, 4), (12, 512, 333, 3), (29, 768, 50, 1), (19, 512, 20, 2), (16, 768, 40, 2)]
     jobs, wants = [], []
     for t, n_in, n_out, ncol in specs:
         w = synth.constructed_rows(t, n_out, n_in, rng)
@@ -124,8 +126,8 @@ def test_mv_refusals_launch_nothing(lib):
         arr = (lib.MvJob * 1)(lib.MvJob(*[f[n] for n, _ in lib.MvJob._fields_]))
         return L.maya_mv(arr, 1, lib._stream())
 
-    assert L.maya_mv_supported(12) == 1 and L.maya_mv_supported(16) == 0
-    assert call(type=16) == 1            # MAYA_E_UNSUPPORTED
+    assert L.maya_mv_supported(12) == 1 and L.maya_mv_supported(10) == 0 and L.maya_mv_supported(16) == 1
+    assert call(type=10) == 1            # MAYA_E_UNSUPPORTED
     assert call(n_in=100) == 2           # MAYA_E_SHAPE
     assert call(ncol=17) == 2
     assert call(y=None) == 3             # MAYA_E_ARG

@@ -60,6 +60,10 @@ def test_codebooks(oracle):
     assert g1[0] == 0xFFFFFFFFFFFFFFFF and g1[1] == 0xFFFFFFFFFFFFFF01
     assert L.mo_crc32(g2.ctypes.data, g2.nbytes) == 0x25AE5BF1
     assert L.mo_crc32(g1.ctypes.data, g1.nbytes) == 0xB85E6CCF
+    gx = np.ctypeslib.as_array(L.mo_iq2xxs_grid(), shape=(256,)).copy()
+    assert set(np.unique(gx.view(np.uint8))) == {8, 25, 43} and len(np.unique(gx)) == 256
+    assert gx[0] == 0x0808080808080808 and gx[1] == 0x080808080808082B   # (ggml-common.h:561)
+    assert L.mo_crc32(gx.ctypes.data, gx.nbytes) == 0x9924FF02
 
 
 def test_codebooks_against_reference_tree(oracle):
@@ -71,7 +75,8 @@ def test_codebooks_against_reference_tree(oracle):
     src = open(path).read()
     L = oracle.lib()
     for decl, fn, n in (("GGML_TABLE_BEGIN(uint64_t, iq2s_grid, 1024)", L.mo_iq2s_grid, 1024),
-                        ("GGML_TABLE_BEGIN(uint64_t, iq1s_grid, NGRID_IQ1S)", L.mo_iq1s_grid, 2048)):
+                        ("GGML_TABLE_BEGIN(uint64_t, iq1s_grid, NGRID_IQ1S)", L.mo_iq1s_grid, 2048),
+                        ("GGML_TABLE_BEGIN(uint64_t, iq2xxs_grid, 256)", L.mo_iq2xxs_grid, 256)):
         m = re.search(re.escape(decl) + r"(.*?)GGML_TABLE_END", src, re.S)
         want = np.array([int(v, 16) for v in re.findall(r"0x[0-9a-fA-F]+", m.group(1))], dtype=np.uint64)
         got = np.ctypeslib.as_array(fn(), shape=(n,))
@@ -189,6 +194,36 @@ def test_iq2_s_dequant_structure(oracle):
     # the alternative association the exact kernels use: (d/8) * (2 ls + 1): the same float outside the subnormals
     alt = ((d[:, None] * np.float32(0.125)) * (2 * ls + 1)).astype(np.float32)
     assert np.array_equal(alt, dl)
+
+
+def test_iq2_xxs_dequant_structure(oracle):
+    """IQ2_XXS from the format's definition (ggml-common.h:380-384: d, then per 32 values four index bytes and one word of
+    four 7-bit sign indices and a 4-bit scale): |w| = d * (0.5 + s) * 0.25 * g, sign bit j of the sign index, bit 7 the
+    parity of the other seven.  Every codebook index, every sign index and every scale occurs."""
+    rng = np.random.default_rng(16)
+    nb = 256
+    w = synth.constructed_rows(16, 1, 256 * nb, rng).reshape(nb, 66)
+    q = w[:, 2:66].reshape(nb, 8, 8)
+    idx = (np.arange(nb)[:, None, None] + 32 * np.arange(8)[None, :, None] + 7 * np.arange(4)[None, None, :]) % 256
+    sgn = (np.arange(nb)[:, None, None] * 5 + 16 * np.arange(8)[None, :, None] + 37 * np.arange(4)[None, None, :]) % 128
+    scl = (np.arange(nb)[:, None] + np.arange(8)[None, :]) % 16
+    q[:, :, 0:4] = idx.astype(np.uint8)
+    aux = (sgn[:, :, 0] | (sgn[:, :, 1] << 7) | (sgn[:, :, 2] << 14) | (sgn[:, :, 3] << 21) | (scl << 28)).astype(np.uint32)
+    q[:, :, 4:8] = aux[:, :, None].view(np.uint8).reshape(nb, 8, 4)
+    assert len(np.unique(idx)) == 256 and len(np.unique(sgn)) == 128
+    got = oracle.dequant_rows(16, w.reshape(-1), 256 * nb, 1).reshape(nb, 8, 4, 8)
+    grid = np.ctypeslib.as_array(oracle.lib().mo_iq2xxs_grid(), shape=(256,)).view(np.uint8).reshape(256, 8)
+    d = w[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(nb)
+    db = ((d[:, None] * (np.float32(0.5) + scl.astype(np.float32))).astype(np.float32) * np.float32(0.25)).astype(np.float32)
+    parity = np.zeros_like(sgn)
+    for j in range(7):
+        parity ^= (sgn >> j) & 1
+    s8 = sgn | (parity << 7)
+    sign = 1.0 - 2.0 * ((s8[..., None] >> np.arange(8)) & 1).astype(np.float32)
+    want = (db[:, :, None, None] * grid[idx].astype(np.float32)).astype(np.float32) * sign
+    assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # an even number of negative values in every group of 8
+    assert np.all(np.count_nonzero(got < 0, axis=3) % 2 == 0)
 
 
 def test_iq1_dequant_structure(oracle):

@@ -8,7 +8,7 @@ import pytest
 
 import synth
 
-TYPES_256 = (22, 12, 29)
+TYPES_256 = (22, 12, 29, 16)
 
 
 def _acts(oracle, k, nt, seed):
