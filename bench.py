@@ -32,9 +32,9 @@ IQ2_S = 22
 HBM_PEAK = 8.0e12
 PARITY_BAR = 1e-3
 # HBM bytes of one gate/up launch on this workload from rocprofv3's FETCH_SIZE and WRITE_SIZE (two runs, each scaled by
-# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,783.1 KiB read + 64.0 KiB written
+# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,961.4 KiB read + 64.0 KiB written
 # (profiles/decode_iq2s_hbm_traffic_pmc.txt)
-GATE_UP_TRAFFIC_BYTES = int((73783.1 + 64.0) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((73961.4 + 64.0) * 1024)
 
 
 def synth_experts_on_device(torch, n_expert, blob_bytes, seed):
@@ -259,7 +259,7 @@ def decode_iq2s(args, np, torch, lib, L, info):
                                 "one HIP graph of the K steps, replayed back to back (>= 256 steps and >= 10 ms a sample) between "
                                 "two HIP events on the launch stream, median of %d samples after the clocks settled" % bw.ROUNDS),
                    "device": info},
-        "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_pos_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
+        "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_tiles_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
                      "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_s * 1e6, 3),
                      "down_kernel": {"kernel": "down_iq2s_pos_kernel", "achieved": round(dn_rate, 2), "frac": round(dn_rate * 1e9 / HBM_PEAK, 4),
