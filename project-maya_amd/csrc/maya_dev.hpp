@@ -142,6 +142,42 @@ __device__ __forceinline__ void q8k_round_lane32(const float (&v)[32], IndexOf i
     }
 }
 
+// A table of NWORDS 32-bit words from global memory into LDS by a workgroup of NT threads, in 16-byte pieces: every
+// piece a thread moves is REQUESTED before the first one is stored, so the table costs one trip to memory.  (Written as
+// a loop "lds[i] = src[i]; i += NT" the compiler waits for each load before it issues the next: one trip a pass, five
+// for an 8 KB table on 448 threads.)  The request and the store are separate calls so that a kernel can put its other
+// first loads between them.  Source and LDS destination 16-byte aligned.
+template <int NWORDS, int NT>
+struct TablePieces {
+    static_assert(NWORDS % 4 == 0, "whole 16-byte pieces");
+    static constexpr int kPieces = NWORDS / 4, kRounds = (kPieces + NT - 1) / NT;
+    int4 r[kRounds];
+};
+template <int NWORDS, int NT>
+__device__ __forceinline__ void table_request(const void* src, TablePieces<NWORDS, NT>& t) {
+    const int4* s4 = (const int4*) src;
+#pragma unroll
+    for (int i = 0; i < TablePieces<NWORDS, NT>::kRounds; ++i) {
+        const int j = (int) threadIdx.x + i * NT;
+        t.r[i] = (i + 1) * NT <= TablePieces<NWORDS, NT>::kPieces || j < TablePieces<NWORDS, NT>::kPieces ? s4[j] : int4{0, 0, 0, 0};
+    }
+}
+template <int NWORDS, int NT, typename Map>
+__device__ __forceinline__ void table_store(int* lds, const TablePieces<NWORDS, NT>& t, Map map) {
+#pragma unroll
+    for (int i = 0; i < TablePieces<NWORDS, NT>::kRounds; ++i) {
+        const int j = (int) threadIdx.x + i * NT;
+        if ((i + 1) * NT <= TablePieces<NWORDS, NT>::kPieces || j < TablePieces<NWORDS, NT>::kPieces) {
+            const int4 v = t.r[i];
+            ((int4*) lds)[j] = int4{map(v.x), map(v.y), map(v.z), map(v.w)};
+        }
+    }
+}
+template <int NWORDS, int NT>
+__device__ __forceinline__ void table_store(int* lds, const TablePieces<NWORDS, NT>& t) {
+    table_store(lds, t, [](int v) { return v; });
+}
+
 struct Unit32 {
     int q[8];    // 32 int8 codes in value order (the IQ1 types: codes + 9 - delta, see Fmt<kIQ1_S>)
     int s0, s1;  // integer scales of values 0..15 / 16..31

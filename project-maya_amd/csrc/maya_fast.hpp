@@ -86,10 +86,11 @@ __device__ __forceinline__ float row_iq2s(const RawIQ2S (&raw)[KU], const uint2*
 }
 
 // LDS: [0, 2048) words the codebook, [2048, 2560) the sign masks
-__device__ __forceinline__ void stage_iq2s_tables(int* lds, const Codebooks& cb, int nthreads) {
-    const int* src = (const int*) cb.iq2s;
-    for (int i = threadIdx.x; i < 2048; i += nthreads) lds[i] = src[i];
-    for (int i = threadIdx.x; i < 256; i += nthreads) {
+template <int NT>
+__device__ __forceinline__ void stage_iq2s_tables(int* lds, const Codebooks& cb) {
+    TablePieces<2048, NT> t;
+    table_request(cb.iq2s, t);
+    for (int i = threadIdx.x; i < 256; i += NT) {
         uint32_t lo = 0, hi = 0;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
@@ -99,6 +100,7 @@ __device__ __forceinline__ void stage_iq2s_tables(int* lds, const Codebooks& cb,
         lds[2048 + 2 * i] = (int) lo;
         lds[2048 + 2 * i + 1] = (int) hi;
     }
+    table_store(lds, t);
 }
 
 constexpr int kFastLdsWords = 2048 + 512;
@@ -106,10 +108,9 @@ constexpr int kFastLdsWords = 2048 + 512;
 // The position-mapped kernels' form of the second table: per sign byte the two v_perm_b32 selectors that pick, for the
 // eight values it covers, each activation code from y (bit clear) or from the negated copy -y (bit set): selector byte i
 // of a word = i + 4 * bit i.  LDS: [0, 2048) words the codebook, [2048, 2560) the selectors.
-__device__ __forceinline__ void stage_iq2s_tables_sel(int* lds, const Codebooks& cb, int nthreads) {
-    const int* src = (const int*) cb.iq2s;
-    for (int i = threadIdx.x; i < 2048; i += nthreads) lds[i] = src[i];
-    for (int j = threadIdx.x; j < 256; j += nthreads) {
+template <int NT>
+__device__ __forceinline__ void store_iq2s_selectors(int* lds) {
+    for (int j = threadIdx.x; j < 256; j += NT) {
         const int i = j;
         uint32_t lo = 0x03020100u, hi = 0x03020100u;
 #pragma unroll
@@ -120,6 +121,13 @@ __device__ __forceinline__ void stage_iq2s_tables_sel(int* lds, const Codebooks&
         lds[2048 + 2 * j] = (int) lo;
         lds[2048 + 2 * j + 1] = (int) hi;
     }
+}
+template <int NT>
+__device__ __forceinline__ void stage_iq2s_tables_sel(int* lds, const Codebooks& cb) {
+    TablePieces<2048, NT> t;
+    table_request(cb.iq2s, t);
+    store_iq2s_selectors<NT>(lds);
+    table_store(lds, t);
 }
 
 // the lane's slice of an activation row: units sub + LPR j
@@ -142,12 +150,12 @@ __device__ __forceinline__ void load_act_slice(const maya_act& x, int row, int k
 // are fetched while this one is decoded; MINB: waves a SIMD must hold (bounds the registers).
 template <int KU, int ROWS, bool YREG, bool PF, int MINB, bool STREAM>
 __global__ __launch_bounds__(512, MINB) void gate_up_iq2s_1tok_kernel(maya_moe_args a, Codebooks cb) {
-    __shared__ int lds[kFastLdsWords + (YREG ? 0 : KU * 32 * 9)];
+    __shared__ __align__(16) int lds[kFastLdsWords + (YREG ? 0 : KU * 32 * 9)];
     if (a.skip && *a.skip) return;
     const int e = blockIdx.y;  // entry = plan slot (one token)
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
-    stage_iq2s_tables(lds, cb, 512);
+    stage_iq2s_tables<512>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int k = a.layout.n_embd, n_ff = a.layout.n_ff;
@@ -213,10 +221,10 @@ __global__ __launch_bounds__(512, MINB) void gate_up_iq2s_1tok_kernel(maya_moe_a
 // row); the slots' partial rows meet in LDS and are summed in slot order.  n_ff = 1024 KU.
 template <int KU, int ROWS, bool STREAM>
 __global__ __launch_bounds__(512) void down_iq2s_1tok_kernel(maya_moe_args a, Codebooks cb) {
-    __shared__ int lds[kFastLdsWords];
+    __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
-    stage_iq2s_tables(lds, cb, 512);
+    stage_iq2s_tables<512>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int k = a.layout.n_ff, n_embd = a.layout.n_embd;
@@ -405,7 +413,7 @@ template <int NW, int ROWS, int DEPTH, int MINW>
 __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads; the ring holds one or two");
     constexpr int NU = 32 * NW;  // sub-blocks a row
-    __shared__ int lds[kFastLdsWords];
+    __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
     // (a window's entries in the order of grp_ent where one is given: the entries of an expert side by side; -1 ends it)
@@ -413,7 +421,7 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
     if (e < 0) return;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
-    stage_iq2s_tables_sel(lds, cb, 64 * NW);
+    stage_iq2s_tables_sel<64 * NW>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
@@ -472,33 +480,155 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
 }
 
 // ---- gate/up, one token, as a stream of tiles: the same arithmetic as gate_up_iq2s_pos_kernel (a row is the same
-// sequence of operations, so its bits are the same), but the workgroups stay: gridDim.x workgroups - as many as the chip
-// holds at once - walk the (entry, 8-row block) tiles t = blockIdx.x, blockIdx.x + gridDim.x, ... and request the next
-// tile's first rows while they compute this one's.  A workgroup pays the cold start (arguments, plan, tables, first
-// weights: three memory round trips one after the other) once instead of once per 16 rows, and no second round of
-// workgroups starts behind the first.  The plan's blob addresses ride in a register, entry i on lane i.
-template <int NW, int MINW>
-__global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(maya_moe_args a, Codebooks cb) {
+// sequence of operations, so its bits are the same), but the workgroups stay: as many workgroups as the chip holds at
+// once walk the (entry, 8-row block) tiles and request the next tile's first rows while they compute this one's.  A
+// workgroup pays the cold start (arguments, plan, tables, first weights: three memory round trips one after the other)
+// once instead of once per 16 rows, and no second round of workgroups starts behind the first.
+//
+// HEAD: the layer's head rides in the same launch, and no workgroup waits for another.  Workgroup 0 is the router: one
+// wave routes the token exactly (route_wave_softmax) and writes ids, weights and the plan for the down launch and the
+// caller.  Every other workgroup finds out for itself which experts were picked - the order of the k + 1 largest logits
+// (route_wave_order_only; the exact router on its first wave in the rare case that this does not settle it) - and rounds
+// its lanes' share of x to Q8_K in registers (q8k_round_lane32: a 256-value block is 8 lanes), while the tables are
+// staged: the picks cost a workgroup some hundred instructions on one wave, against a launch and two memory round
+// trips between a head kernel and this one.
+struct LayerHead {
+    const float* logits;     // [n_expert]
+    const uint64_t* table;   // [n_expert] blob addresses, 0 = absent
+    int32_t* ids;            // [k]
+    float* weights;          // [k]
+    uint64_t* plan;          // [k]
+    const void* x;           // [n_embd] of x_dtype
+    int n_expert, x_dtype;
+};
+template <int NW, int MINW, bool HEAD>
+__global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(maya_moe_args a, Codebooks cb, LayerHead hd) {
     constexpr int NU = 32 * NW;  // sub-blocks a row
-    __shared__ int lds[kFastLdsWords];
+    __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[2][2 * NW][8];
+    __shared__ uint64_t s_blob[HEAD ? MAYA_MAX_K : 1];
+    __shared__ float s_lv[HEAD ? 256 : 1];              // the picker's scratch: the logits, the table
+    __shared__ uint64_t s_tab[HEAD ? 256 : 1];
+    __shared__ int s_y[HEAD ? 9 : 1][HEAD ? NU : 1];   // a position's codes and scale, from its gate lane to its up lane
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
     const int u = is_up ? t - NU : t;
     const int n_ent = a.k;   // one token: entry = plan slot
-    // everything the first tile needs is requested side by side: no load waits on another
-    const int skipv = a.skip ? *a.skip : 0;
     int y[8];
-    {
-        const int4* q = (const int4*) a.x.q;
-        const int4 ya = q[2 * u], yb = q[2 * u + 1];
-        y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+    float dy8;
+    int first_tile = blockIdx.x, tile_step = gridDim.x;
+    TablePieces<2048, 64 * NW> tp;   // the codebook: requested first, stored once the other first loads are on their way
+    table_request(cb.iq2s, tp);
+    if constexpr (HEAD) {
+        // The workgroup's last wave holds up rows only; it picks the experts while the gate lanes round x (a gate lane and
+        // the up lane of the same position need the same codes: the gate lane rounds, the up lane takes them from LDS).
+        const int ne = hd.n_expert;
+        const bool picker = t >= 64 * (NW - 1);
+        float lv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        uint64_t tab[4] = {0ull, 0ull, 0ull, 0ull};
+        if (picker) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int e = 64 * r + lane;
+                lv[r] = e < ne ? hd.logits[e] : -INFINITY;
+                tab[r] = e < ne ? hd.table[e] : 0ull;
+            }
+        }
+        if (blockIdx.x == 0) {   // the router (it looks at no skip flag, like the head kernel)
+            if (!picker) return;
+            int id;
+            float w;
+            uint64_t ptr;
+            route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+            if (lane < n_ent) {
+                hd.ids[lane] = id;
+                hd.weights[lane] = w;
+                hd.plan[lane] = ptr;
+            }
+            return;
+        }
+        first_tile = (int) blockIdx.x - 1, tile_step = (int) gridDim.x - 1;
+        const int skipv = a.skip ? *a.skip : 0;
+        if (skipv) return;
+        if (picker) {   // (before x is loaded: the values of x then take no registers here)
+            __builtin_amdgcn_s_setprio(3);   // the workgroup waits for this wave: it goes first on its SIMD
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s_tab[64 * r + lane] = tab[r];
+            int id;
+            uint64_t ptr;
+            if (route_wave_order_only(lv, ne, n_ent, s_lv, id)) {
+                ptr = s_tab[lane < n_ent ? id : 0];
+            } else {
+                float w;
+                route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+            }
+            if (lane < n_ent) s_blob[lane] = ptr;
+            __builtin_amdgcn_s_setprio(0);
+        }
+        float v[32];
+        if (!is_up) {
+            if (hd.x_dtype == MAYA_DT_F32) {
+                const float4* xv = (const float4*) hd.x + 8 * u;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float4 q = xv[i];
+                    v[4 * i] = q.x, v[4 * i + 1] = q.y, v[4 * i + 2] = q.z, v[4 * i + 3] = q.w;
+                }
+            } else {
+                const uint4* xv = (const uint4*) hd.x + 4 * u;
+                uint32_t w4[16];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint4 q = xv[i];
+                    w4[4 * i] = q.x, w4[4 * i + 1] = q.y, w4[4 * i + 2] = q.z, w4[4 * i + 3] = q.w;
+                }
+                if (hd.x_dtype == MAYA_DT_BF16) {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        v[2 * j] = __uint_as_float(w4[j] << 16);
+                        v[2 * j + 1] = __uint_as_float(w4[j] & 0xffff0000u);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        v[2 * j] = f16_bits_to_f32((uint16_t) (w4[j] & 0xffffu));
+                        v[2 * j + 1] = f16_bits_to_f32((uint16_t) (w4[j] >> 16));
+                    }
+                }
+            }
+        }
+        store_iq2s_selectors<64 * NW>(lds);
+        table_store(lds, tp);
+        // (a wave with a gate lane rounds: the block's 8 lanes are all gate lanes or all up lanes, NU being a multiple of 8)
+        if (64 * (t >> 6) < NU) {
+            float d;
+            q8k_round_lane32(v, [&](int i) { return 32 * (lane & 7) + i; }, y, d);
+            dy8 = d * 0.125f;
+            if (!is_up) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s_y[i][u] = y[i];
+                s_y[8][u] = __float_as_int(dy8);
+            }
+        }
+        __syncthreads();
+        if (is_up) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = s_y[i][u];
+            dy8 = __int_as_float(s_y[8][u]);
+        }
+    } else {
+        // everything the first tile needs is requested side by side: no load waits on another
+        const int skipv = a.skip ? *a.skip : 0;
+        {
+            const int4* q = (const int4*) a.x.q;
+            const int4 ya = q[2 * u], yb = q[2 * u + 1];
+            y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+        }
+        dy8 = a.x.d[u] * 0.125f;
+        if (skipv) return;
     }
-    const float dy8 = a.x.d[u] * 0.125f;
-    stage_iq2s_tables_sel(lds, cb, 64 * NW);
-    if (skipv) return;
     int yn[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
@@ -508,14 +638,29 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
     const uint32_t gu_bytes = (uint32_t) (a.layout.down_off - a.layout.gate_off);
     const QuadOffs qo = quad_offs<NU>(is_up ? (uint32_t) (a.layout.up_off - a.layout.gate_off) : 0u, u);
     // the resource of a tile's expert (an absent expert: an empty resource, whose loads read as zero and touch nothing);
-    // the entry is the same for the whole workgroup, so its blob address is a scalar load
-    int tile = blockIdx.x;
+    // the entry is the same for the whole workgroup: its blob address is a scalar load (HEAD: read from LDS and moved to
+    // scalar registers)
+    auto blob_of = [&](int e) -> uint64_t {
+        if constexpr (HEAD) {
+            const uint64_t b = s_blob[e];
+            const uint32_t lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) b);
+            const uint32_t hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (b >> 32));
+            return ((uint64_t) hi << 32) | lo;
+        } else {
+            return a.plan_ptr[e];
+        }
+    };
+    int tile = first_tile;
     if (tile >= n_tiles) return;
     int e = tile / tiles_per_entry, rb = tile - e * tiles_per_entry;
-    uint64_t blob = a.plan_ptr[e];
+    uint64_t blob = blob_of(e);
     __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob ? blob + a.layout.gate_off : 0ull, blob ? gu_bytes : 0u);
     QuadIQ2S ring = load_quad(rs, qo, (uint32_t) (2 * rb) * qb);
-    __syncthreads();
+    if constexpr (!HEAD) {
+        store_iq2s_selectors<64 * NW>(lds);
+        table_store(lds, tp);
+        __syncthreads();
+    }
     float acc[8];
     int buf = 0;
     // The ring is consumed in place: a register pair of the quad is requested again, for the quad after, as soon as its
@@ -534,10 +679,10 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
         ring.hs = __builtin_amdgcn_raw_buffer_load_b64(rs, qo.hs, o1, 0);
         ring.d = __builtin_amdgcn_raw_buffer_load_b64(rs, qo.d, o1, 0);
         // the next tile (past the end: the empty resource)
-        const int nt = tile + (int) gridDim.x;
+        const int nt = tile + tile_step;
         const bool more = nt < n_tiles;
         const int ne = more ? nt / tiles_per_entry : 0, nrb = nt - ne * tiles_per_entry;
-        const uint64_t pblob = a.plan_ptr[ne];
+        const uint64_t pblob = blob_of(ne);
         const uint64_t nblob = more ? pblob : 0ull;
         const __amdgpu_buffer_rsrc_t nrs = weight_rsrc(nblob ? nblob + a.layout.gate_off : 0ull, nblob ? gu_bytes : 0u);
         const uint32_t o2 = (uint32_t) (2 * nrb) * qb;
@@ -573,7 +718,7 @@ template <int ROWS, int DEPTH, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 4 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads (the last may be one); the ring holds one or two");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
-    __shared__ int lds[kFastLdsWords];
+    __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[8][ROWS];
     __shared__ float s_w[8];
     __shared__ int s_on[8];
@@ -589,6 +734,8 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     // flag, the plan (the wave's slot; the slots' presence and weights for the combine), the slot's h and the tables.
     // A wave past slot k - 1 reads that slot's data and drops it: no branch, and no load waits on another.
     const int skipv = a.skip ? *a.skip : 0;
+    TablePieces<2048, 512> tp;
+    table_request(cb.iq2s, tp);
     const int ent = e0 + min(wave, a.k - 1);
     uint64_t blob = a.plan_ptr[ent];
     const int ci = e0 + min((int) threadIdx.x & 7, a.k - 1);
@@ -613,29 +760,31 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
             v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
         }
     }
-    stage_iq2s_tables_sel(lds, cb, 512);
+    if (skipv) return;
+    if (wave >= a.k) blob = 0ull;
+    constexpr uint32_t qb = NU / 8 * 82 * 4;
+    // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
+    // scalar registers for the buffer resource (no blob: an empty resource, whose loads read as zero and touch nothing)
+    const uint64_t mat = blob ? blob + a.layout.down_off : 0ull;
+    const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
+    const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
+    const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (mat_lo | mat_hi) != 0u ? (uint32_t) (n_embd >> 2) * qb : 0u);
+    const QuadOffs qo = quad_offs<NU>(0u, pos);
+    const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
+    constexpr int NQ = ROWS / 4;
+    // the first rows' weights are requested before the tables are stored and h is rounded: one trip to memory for the
+    // tables, the plan and h, a second for the weights, and the barrier and the rounding sit under the second
+    QuadIQ2S ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
+    store_iq2s_selectors<512>(lds);
+    table_store(lds, tp);
     if (threadIdx.x < 8) {
         s_on[threadIdx.x] = (int) threadIdx.x < a.k && c_ptr != 0ull;
         s_w[threadIdx.x] = c_w;
     }
     __syncthreads();
-    if (skipv) return;
-    if (wave >= a.k) blob = 0ull;
     if (blob != 0ull) {
-        constexpr uint32_t qb = NU / 8 * 82 * 4;
-        // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
-        // scalar registers for the buffer resource
-        const uint64_t mat = blob + a.layout.down_off;
-        const uint32_t mat_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) mat);
-        const uint32_t mat_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (mat >> 32));
-        const __amdgpu_buffer_rsrc_t rs = weight_rsrc(((uint64_t) mat_hi << 32) | (uint64_t) mat_lo, (uint32_t) (n_embd >> 2) * qb);
-        const QuadOffs qo = quad_offs<NU>(0u, pos);
-        const uint32_t quad0 = (uint32_t) (r0 >> 2) * qb;
-        constexpr int NQ = ROWS / 4;
-        // the first rows' weights are requested before h is rounded: their latency hides behind that arithmetic
-        QuadIQ2S ring[DEPTH];
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) ring[d] = load_quad(rs, qo, quad0 + (uint32_t) d * qb);
         if (rounded) {
             if (!on) {
 #pragma unroll

@@ -18,13 +18,15 @@
 
 namespace maya {
 
-__device__ __forceinline__ void stage_iq1s_table(int* lds, const Codebooks& cb, int nthreads) {
-    const uint32_t* src = (const uint32_t*) cb.iq1s;
-    for (int i = threadIdx.x; i < 4096; i += nthreads) {
-        const uint32_t g = src[i];
+template <int NT>
+__device__ __forceinline__ void stage_iq1s_table(int* lds, const Codebooks& cb) {
+    TablePieces<4096, NT> t;
+    table_request(cb.iq1s, t);
+    table_store(lds, t, [](int w) {
+        const uint32_t g = (uint32_t) w;
         const uint32_t neg = (g >> 1) & 0x01010101u, pos = g & ~(g >> 1) & 0x01010101u;
-        lds[i] = (int) (0x09090909u + (pos << 3) - (neg << 3));
-    }
+        return (int) (0x09090909u + (pos << 3) - (neg << 3));
+    });
 }
 constexpr int kFast1LdsWords = 4096;
 
@@ -86,13 +88,13 @@ template <int NW, int ROWS, int MINW>
 __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
     constexpr int NU = 32 * NW;
-    __shared__ int lds[kFast1LdsWords];
+    __shared__ __align__(16) int lds[kFast1LdsWords];
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
     const int e = blockIdx.y;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
-    stage_iq1s_table(lds, cb, 64 * NW);
+    stage_iq1s_table<64 * NW>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
@@ -151,10 +153,10 @@ template <int ROWS, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
-    __shared__ int lds[kFast1LdsWords];
+    __shared__ __align__(16) int lds[kFast1LdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
-    stage_iq1s_table(lds, cb, 512);
+    stage_iq1s_table<512>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -311,13 +313,13 @@ template <int NW, int ROWS, int MINW>
 __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1m_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
     constexpr int NU = 32 * NW;
-    __shared__ int lds[kFast1LdsWords];
+    __shared__ __align__(16) int lds[kFast1LdsWords];
     __shared__ float part[2][2 * NW][8];
     if (a.skip && *a.skip) return;
     const int e = blockIdx.y;
     const uint64_t blob = a.plan_ptr[e];
     if (blob == 0ull) return;
-    stage_iq1s_table(lds, cb, 64 * NW);
+    stage_iq1s_table<64 * NW>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
@@ -378,10 +380,10 @@ template <int ROWS, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq1m_pos_kernel(maya_moe_args a, Codebooks cb) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
-    __shared__ int lds[kFast1LdsWords];
+    __shared__ __align__(16) int lds[kFast1LdsWords];
     __shared__ float part[8][ROWS];
     if (a.skip && *a.skip) return;
-    stage_iq1s_table(lds, cb, 512);
+    stage_iq1s_table<512>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;

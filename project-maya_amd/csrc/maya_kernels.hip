@@ -817,6 +817,72 @@ __device__ __forceinline__ void route_any(const float* __restrict__ l, int n_exp
     else route_token<NTH>(l, n_expert, k, sm);
 }
 
+// The softmax router on ONE wave, nothing but registers (up to 256 experts, 4 a lane: lane L holds experts L, L + 64, ...;
+// lv = -inf and tab = 0 past the end): the maximum, the exponentials, then route_narrow_regs.  Lane i < k returns slot i.
+__device__ __forceinline__ void route_wave_softmax(const float (&lv)[4], const uint64_t (&tab)[4], int n_expert, int k, int& id,
+                                                   float& w, uint64_t& ptr) {
+    const int lane = threadIdx.x & 63;
+    float mx = fmaxf(fmaxf(lv[0], lv[1]), fmaxf(lv[2], lv[3]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    double ex[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ex[r] = 64 * r + lane < n_expert ? exp((double) lv[r] - (double) mx) : 0.0;
+    route_narrow_regs(n_expert, k, ex, tab, id, w, ptr);
+}
+
+// Which k experts the softmax router picks, and in which order, WITHOUT the probabilities: p = exp(l - max) / sum grows
+// with the logit, so the k largest logits in descending order are the k largest probabilities in descending order as long
+// as rounding cannot merge or reorder two of them.  Two logits more than 1e-6 apart give probabilities whose ratio
+// exceeds 1 + 1e-6, far beyond the 2^-24 relative rounding of a float, and a probability within e^-60 of the largest
+// is a normal float.  So: every logit finite, each pick more than 1e-6 above the next, the k-th more than 1e-6 above
+// everything not picked, and all of that within 60 of the first - then the picks and their order are the exact router's.
+// Anything else (ties, near ties, the sub-normal range, NaN / Inf) returns false and the caller runs the exact router.
+//
+// A round must be short (k + 1 of them run one after the other on one wave while its workgroup waits), so a key is one
+// word that names its expert: the logit's ordered bits with the low byte replaced by 255 - index.  The largest key of
+// the wave IS the pick, with no search for the lane that holds it.  The 8 bits given up make picks inside one
+// 256-ulp bucket come out in index order: the check below therefore compares the picks' TRUE logits (a wrong order
+// shows as a negative gap), and holds the k-th pick against the upper end of the (k + 1)-th pick's bucket, above which
+// nothing unpicked can lie.  One wave, k < n_expert <= 256, k + 1 <= 64; s_lv [256] floats of LDS scratch; lane i < k
+// gets slot i's expert.
+__device__ __forceinline__ bool route_wave_order_only(const float (&lv)[4], int n_expert, int k, float* s_lv, int& my_id) {
+    const int lane = threadIdx.x & 63;
+    constexpr int kNone = (int) 0x80000000;
+    int k0, k1, k2, k3;
+    bool fin = true;
+    {
+        int key[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int e = 64 * r + lane;
+            const bool have = e < n_expert;
+            key[r] = have ? (int) (((uint32_t) float_order_key(lv[r]) & 0xffffff00u) | (uint32_t) (255 - e)) : kNone;
+            fin = fin && (!have || isfinite(lv[r]));
+            s_lv[e] = lv[r];
+        }
+        k0 = key[0], k1 = key[1], k2 = key[2], k3 = key[3];
+    }
+    int my_key = kNone;
+    for (int i = 0; i <= k; ++i) {
+        const int top = wave_max_i32(max(max(k0, k1), max(k2, k3)));
+        k0 = k0 == top ? kNone : k0;
+        k1 = k1 == top ? kNone : k1;
+        k2 = k2 == top ? kNone : k2;
+        k3 = k3 == top ? kNone : k3;
+        my_key = lane == i ? top : my_key;
+    }
+    const int id = 255 - (my_key & 255);
+    const float val = lane <= k ? s_lv[id] : 0.0f;
+    const int ub_key = my_key | 255;
+    const float ub = __int_as_float(ub_key >= 0 ? ub_key : ub_key ^ 0x7fffffff);   // the bucket's upper end
+    const float nxt = __shfl_down(lane == k ? ub : val, 1, kWave);
+    const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(val), 0));
+    const bool apart = lane >= k || (val - nxt > 1e-6f && first - nxt <= 60.0f);
+    my_id = id;
+    return __all(fin && apart) != 0;
+}
+
 __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec r,
                                                      int32_t* __restrict__ ids, float* __restrict__ weights) {
     __shared__ RouterLds sm;
@@ -965,23 +1031,16 @@ __global__ __launch_bounds__(256) void window_head_kernel(const float* __restric
             const float* l = logits + (size_t) t * n_expert;
             float lv[4];
             uint64_t tab[4];
-            float mx = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int e = 64 * r + lane;
                 lv[r] = e < n_expert ? l[e] : -INFINITY;
                 tab[r] = e < n_expert ? table[e] : 0ull;
-                mx = fmaxf(mx, lv[r]);
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
-            double ex[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) ex[r] = 64 * r + lane < n_expert ? exp((double) lv[r] - (double) mx) : 0.0;
             int id;
             float w;
             uint64_t ptr;
-            route_narrow_regs(n_expert, k, ex, tab, id, w, ptr);
+            route_wave_softmax(lv, tab, n_expert, k, id, w, ptr);
             if (lane < k) {
                 ids[(size_t) t * k + lane] = id;
                 weights[(size_t) t * k + lane] = w;
@@ -1107,19 +1166,20 @@ template <int TYPE> __device__ __forceinline__ const uint64_t* codebook_of(const
 }
 
 // a type's codebook into LDS; the IQ1 grid (bytes -1 / 0 / +1) as 8 g + 9 (see Fmt<kIQ1_S>)
-template <int TYPE>
-__device__ __forceinline__ void stage_codebook(int* lds, const Codebooks& cb, int nthreads) {
+template <int TYPE, int NT>
+__device__ __forceinline__ void stage_codebook(int* lds, const Codebooks& cb) {
     constexpr int n = Fmt<TYPE>::kLdsWords;
     if constexpr (n > 0) {
-        const uint32_t* src = (const uint32_t*) codebook_of<TYPE>(cb);
-        for (int i = threadIdx.x; i < n; i += nthreads) {
-            uint32_t g = src[i];
+        TablePieces<n, NT> t;
+        table_request(codebook_of<TYPE>(cb), t);
+        table_store(lds, t, [](int w) {
+            uint32_t g = (uint32_t) w;
             if constexpr (Fmt<TYPE>::kBiased) {
                 const uint32_t neg = (g >> 1) & 0x01010101u, pos = g & ~(g >> 1) & 0x01010101u;
                 g = 0x09090909u + (pos << 3) - (neg << 3);
             }
-            lds[i] = (int) g;
-        }
+            return (int) g;
+        });
     }
 }
 
@@ -1188,15 +1248,15 @@ inline int rows_per_wg(int n_rows, int entries, int unit, int most) {
 // grid (n_ff / kGuRows, groups): wave w takes row pairs w, w + 8, ...: lanes 0..31 the gate row, 32..63 the up row
 template <int TG, int TU, int NT>
 __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Codebooks cb, int wg_rows) {
-    extern __shared__ int lds[];
+    extern __shared__ __align__(16) int lds[];
     GroupRef gr;
     if (!group_of(a, blockIdx.y, gr)) return;
     const int k = a.layout.n_embd, n_ff = a.layout.n_ff;
     // the codebooks of the gate and of the up type (one copy when they share it)
     constexpr int cbg = Fmt<TG>::kLdsWords, cbu = Fmt<TG>::kLdsWords == Fmt<TU>::kLdsWords ? 0 : Fmt<TU>::kLdsWords;
     constexpr int cbw = cbg + cbu;
-    stage_codebook<TG>(lds, cb, kGuThreads);
-    if constexpr (cbu > 0) stage_codebook<TU>(lds + cbg, cb, kGuThreads);
+    stage_codebook<TG, kGuThreads>(lds, cb);
+    if constexpr (cbu > 0) stage_codebook<TU, kGuThreads>(lds + cbg, cb);
     const uint2* grid_g = (const uint2*) lds;
     const uint2* grid_u = (const uint2*) (lds + (cbu > 0 ? cbg : 0));
     int* lds_act = lds + cbw;
@@ -1248,12 +1308,12 @@ __global__ __launch_bounds__(kGuThreads) void gate_up_kernel(maya_moe_args a, Co
 // row over lanes, so a window's rows get the token path's bits)
 template <int TD, int NT>
 __global__ __launch_bounds__(kDnThreads) void down_kernel(maya_moe_args a, Codebooks cb, int wg_rows) {
-    extern __shared__ int lds[];
+    extern __shared__ __align__(16) int lds[];
     GroupRef gr;
     if (!group_of(a, blockIdx.y, gr)) return;
     const int k = a.layout.n_ff, n_embd = a.layout.n_embd;
     constexpr int cbw = Fmt<TD>::kLdsWords;
-    stage_codebook<TD>(lds, cb, kDnThreads);
+    stage_codebook<TD, kDnThreads>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     int* lds_act = lds + cbw;
     const int kq = k >> 2, kd = k >> 5;
@@ -1322,12 +1382,12 @@ struct MvBatch {
 };
 template <int T, int NT>
 __global__ __launch_bounds__(kDnThreads) void mv_kernel(MvBatch b, Codebooks cb, int wg_rows) {
-    extern __shared__ int lds[];
+    extern __shared__ __align__(16) int lds[];
     const MvJobDev& j = b.job[blockIdx.y];
     const int k = j.n_in, n_out = j.n_out;
     if ((int) blockIdx.x * wg_rows >= n_out) return;
     constexpr int cbw = Fmt<T>::kLdsWords;
-    stage_codebook<T>(lds, cb, kDnThreads);
+    stage_codebook<T, kDnThreads>(lds, cb);
     const uint2* grid = (const uint2*) lds;
     int* lds_act = lds + cbw;
     const int kq = k >> 2, kd = k >> 5;
@@ -1471,18 +1531,45 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 // shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
 // tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
 template <int NW>
-int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hipStream_t s, const LayerHead* hd = nullptr) {
     static int per_cu = 0;
     if (per_cu == 0) {
-        int n = 0;
-        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gate_up_iq2s_tiles_kernel<NW, 8>, 64 * NW, 0));
+        int n = 0, m = 0;
+        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gate_up_iq2s_tiles_kernel<NW, 8, false>, 64 * NW, 0));
+        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, gate_up_iq2s_tiles_kernel<NW, 8, true>, 64 * NW, 0));
+        n = m < n ? m : n;
         per_cu = n > 3 ? 3 : n > 0 ? n : 1;
     }
     const int n_tiles = a.k * (a.layout.n_ff / 8);
     const int wgs = per_cu * st.n_cu;
-    hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8>), dim3((unsigned) (wgs < n_tiles ? wgs : n_tiles)), dim3(64 * NW), 0, s, a, st.cb);
+    const unsigned walkers = (unsigned) (wgs < n_tiles ? wgs : n_tiles);
+    if (hd) {   // workgroup 0 routes, the others walk the tiles
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, a, st.cb, *hd);
+    } else {
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, false>), dim3(walkers), dim3(64 * NW), 0, s, a, st.cb, LayerHead{});
+    }
     MAYA_LAUNCHED("gate_up_iq2s_tiles_kernel");
     return MAYA_OK;
+}
+// The single-token IQ2_S layer whose head rides in the gate/up launch (gate_up_iq2s_tiles_kernel<.., true>): the softmax
+// router over up to 256 experts with more experts than slots, x aligned for 16-byte loads, the stream packing's shapes.
+static bool layer_head_in_gate_up_ok(const maya_moe_args& a, const RouterSpec& rs, const float* logits, int n_expert, const void* x,
+                                     int x_dtype) {
+    const maya_moe_layout& l = a.layout;
+    return logits && a.n_tokens == 1 && rs.kind == MAYA_ROUTER_SOFTMAX && n_expert <= 256 && a.k < n_expert && x_dtype >= 0 &&
+           x_dtype <= 2 && ((uintptr_t) x & 15) == 0 && l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM &&
+           l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 && l.n_embd >= 2048 && l.n_embd <= 8192;
+}
+static int launch_layer_gate_up_iq2s(const maya_moe_args& a, const LayerHead& hd, const DeviceState& st, hipStream_t s) {
+    switch (a.layout.n_embd / 1024) {
+        case 2: return launch_gate_up_iq2s_tiles<2>(a, st, s, &hd);
+        case 3: return launch_gate_up_iq2s_tiles<3>(a, st, s, &hd);
+        case 4: return launch_gate_up_iq2s_tiles<4>(a, st, s, &hd);
+        case 5: return launch_gate_up_iq2s_tiles<5>(a, st, s, &hd);
+        case 6: return launch_gate_up_iq2s_tiles<6>(a, st, s, &hd);
+        case 7: return launch_gate_up_iq2s_tiles<7>(a, st, s, &hd);
+        default: return launch_gate_up_iq2s_tiles<8>(a, st, s, &hd);
+    }
 }
 // the rows the position-mapped down kernels take on one wave: n_ff = 1024, 1536 or 2048
 static bool down_pos_nff_ok(int n_ff) { return n_ff == 1024 || n_ff == 1536 || n_ff == 2048; }
@@ -2453,8 +2540,13 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
                                     workspace, workspace_bytes, *st, rs, w, a))
         return rc0;
     int rc;
-    bool grouped = false;
-    if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
+    bool grouped = false, gate_up_done = false;
+    if (layer_head_in_gate_up_ok(a, rs, logits, n_expert, x, x_dtype)) {
+        // one token of IQ2_S experts: route, plan, Q8_K of x and gate/up in one launch
+        const LayerHead hd{logits, expert_table, ids, weights, w.plan_ptr, x, n_expert, x_dtype};
+        if ((rc = launch_layer_gate_up_iq2s(a, hd, *st, as_stream(stream)))) return rc;
+        gate_up_done = true;
+    } else if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
         n_tokens <= kWindowHeadTokens && maya_moe_route_window_ok(router, n_tokens, n_expert, k)) {
         // a window, one launch: route every token, plan, group, Q8_K of x
         const dim3 grid((unsigned) (1 + l->n_embd / 256), (unsigned) n_tokens);
@@ -2499,7 +2591,7 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
             a.n_groups = w.n_groups;
         }
     }
-    if ((rc = maya_moe_gate_up(&a, stream))) return rc;
+    if (!gate_up_done && (rc = maya_moe_gate_up(&a, stream))) return rc;
     if (down_rounds_h(a)) {
         a.hq = maya_act{nullptr, nullptr, nullptr};
         a.part = nullptr;

@@ -1,0 +1,179 @@
+"""GPU parity of the single-token IQ2_S layer whose head rides in the gate/up launch: every gate/up workgroup picks the
+token's experts from the ORDER of the logits and rounds x itself, so the cases here are the ones where the order of the
+logits and the order of the rounded probabilities can differ (ties, near ties, probabilities in the sub-normal range,
+NaN / Inf) - the layer must give the ids, weights and output, bit for bit, of the layer that routes with the exact
+router in a launch of its own.  That layer is reached by handing x over at an address that is not 16-byte aligned."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev, make_experts, oracle_layer, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+N_EMBD, N_FF, NE, K = 2048, 512, 40, 8
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from maya_amd import lib as L
+    L.load()
+    return L
+
+
+@pytest.fixture(scope="module")
+def layer(lib):
+    blobs = make_experts(22, 22, N_EMBD, N_FF, NE, 77)
+    gguf_layout, _ = lib.layout(22, 22, N_EMBD, N_FF)
+    store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+    return blobs, store, lib.MoeLayer(22, 22, N_EMBD, N_FF, NE, K, packing=1), lib.MoeLayer(22, 22, N_EMBD, N_FF, NE, K, packing=1)
+
+
+def logit_cases():
+    rng = np.random.default_rng(5)
+    base = rng.standard_normal(NE).astype(np.float32)
+    cases = {"random": base.copy()}
+    c = base.copy()
+    c[[31, 7, 19]] = np.float32(2.5)           # three equal logits at the top: the lower index first
+    cases["ties at the top"] = c
+    c = base.copy()
+    order = np.argsort(-c)
+    c[order[8]] = c[order[7]]                  # the 8th and 9th equal: the lower index is in, the other out
+    cases["tie at the cut"] = c
+    c = base.copy()
+    c[order[3]] = np.nextafter(c[order[2]], np.float32(-10))   # one unit in the last place apart
+    c[order[8]] = np.nextafter(c[order[7]], np.float32(-10))
+    cases["one ulp apart"] = c
+    c = np.zeros(NE, dtype=np.float32)
+    c[5] = -0.0
+    c[9] = -0.0
+    cases["all equal, signed zeros"] = c
+    c = base.copy()
+    c[17] = np.float32(300.0)                  # every other probability underflows to zero: ties at p = 0
+    cases["one logit far above"] = c
+    c = (base * np.float32(40.0)).astype(np.float32)   # probabilities down to the sub-normal range
+    cases["wide range"] = c
+    c = base.copy()
+    c[11] = np.float32(np.inf)
+    cases["+inf"] = c
+    c = base.copy()
+    c[3] = np.float32(-np.inf)
+    cases["-inf"] = c
+    c = base.copy()
+    c[20] = np.float32(np.nan)
+    cases["nan"] = c
+    c = np.arange(NE, dtype=np.float32) * np.float32(5e-7)   # a ladder of steps below the bar
+    cases["ladder below the bar"] = c
+    return cases
+
+
+@pytest.mark.parametrize("dtype", (torch.float32, torch.bfloat16, torch.float16))
+def test_head_in_the_gate_up_launch_is_the_exact_router(lib, oracle, layer, dtype):
+    blobs, store, fused, plain = layer
+    rng = np.random.default_rng(9)
+    x32 = rng.standard_normal(N_EMBD).astype(np.float32)
+    x32[256:512] = 0.0                                          # a block of zeros
+    x32[600], x32[700] = 9.0, -9.0                              # equal magnitudes of either sign: the first one's sign
+    xa = torch.zeros(N_EMBD + 16, dtype=dtype, device="cuda")
+    off = 8 // xa.element_size()                                # 8 bytes off a 16-byte boundary
+    x_al = xa[:N_EMBD].view(1, N_EMBD)
+    x_un = xa[off:off + N_EMBD].view(1, N_EMBD)
+    assert x_al.data_ptr() % 16 == 0 and x_un.data_ptr() % 16 == 8
+    for name, lg in logit_cases().items():
+        print("case", name, dtype, flush=True)
+        logits = dev(lg.reshape(1, NE))
+        x_al.copy_(torch.from_numpy(x32).to(dtype).view(1, -1))
+        out_f = fused.forward(store.table, logits, x_al).clone()
+        ids_f, w_f = fused.ids.clone(), fused.weights.clone()
+        x_un.copy_(torch.from_numpy(x32).to(dtype).view(1, -1))
+        out_p = plain.forward(store.table, logits, x_un).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(ids_f, plain.ids), (name, ids_f, plain.ids)
+        assert torch.equal(w_f.view(torch.int32), plain.weights.view(torch.int32)), name
+        assert torch.equal(out_f.view(torch.int32), out_p.view(torch.int32)), name
+    # and against the CPU path on the plain case
+    lg = logit_cases()["random"].reshape(1, NE)
+    xin = torch.from_numpy(x32).to(dtype)
+    out = fused.forward(store.table, dev(lg), xin.cuda().view(1, -1)).cpu().numpy()
+    wi, ww, wout = oracle_layer(oracle, 22, 22, blobs, K, N_EMBD, N_FF, lg, xin.float().numpy().reshape(1, -1))
+    assert np.array_equal(fused.ids.cpu().numpy(), wi) and rel_l2(out[0], wout[0]) <= 1e-3
+
+
+def test_absent_experts_and_k_next_to_the_expert_count(lib, oracle):
+    """k = n_expert - 1 (the order-only pick needs one expert beyond the slots) and k = n_expert (the head then stays a
+    launch of its own); experts missing from the table give no contribution on either path."""
+    n_embd, n_ff = 2048, 512
+    for ne, k in ((5, 4), (4, 4), (9, 8)):
+        blobs = make_experts(22, 22, n_embd, n_ff, ne, 90 + ne)
+        gguf_layout, _ = lib.layout(22, 22, n_embd, n_ff)
+        store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+        table = store.table.clone()
+        table[1] = 0
+        rng = np.random.default_rng(ne)
+        logits = dev(rng.standard_normal((1, ne)).astype(np.float32))
+        xa = torch.zeros(n_embd + 8, dtype=torch.float32, device="cuda")
+        x32 = torch.from_numpy(rng.standard_normal(n_embd).astype(np.float32)).cuda()
+        a, b = lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1), lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1)
+        x_al, x_un = xa[:n_embd].view(1, -1), xa[2:2 + n_embd].view(1, -1)
+        x_al.copy_(x32.view(1, -1))
+        out_a = a.forward(table, logits, x_al).clone()
+        x_un.copy_(x32.view(1, -1))
+        out_b = b.forward(table, logits, x_un).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a.ids, b.ids) and torch.equal(a.weights.view(torch.int32), b.weights.view(torch.int32))
+        assert torch.equal(out_a.view(torch.int32), out_b.view(torch.int32)), (ne, k)
+        assert float(out_a.abs().max()) > 0
+
+
+def test_order_only_pick_against_the_exact_router_on_adversarial_rows(lib):
+    """Rows built to sit on the order-only pick's edges: values on a coarse grid (many exact ties), values a few units in
+    the last place apart at magnitudes from 1e-3 to 1e3 and of either sign (one 256-ulp bucket holds several), steps just
+    under and just over the 1e-6 bar, everything within 1e-6 of zero.  ids and weights must be the exact router's
+    (maya_moe_route_topk), and the output - which depends on what the gate/up workgroups picked for themselves - the
+    output of the layer that routes in a launch of its own (x handed over unaligned), all bit for bit."""
+    n_embd, n_ff, ne, k = 2048, 512, 256, 8
+    blobs = make_experts(22, 22, n_embd, n_ff, ne, 123)
+    gguf_layout, _ = lib.layout(22, 22, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+    fused, plain = lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1), lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1)
+    xa = torch.zeros(n_embd + 8, dtype=torch.float32, device="cuda")
+    x32 = torch.randn(n_embd, device="cuda")
+    x_al, x_un = xa[:n_embd].view(1, -1), xa[2:2 + n_embd].view(1, -1)
+    rng = np.random.default_rng(2024)
+    rows = []
+    for trial in range(25):
+        base = rng.standard_normal(ne).astype(np.float32)
+        rows.append(base)
+        rows.append((np.round(base * 4) / 4).astype(np.float32))              # a coarse grid: ties everywhere
+        for mag in (1e-3, 0.3, 1.0, 3.0, 50.0, 1e3):
+            for sign in (1.0, -1.0):
+                c = (-np.abs(base) * np.float32(mag) - np.float32(2 * mag)).astype(np.float32)
+                top = rng.permutation(ne)[:12]
+                steps = rng.integers(0, 6, size=12)                           # 0 .. 5 ulps apart, some equal
+                v = np.float32(sign * mag)
+                for j, st in zip(top, steps):
+                    c[j] = v
+                    for _ in range(int(st)):
+                        v = np.nextafter(v, np.float32(-np.inf))
+                rows.append(c)
+        c = base.copy()
+        top = np.argsort(-c)[:10]
+        c[top] = np.float32(1.0) - np.arange(10, dtype=np.float32) * np.float32(rng.choice([0.9e-6, 1.1e-6, 2e-6]))
+        rows.append(c)
+        rows.append((base * np.float32(1e-7)).astype(np.float32))             # everything within 1e-6 of zero, both signs
+    rows = np.stack(rows).astype(np.float32)
+    want_ids, want_w = lib.route_topk(dev(rows), k)
+    bad = 0
+    for i in range(rows.shape[0]):
+        lg = dev(rows[i:i + 1])
+        x_al.copy_(x32.view(1, -1))
+        out_f = fused.forward(store.table, lg, x_al).clone()
+        x_un.copy_(x32.view(1, -1))
+        out_p = plain.forward(store.table, lg, x_un)
+        ok = (torch.equal(fused.ids[0], want_ids[i]) and torch.equal(fused.weights[0].view(torch.int32), want_w[i].view(torch.int32))
+              and torch.equal(plain.ids[0], want_ids[i]) and torch.equal(out_f.view(torch.int32), out_p.view(torch.int32)))
+        if not ok:
+            bad += 1
+            print("row", i, fused.ids[0].tolist(), want_ids[i].tolist(), flush=True)
+    torch.cuda.synchronize()
+    assert bad == 0, bad
