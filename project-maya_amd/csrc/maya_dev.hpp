@@ -34,6 +34,13 @@ __device__ __forceinline__ uint32_t ld32_a2(const uint8_t* p) { return *(const u
 __device__ __forceinline__ uint32_t ld16(const uint8_t* p) { return *(const uint16_t*) p; }
 
 __device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+// a . b alone: the three-operand encoding with a literal zero as the addend (the compiler's own choice for
+// dot4(a, b, 0) is the two-operand accumulate form behind a v_mov of zero: one instruction more)
+__device__ __forceinline__ int dot4_first(int a, int b) {
+    int d;
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
 
 // sum over the lanes of an aligned group of `width` lanes (a power of two <= 64); every lane gets the sum
 template <int WIDTH>

@@ -367,6 +367,9 @@ __device__ __forceinline__ RawIQ2S quad_row(const QuadIQ2S& q) {
 // the weight: v_perm_b32 over the pair (-y word, y word) with the sign byte's selector takes -y_i where value i is
 // negative, and the codebook word meets it in one dot4 - two instructions per four weights, no xor, no mask term.
 // dy8 = the activation scale / 8.
+// Z3: the first product of a sum in the three-operand encoding (dot4_first): one instruction less a sum; it pays in
+// the down kernel and costs in the gate/up kernels (measured: their register count goes from 57 to 64).
+template <bool Z3 = false>
 __device__ __forceinline__ float unit_value(const RawIQ2S& r, const uint2* grid, const uint2* ssel, const int (&y)[8],
                                             const int (&yn)[8], float dy8) {
     int t0 = 0, t1 = 0;
@@ -377,13 +380,12 @@ __device__ __forceinline__ float unit_value(const RawIQ2S& r, const uint2* grid,
         const uint2 sl = ssel[(r.sg4 >> (8 * l)) & 255u];
         const int ya = (int) __builtin_amdgcn_perm((uint32_t) yn[2 * l], (uint32_t) y[2 * l], sl.x);
         const int yb = (int) __builtin_amdgcn_perm((uint32_t) yn[2 * l + 1], (uint32_t) y[2 * l + 1], sl.y);
-        if (l < 2) {
-            t0 = dot4((int) g.x, ya, t0);
-            t0 = dot4((int) g.y, yb, t0);
-        } else {
-            t1 = dot4((int) g.x, ya, t1);
-            t1 = dot4((int) g.y, yb, t1);
-        }
+        if (Z3 && l == 0) t0 = dot4_first((int) g.x, ya);
+        else if (Z3 && l == 2) t1 = dot4_first((int) g.x, ya);
+        else if (l < 2) t0 = dot4((int) g.x, ya, t0);
+        else t1 = dot4((int) g.x, ya, t1);
+        if (l < 2) t0 = dot4((int) g.y, yb, t0);
+        else t1 = dot4((int) g.y, yb, t1);
     }
     const int s0 = 2 * (int) ((r.hs >> 8) & 15u) + 1, s1 = 2 * (int) ((r.hs >> 12) & 15u) + 1;
     const int isum = __mul24(s0, t0) + __mul24(s1, t1);
@@ -396,11 +398,11 @@ __device__ __forceinline__ int neg4(int v) {
 }
 // the four rows of a quad: acc[B + r] = this lane's value for row r.  Each value is pinned where it is made: without
 // that the optimizer sinks all the batch's decodes down to the reduction and keeps every prefetched quad live.
-template <int B>
+template <int B, bool Z3 = false>
 __device__ __forceinline__ void quad_values(const QuadIQ2S& q, const uint2* grid, const uint2* stab, const int (&y)[8],
                                             const int (&yn)[8], float dy8, float (&acc)[8]) {
 #define MAYA_ROW(R)                                                              \
-    acc[B + R] = unit_value(quad_row<R>(q), grid, stab, y, yn, dy8);             \
+    acc[B + R] = unit_value<Z3>(quad_row<R>(q), grid, stab, y, yn, dy8);         \
     asm volatile("" : "+v"(acc[B + R]));                                         \
     __builtin_amdgcn_sched_barrier(0);
     MAYA_ROW(0) MAYA_ROW(1) MAYA_ROW(2) MAYA_ROW(3)
@@ -519,8 +521,8 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
     int y[8];
     float dy8;
     int first_tile = blockIdx.x, tile_step = gridDim.x;
-    TablePieces<2048, 64 * NW> tp;   // the codebook: requested first, stored once the other first loads are on their way
-    table_request(cb.iq2s, tp);
+    TablePieces<2048, 64 * NW> tp;   // the codebook: requested early, stored once the other first loads are on their way
+    if constexpr (!HEAD) table_request(cb.iq2s, tp);
     if constexpr (HEAD) {
         // The workgroup's last wave holds up rows only; it picks the experts while the gate lanes round x (a gate lane and
         // the up lane of the same position need the same codes: the gate lane rounds, the up lane takes them from LDS).
@@ -536,6 +538,7 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
                 tab[r] = e < ne ? hd.table[e] : 0ull;
             }
         }
+        table_request(cb.iq2s, tp);   // (behind the picker's loads: loads come back in the order they were asked for)
         if (blockIdx.x == 0) {   // the router (it looks at no skip flag, like the head kernel)
             if (!picker) return;
             int id;
@@ -716,7 +719,7 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
 // meet in LDS and are summed in slot order.
 template <int ROWS, int DEPTH, int MINW, int NU = 64>
 __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
-    static_assert(ROWS % 4 == 0 && (DEPTH == 1 || DEPTH == 2), "a batch is two quads (the last may be one); the ring holds one or two");
+    static_assert(ROWS % 4 == 0 && DEPTH >= 1 && DEPTH <= ROWS / 4, "a batch is two quads (the last may be one); the ring holds DEPTH quads");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[8][ROWS];
@@ -807,18 +810,19 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
 #pragma unroll
         for (int i = 0; i < 8; ++i) yn[i] = neg4(y[i]);
         float acc[8];
-#pragma unroll 1
+        // (unrolled: the ring's slots are then fixed registers whatever its depth)
+#pragma unroll
         for (int r = 0; r < ROWS; r += 8) {
             const int q = r >> 2;
             {
-                const QuadIQ2S cur = ring[0];
-                if (q + DEPTH < NQ) ring[0] = load_quad(rs, qo, quad0 + (uint32_t) (q + DEPTH) * qb);
-                quad_values<0>(cur, grid, stab, y, yn, dy8, acc);
+                const QuadIQ2S cur = ring[q % DEPTH];
+                if (q + DEPTH < NQ) ring[q % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + DEPTH) * qb);
+                quad_values<0, true>(cur, grid, stab, y, yn, dy8, acc);
             }
-            if (NQ % 2 == 0 || q + 1 < NQ) {
-                const QuadIQ2S cur = ring[1 % DEPTH];
-                if (q + 1 + DEPTH < NQ) ring[1 % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + 1 + DEPTH) * qb);
-                quad_values<4>(cur, grid, stab, y, yn, dy8, acc);
+            if (q + 1 < NQ) {
+                const QuadIQ2S cur = ring[(q + 1) % DEPTH];
+                if (q + 1 + DEPTH < NQ) ring[(q + 1) % DEPTH] = load_quad(rs, qo, quad0 + (uint32_t) (q + 1 + DEPTH) * qb);
+                quad_values<4, true>(cur, grid, stab, y, yn, dy8, acc);
             } else {
 #pragma unroll
                 for (int i = 4; i < 8; ++i) acc[i] = 0.0f;   // an odd number of quads: the last batch's second half is empty

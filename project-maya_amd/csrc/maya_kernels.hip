@@ -1574,6 +1574,8 @@ static int launch_layer_gate_up_iq2s(const maya_moe_args& a, const LayerHead& hd
 // the rows the position-mapped down kernels take on one wave: n_ff = 1024, 1536 or 2048
 static bool down_pos_nff_ok(int n_ff) { return n_ff == 1024 || n_ff == 1536 || n_ff == 2048; }
 int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
+    // One quad of rows in flight a wave: with 2, 4 or all 7 of a wave's quads requested ahead the 7168 x 2048 launch took
+    // 12.6, 14.0 and 15.9 us against 11.9.
     // Rows a workgroup: n_embd / 256 for the wide rows (20 ... 32: one workgroup a compute unit on a single token, every
     // SIMD the same number of rows, and half as many waves rounding h as with 16), else 16.
     const int n_embd = a.layout.n_embd;
