@@ -184,37 +184,20 @@ def decode_iq2s(args, np, torch, lib, L, info):
     else:
         dt = bw.timed_graph(step, K, W, stream)
 
-    # ---- the two weight-streaming kernels alone, HIP events on the launch stream (the stage calls of the C ABI on the
-    # same rotating plans; the down call given no rounded h rounds it itself, as it does inside the layer)
+    # ---- the layer's two launches apart, HIP events on the launch stream: its first half (maya_moe_layer_decode_begin:
+    # head + gate/up in one launch) and its second (maya_moe_layer_decode_end: the down launch, which rounds h itself), on
+    # the same rotating logits - the kernels the layer runs, launched as the layer launches them
     with torch.cuda.stream(stream):
-        ids_all, w_all = lib.route_topk(logits, TOP_K)
-        plans = lib.plan(ids_all.view(-1), table).view(n_sets, TOP_K)
-        xq = lib.quant_act(IQ2_S, x.to(torch.float32))
-        h = torch.empty((TOP_K, N_FF), dtype=torch.float32, device="cuda")
-        outk = torch.empty((1, N_EMBD), dtype=torch.float32, device="cuda")
-        arg_list = []
-        for j in range(n_sets):
-            b = lib.Args()
-            b.layout = layer.layout
-            b.n_tokens, b.k = 1, TOP_K
-            b.limit = float("inf")
-            b.x = xq.c()
-            b.h = h.data_ptr()
-            b.out = outk.data_ptr()
-            b.plan_ptr = plans[j].data_ptr()
-            b.plan_w = w_all[j].data_ptr()
-            arg_list.append(b)
-        assert L.maya_moe_down_rounds_h(C.byref(arg_list[0])) == 1
-        sp = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)   # noqa: E731
         reps = 64
-        gu_s = bw.event_time(lambda i: lib.check(L.maya_moe_gate_up(C.byref(arg_list[(5 + i) % n_sets]), sp())), reps, stream)
-        dn_s = bw.event_time(lambda i: lib.check(L.maya_moe_down(C.byref(arg_list[(5 + i) % n_sets]), sp())), reps, stream)
+        gu_s = bw.event_time(lambda i: layer.forward(table, logits[(5 + i) % n_sets:(5 + i) % n_sets + 1], x, half="begin"), reps, stream)
+        dn_s = bw.event_time(lambda i: layer.forward(table, logits[(5 + i) % n_sets:(5 + i) % n_sets + 1], x, half="end"), reps, stream)
 
     sec = dt / K
     w_bytes = TOP_K * blob_bytes
     bytes_step = w_bytes + N_EXPERT * 4 + N_EMBD * 2 + N_EMBD * 4
     value = bytes_step / sec / 1e9
-    gu_bytes = TOP_K * 2 * N_FF * lib.row_bytes(IQ2_S, N_EMBD) + N_EMBD + (N_EMBD // 32) * 4 + TOP_K * N_FF * 4
+    # (the launch with the head in it reads the logits, the table and x and writes h, ids, weights and the plan)
+    gu_bytes = TOP_K * 2 * N_FF * lib.row_bytes(IQ2_S, N_EMBD) + N_EXPERT * 12 + N_EMBD * 2 + TOP_K * N_FF * 4 + TOP_K * 16
     dn_bytes = TOP_K * N_EMBD * lib.row_bytes(IQ2_S, N_FF) + TOP_K * N_FF * 4 + N_EMBD * 4
     gu_rate, dn_rate = gu_bytes / gu_s / 1e9, dn_bytes / dn_s / 1e9
 
@@ -259,14 +242,14 @@ def decode_iq2s(args, np, torch, lib, L, info):
                                 "one HIP graph of the K steps, replayed back to back (>= 256 steps and >= 10 ms a sample) between "
                                 "two HIP events on the launch stream, median of %d samples after the clocks settled" % bw.ROUNDS),
                    "device": info},
-        "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_tiles_kernel", "achieved": round(gu_rate, 2), "peak": 8000.0,
+        "roofline": {"bound": "hbm", "kernel": "gate_up_iq2s_tiles_kernel (the head in the same launch)", "achieved": round(gu_rate, 2), "peak": 8000.0,
                      "unit": "GB/s", "frac": round(gu_rate * 1e9 / HBM_PEAK, 4), "traffic": GATE_UP_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_s * 1e6, 3),
                      "down_kernel": {"kernel": "down_iq2s_pos_kernel", "achieved": round(dn_rate, 2), "frac": round(dn_rate * 1e9 / HBM_PEAK, 4),
                                      "algorithmic_bytes_per_launch": dn_bytes, "avg_launch_us": round(dn_s * 1e6, 3)},
                      "layer": {"achieved": round(value, 2), "frac": round(value * 1e9 / HBM_PEAK, 4),
                                "algorithmic_bytes_per_step": bytes_step, "us_per_step": round(sec * 1e6, 3),
-                               "us_outside_the_two_kernels": round((sec - gu_s - dn_s) * 1e6, 3)}},
+                               "us_outside_the_two_launches": round((sec - gu_s - dn_s) * 1e6, 3)}},
         "cpu_baseline": cpu,
         "parity_rel_l2_vs_cpu_path": err,
         "parity_ids_exact": ids_ok,

@@ -317,6 +317,21 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
                                  float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* The same layer in its two halves, for a caller that puts work of its own between them or times them apart (the
+ * reference's engines call glmf::moe_route / moe_gate_up and moe_down one by one, glm_fast_path.cu:2688-2691):
+ *   _begin: route -> plan -> group -> quantize x -> gate/up, h left in the workspace;
+ *   _end:   quantize h -> down -> combine, from that workspace.
+ * Both take maya_moe_layer_decode_routed's arguments, the same in both calls; _begin followed by _end on one stream
+ * launches what that call launches, in the same order, and gives its bits. */
+int maya_moe_layer_decode_begin(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                                const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
+                                float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
+                                size_t workspace_bytes, void* stream);
+int maya_moe_layer_decode_end(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k,
+                              const maya_router* router, const float* logits, const void* x, int x_dtype, int n_tokens,
+                              float limit, const float* add, int32_t* ids, float* weights, float* out, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* The routed layer and the expert EVERY token takes (a shared expert), side by side:
  *   out[t] = shared->add[t] + shared_expert(x[t]) + sum_j weights[t][j] * expert_{ids[t][j]}(x[t]).
  * The reference runs the shared expert's down rows as extra blocks of the routed experts' gate/up launch

@@ -495,16 +495,21 @@ __global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq2s_pos_kernel(maya_mo
 // staged: the picks cost a workgroup some hundred instructions on one wave, against a launch and two memory round
 // trips between a head kernel and this one.
 struct LayerHead {
-    const float* logits;     // [n_expert]
-    const uint64_t* table;   // [n_expert] blob addresses, 0 = absent
     int32_t* ids;            // [k]
     float* weights;          // [k]
     uint64_t* plan;          // [k]
-    const void* x;           // [n_embd] of x_dtype
-    int n_expert, x_dtype;
 };
+// The leading arguments are what the kernel asks of memory first; as plain pointers and integers at the head of the
+// argument list they arrive in scalar registers with the dispatch (a structure passed by value is read from memory
+// first).  HEAD: p0 = the logits [n_expert], p1 = the table [n_expert] of blob addresses (0 = absent), p2 = x [n_embd] of
+// x_dtype; else p0 = the plan's blob addresses (a.plan_ptr), p1 = the codes of x (a.x.q), p2 = their scales (a.x.d).
 template <int NW, int MINW, bool HEAD>
-__global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(maya_moe_args a, Codebooks cb, LayerHead hd) {
+__global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(const void* __restrict__ p0, const void* __restrict__ p1,
+                                                                                      const void* __restrict__ p2,
+                                                                                      const uint64_t* __restrict__ iq2s_grid,
+                                                                                      const int32_t* __restrict__ skip, int n_expert,
+                                                                                      int x_dtype, int n_ent, maya_moe_args a,
+                                                                                      LayerHead hd) {
     constexpr int NU = 32 * NW;  // sub-blocks a row
     __shared__ __align__(16) int lds[kFastLdsWords];
     __shared__ float part[2][2 * NW][8];
@@ -517,16 +522,18 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
     const int u = is_up ? t - NU : t;
-    const int n_ent = a.k;   // one token: entry = plan slot
+    // (n_ent = a.k: one token, entry = plan slot)
     int y[8];
     float dy8;
     int first_tile = blockIdx.x, tile_step = gridDim.x;
     TablePieces<2048, 64 * NW> tp;   // the codebook: requested early, stored once the other first loads are on their way
-    if constexpr (!HEAD) table_request(cb.iq2s, tp);
+    if constexpr (!HEAD) table_request(iq2s_grid, tp);
     if constexpr (HEAD) {
         // The workgroup's last wave holds up rows only; it picks the experts while the gate lanes round x (a gate lane and
         // the up lane of the same position need the same codes: the gate lane rounds, the up lane takes them from LDS).
-        const int ne = hd.n_expert;
+        const int ne = n_expert;
+        const float* logits = (const float*) p0;
+        const uint64_t* table = (const uint64_t*) p1;
         const bool picker = t >= 64 * (NW - 1);
         float lv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         uint64_t tab[4] = {0ull, 0ull, 0ull, 0ull};
@@ -534,11 +541,11 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int e = 64 * r + lane;
-                lv[r] = e < ne ? hd.logits[e] : -INFINITY;
-                tab[r] = e < ne ? hd.table[e] : 0ull;
+                lv[r] = e < ne ? logits[e] : -INFINITY;
+                tab[r] = e < ne ? table[e] : 0ull;
             }
         }
-        table_request(cb.iq2s, tp);   // (behind the picker's loads: loads come back in the order they were asked for)
+        table_request(iq2s_grid, tp);   // (behind the picker's loads: loads come back in the order they were asked for)
         if (blockIdx.x == 0) {   // the router (it looks at no skip flag, like the head kernel)
             if (!picker) return;
             int id;
@@ -553,7 +560,7 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
             return;
         }
         first_tile = (int) blockIdx.x - 1, tile_step = (int) gridDim.x - 1;
-        const int skipv = a.skip ? *a.skip : 0;
+        const int skipv = skip ? *skip : 0;
         if (skipv) return;
         if (picker) {   // (before x is loaded: the values of x then take no registers here)
             __builtin_amdgcn_s_setprio(3);   // the workgroup waits for this wave: it goes first on its SIMD
@@ -572,22 +579,22 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
         }
         float v[32];
         if (!is_up) {
-            if (hd.x_dtype == MAYA_DT_F32) {
-                const float4* xv = (const float4*) hd.x + 8 * u;
+            if (x_dtype == MAYA_DT_F32) {
+                const float4* xv = (const float4*) p2 + 8 * u;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const float4 q = xv[i];
                     v[4 * i] = q.x, v[4 * i + 1] = q.y, v[4 * i + 2] = q.z, v[4 * i + 3] = q.w;
                 }
             } else {
-                const uint4* xv = (const uint4*) hd.x + 4 * u;
+                const uint4* xv = (const uint4*) p2 + 4 * u;
                 uint32_t w4[16];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const uint4 q = xv[i];
                     w4[4 * i] = q.x, w4[4 * i + 1] = q.y, w4[4 * i + 2] = q.z, w4[4 * i + 3] = q.w;
                 }
-                if (hd.x_dtype == MAYA_DT_BF16) {
+                if (x_dtype == MAYA_DT_BF16) {
 #pragma unroll
                     for (int j = 0; j < 16; ++j) {
                         v[2 * j] = __uint_as_float(w4[j] << 16);
@@ -623,13 +630,13 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
         }
     } else {
         // everything the first tile needs is requested side by side: no load waits on another
-        const int skipv = a.skip ? *a.skip : 0;
+        const int skipv = skip ? *skip : 0;
         {
-            const int4* q = (const int4*) a.x.q;
+            const int4* q = (const int4*) p1;
             const int4 ya = q[2 * u], yb = q[2 * u + 1];
             y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
         }
-        dy8 = a.x.d[u] * 0.125f;
+        dy8 = ((const float*) p2)[u] * 0.125f;
         if (skipv) return;
     }
     int yn[8];
@@ -650,7 +657,7 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
             const uint32_t hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (b >> 32));
             return ((uint64_t) hi << 32) | lo;
         } else {
-            return a.plan_ptr[e];
+            return ((const uint64_t*) p0)[e];
         }
     };
     int tile = first_tile;
@@ -718,7 +725,13 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
 // multiple of 8, the lanes past it idle): wave w = plan slot w, rows in batches of 8; grid (n_embd / ROWS).  The slots' rows
 // meet in LDS and are summed in slot order.
 template <int ROWS, int DEPTH, int MINW, int NU = 64>
-__global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args a, Codebooks cb) {
+__global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(const uint64_t* __restrict__ plan_ptr, const float* __restrict__ plan_w,
+                                                                  const float* __restrict__ h, const uint64_t* __restrict__ iq2s_grid,
+                                                                  const int32_t* __restrict__ skip, const int8_t* __restrict__ hq_q, int k,
+                                                                  int n_embd, maya_moe_args a, Codebooks cb) {
+    // (the leading arguments repeat a.plan_ptr, a.plan_w, a.h, cb.iq2s, a.skip, a.hq.q, a.k, a.layout.n_embd: plain pointers
+    // and integers at the head of the argument list arrive in scalar registers with the dispatch, a structure passed by
+    // value is read from memory first - and everything the kernel asks of memory at its start hangs on these)
     static_assert(ROWS % 4 == 0 && DEPTH >= 1 && DEPTH <= ROWS / 4, "a batch is two quads (the last may be one); the ring holds DEPTH quads");
     static_assert(NU % 8 == 0 && NU >= 8 && NU <= 64, "whole 256-value blocks on one wave");
     __shared__ __align__(16) int lds[kFastLdsWords];
@@ -727,36 +740,35 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     __shared__ int s_on[8];
     const uint2* grid = (const uint2*) lds;
     const uint2* stab = (const uint2*) (lds + 2048);
-    const int n_embd = a.layout.n_embd;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int bx, by;
     down_block_of_grid(bx, by);
     const int r0 = bx * ROWS;
-    const int e0 = by * a.k;   // the token's first entry; wave w = its slot w
+    const int e0 = by * k;   // the token's first entry; wave w = its slot w
     // Everything the workgroup needs before its weights is requested side by side, ahead of the one barrier: the skip
     // flag, the plan (the wave's slot; the slots' presence and weights for the combine), the slot's h and the tables.
     // A wave past slot k - 1 reads that slot's data and drops it: no branch, and no load waits on another.
-    const int skipv = a.skip ? *a.skip : 0;
+    const int skipv = skip ? *skip : 0;
     TablePieces<2048, 512> tp;
-    table_request(cb.iq2s, tp);
-    const int ent = e0 + min(wave, a.k - 1);
-    uint64_t blob = a.plan_ptr[ent];
-    const int ci = e0 + min((int) threadIdx.x & 7, a.k - 1);
-    const uint64_t c_ptr = a.plan_ptr[ci];
-    const float c_w = a.plan_w[ci];
+    table_request(iq2s_grid, tp);
+    const int ent = e0 + min(wave, k - 1);
+    uint64_t blob = plan_ptr[ent];
+    const int ci = e0 + min((int) threadIdx.x & 7, k - 1);
+    const uint64_t c_ptr = plan_ptr[ci];
+    const float c_w = plan_w[ci];
     const bool on = NU == 64 || lane < NU;   // (an idle lane reads the last position's data and uses zeros)
     const int pos = on ? lane : NU - 1;
-    const bool rounded = a.hq.q != nullptr;
+    const bool rounded = hq_q != nullptr;
     int y[8];
     float dy8 = 0.0f;
     float v[32];
     if (rounded) {
-        const int4* q = (const int4*) (a.hq.q + (size_t) ent * (32 * NU));
+        const int4* q = (const int4*) (hq_q + (size_t) ent * (32 * NU));
         const int4 ya = q[2 * pos], yb = q[2 * pos + 1];
         y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
         dy8 = a.hq.d[(size_t) ent * NU + pos] * 0.125f;
     } else {
-        const float4* hv = (const float4*) (a.h + (size_t) ent * (32 * NU) + 32 * pos);
+        const float4* hv = (const float4*) (h + (size_t) ent * (32 * NU) + 32 * pos);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float4 t = hv[i];
@@ -764,7 +776,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
         }
     }
     if (skipv) return;
-    if (wave >= a.k) blob = 0ull;
+    if (wave >= k) blob = 0ull;
     constexpr uint32_t qb = NU / 8 * 82 * 4;
     // the wave's blob address is wave-uniform; readfirstlane (a signed int: widened through uint32_t) moves it to
     // scalar registers for the buffer resource (no blob: an empty resource, whose loads read as zero and touch nothing)
@@ -783,7 +795,7 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(maya_moe_args 
     store_iq2s_selectors<512>(lds);
     table_store(lds, tp);
     if (threadIdx.x < 8) {
-        s_on[threadIdx.x] = (int) threadIdx.x < a.k && c_ptr != 0ull;
+        s_on[threadIdx.x] = (int) threadIdx.x < k && c_ptr != 0ull;
         s_w[threadIdx.x] = c_w;
     }
     __syncthreads();

@@ -1530,8 +1530,16 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
 // one token: the tile-streaming form, launched with the workgroups the chip holds at once (asked of the runtime once a
 // shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
 // tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
+// the head's inputs when it rides in the gate/up launch, and where its results go
+struct LayerHeadIn {
+    const float* logits;
+    const uint64_t* table;
+    const void* x;
+    int n_expert, x_dtype;
+    LayerHead out;
+};
 template <int NW>
-int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hipStream_t s, const LayerHead* hd = nullptr) {
+int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hipStream_t s, const LayerHeadIn* hd = nullptr) {
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0, m = 0;
@@ -1544,9 +1552,11 @@ int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hip
     const int wgs = per_cu * st.n_cu;
     const unsigned walkers = (unsigned) (wgs < n_tiles ? wgs : n_tiles);
     if (hd) {   // workgroup 0 routes, the others walk the tiles
-        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, a, st.cb, *hd);
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, (const void*) hd->logits,
+                           (const void*) hd->table, hd->x, st.cb.iq2s, a.skip, hd->n_expert, hd->x_dtype, a.k, a, hd->out);
     } else {
-        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, false>), dim3(walkers), dim3(64 * NW), 0, s, a, st.cb, LayerHead{});
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, false>), dim3(walkers), dim3(64 * NW), 0, s, (const void*) a.plan_ptr,
+                           (const void*) a.x.q, (const void*) a.x.d, st.cb.iq2s, a.skip, 0, 0, a.k, a, LayerHead{});
     }
     MAYA_LAUNCHED("gate_up_iq2s_tiles_kernel");
     return MAYA_OK;
@@ -1560,7 +1570,7 @@ static bool layer_head_in_gate_up_ok(const maya_moe_args& a, const RouterSpec& r
            x_dtype <= 2 && ((uintptr_t) x & 15) == 0 && l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM &&
            l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 && l.n_embd >= 2048 && l.n_embd <= 8192;
 }
-static int launch_layer_gate_up_iq2s(const maya_moe_args& a, const LayerHead& hd, const DeviceState& st, hipStream_t s) {
+static int launch_layer_gate_up_iq2s(const maya_moe_args& a, const LayerHeadIn& hd, const DeviceState& st, hipStream_t s) {
     switch (a.layout.n_embd / 1024) {
         case 2: return launch_gate_up_iq2s_tiles<2>(a, st, s, &hd);
         case 3: return launch_gate_up_iq2s_tiles<3>(a, st, s, &hd);
@@ -1580,12 +1590,13 @@ int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStrea
     // SIMD the same number of rows, and half as many waves rounding h as with 16), else 16.
     const int n_embd = a.layout.n_embd;
     const int wide = n_embd % 1024 == 0 && n_embd >= 5120 && n_embd <= 8192 ? n_embd / 256 : 16;
+#define MAYA_DN_HEAD a.plan_ptr, a.plan_w, a.h, st.cb.iq2s, a.skip, a.hq.q, a.k, a.layout.n_embd
 #define MAYA_ROWS(R, MINW)                                                                                             \
     {                                                                                                                  \
         const dim3 grid((unsigned) (n_embd / R), (unsigned) a.n_tokens);                                               \
-        if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 32>), grid, dim3(512), 0, s, a, st.cb);      \
-        else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 48>), grid, dim3(512), 0, s, a, st.cb); \
-        else hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW>), grid, dim3(512), 0, s, a, st.cb);                  \
+        if (a.layout.n_ff == 1024) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 32>), grid, dim3(512), 0, s, MAYA_DN_HEAD, a, st.cb);      \
+        else if (a.layout.n_ff == 1536) hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW, 48>), grid, dim3(512), 0, s, MAYA_DN_HEAD, a, st.cb); \
+        else hipLaunchKernelGGL((down_iq2s_pos_kernel<R, 1, MINW>), grid, dim3(512), 0, s, MAYA_DN_HEAD, a, st.cb);                  \
     }
     switch (wide) {
         case 20: MAYA_ROWS(20, 4) break;
@@ -1594,6 +1605,7 @@ int launch_down_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipStrea
         case 32: MAYA_ROWS(32, 4) break;
         default: MAYA_ROWS(16, 7) break;
     }
+#undef MAYA_DN_HEAD
 #undef MAYA_ROWS
     MAYA_LAUNCHED("down_iq2s_pos_kernel");
     return MAYA_OK;
@@ -2529,23 +2541,27 @@ static int layer_setup(const maya_moe_layout* l, const uint64_t* expert_table, i
     return down_refusal(&probe, st);
 }
 
+enum { kLayerWhole = 0, kLayerBegin = 1, kLayerEnd = 2 };
 static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
                              const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
                              int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream,
-                             hipEvent_t join, bool* joined) {
+                             hipEvent_t join, bool* joined, int phase = kLayerWhole) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;
     RouterSpec rs;
     LayerWs w;
     maya_moe_args a;
+    const bool head = phase != kLayerEnd, tail = phase != kLayerBegin;
     if (const int rc0 = layer_setup(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out,
                                     workspace, workspace_bytes, *st, rs, w, a))
         return rc0;
     int rc;
-    bool grouped = false, gate_up_done = false;
-    if (layer_head_in_gate_up_ok(a, rs, logits, n_expert, x, x_dtype)) {
+    bool grouped = !head, gate_up_done = !head;
+    if (!head) {
+        // (the second half of a call made in two: the plan, the groups and h are in the workspace)
+    } else if (layer_head_in_gate_up_ok(a, rs, logits, n_expert, x, x_dtype)) {
         // one token of IQ2_S experts: route, plan, Q8_K of x and gate/up in one launch
-        const LayerHead hd{logits, expert_table, ids, weights, w.plan_ptr, x, n_expert, x_dtype};
+        const LayerHeadIn hd{logits, expert_table, x, n_expert, x_dtype, LayerHead{ids, weights, w.plan_ptr}};
         if ((rc = launch_layer_gate_up_iq2s(a, hd, *st, as_stream(stream)))) return rc;
         gate_up_done = true;
     } else if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
@@ -2594,6 +2610,7 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
         }
     }
     if (!gate_up_done && (rc = maya_moe_gate_up(&a, stream))) return rc;
+    if (!tail) return MAYA_OK;
     if (down_rounds_h(a)) {
         a.hq = maya_act{nullptr, nullptr, nullptr};
         a.part = nullptr;
@@ -2614,6 +2631,19 @@ int maya_moe_layer_decode_routed(const maya_moe_layout* l, const uint64_t* exper
                                  int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
     return layer_decode_core(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out, workspace,
                              workspace_bytes, stream, nullptr, nullptr);
+}
+
+int maya_moe_layer_decode_begin(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                                const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                                int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    return layer_decode_core(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out, workspace,
+                             workspace_bytes, stream, nullptr, nullptr, kLayerBegin);
+}
+int maya_moe_layer_decode_end(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,
+                              const float* logits, const void* x, int x_dtype, int n_tokens, float limit, const float* add,
+                              int32_t* ids, float* weights, float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    return layer_decode_core(l, expert_table, n_expert, k, router, logits, x, x_dtype, n_tokens, limit, add, ids, weights, out, workspace,
+                             workspace_bytes, stream, nullptr, nullptr, kLayerEnd);
 }
 
 int maya_moe_layer_decode_shared(const maya_moe_layout* l, const uint64_t* expert_table, int n_expert, int k, const maya_router* router,

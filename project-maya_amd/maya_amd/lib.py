@@ -21,7 +21,8 @@ EXPORTS = [
     "maya_moe_route_sigmoid", "maya_moe_layer_decode_routed", "maya_moe_route_plan", "maya_moe_route_tiered", "maya_moe_fetch",
     "maya_moe_tab_update",
     "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv", "maya_moe_layer_decode_static",
-    "maya_moe_layer_decode_shared", "maya_moe_route_window_ok", "maya_moe_route_window",
+    "maya_moe_layer_decode_shared", "maya_moe_route_window_ok", "maya_moe_route_window", "maya_moe_layer_decode_begin",
+    "maya_moe_layer_decode_end",
 ]
 
 
@@ -113,6 +114,8 @@ def load():
     L.maya_moe_layer_decode.argtypes = [C.POINTER(Layout), vp, i32, i32, vp, vp, i32, i32, f32, vp, vp, vp, vp, vp, sz, vp]
     L.maya_moe_layer_decode_routed.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32, vp, vp, vp,
                                                vp, vp, sz, vp]
+    L.maya_moe_layer_decode_begin.argtypes = L.maya_moe_layer_decode_routed.argtypes
+    L.maya_moe_layer_decode_end.argtypes = L.maya_moe_layer_decode_routed.argtypes
     L.maya_moe_layer_decode_shared.argtypes = [C.POINTER(Layout), vp, i32, i32, C.POINTER(Router), vp, vp, i32, i32, f32,
                                                C.POINTER(Args), vp, vp, vp, vp, sz, vp]
     L.maya_moe_route_sigmoid.argtypes = [vp, vp, i32, i32, i32, f32, i32, vp, vp, vp]
@@ -364,10 +367,11 @@ class MoeLayer:
         self.out = torch.empty((max_tokens, n_embd), dtype=torch.float32, device=device)
 
     def forward(self, expert_table, logits, x, limit=float("inf"), add=None, stream=None, router=None, routed=None, shared=None,
-                shared_limit=float("inf")):
+                shared_limit=float("inf"), half=None):
         """router: None (the softmax router) or a Router (kind, norm, bias pointer, w_scale); routed = (ids, weights)
         [nt, k] tensors: the tokens are already routed (logits is then ignored); shared: a DenseExpert over the same
-        tokens that runs beside the routed experts (maya_moe_layer_decode_shared) - out = add + shared(x) + routed(x)."""
+        tokens that runs beside the routed experts (maya_moe_layer_decode_shared) - out = add + shared(x) + routed(x);
+        half: "begin" / "end" = the layer's two halves (maya_moe_layer_decode_begin / _end), same arguments in both."""
         nt = x.shape[0]
         assert nt <= self.max_tokens and x.is_contiguous()
         if routed is not None:
@@ -385,6 +389,12 @@ class MoeLayer:
                                                       nt, limit, C.byref(a), _p(self.ids), _p(self.weights), _p(self.out), _p(self.ws),
                                                       self.ws_bytes, _stream(stream)))
             a.add = None
+            return self.out[:nt]
+        if half is not None:
+            fn = load().maya_moe_layer_decode_begin if half == "begin" else load().maya_moe_layer_decode_end
+            check(fn(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, C.byref(router) if router is not None else None,
+                     _p(logits), _p(x), dtype_id(x), nt, limit, _p(add), _p(self.ids), _p(self.weights), _p(self.out), _p(self.ws),
+                     self.ws_bytes, _stream(stream)))
             return self.out[:nt]
         if router is not None:
             check(load().maya_moe_layer_decode_routed(C.byref(self.layout), _p(expert_table), self.n_expert, self.k, C.byref(router),

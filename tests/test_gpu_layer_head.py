@@ -177,3 +177,27 @@ def test_order_only_pick_against_the_exact_router_on_adversarial_rows(lib):
             print("row", i, fused.ids[0].tolist(), want_ids[i].tolist(), flush=True)
     torch.cuda.synchronize()
     assert bad == 0, bad
+
+
+@pytest.mark.parametrize("gt,dt,n_embd,n_ff,ne,k,nt", ((22, 22, 2048, 512, 12, 4, 1), (22, 22, 2048, 1024, 12, 4, 3),
+                                                      (12, 12, 2048, 2048, 6, 3, 1), (22, 12, 1024, 512, 8, 8, 6)))
+def test_the_layer_in_two_calls_is_the_layer(lib, gt, dt, n_embd, n_ff, ne, k, nt):
+    """maya_moe_layer_decode_begin + maya_moe_layer_decode_end on the same arguments = maya_moe_layer_decode, bit for bit."""
+    blobs = make_experts(gt, dt, n_embd, n_ff, ne, 31 + nt)
+    gguf_layout, _ = lib.layout(gt, dt, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+    rng = np.random.default_rng(nt)
+    logits = dev(rng.standard_normal((nt, ne)).astype(np.float32))
+    x = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    add = dev(rng.standard_normal((nt, n_embd)).astype(np.float32))
+    whole = lib.MoeLayer(gt, dt, n_embd, n_ff, ne, k, max_tokens=nt, packing=1)
+    halves = lib.MoeLayer(gt, dt, n_embd, n_ff, ne, k, max_tokens=nt, packing=1)
+    want = whole.forward(store.table, logits, x, add=add).clone()
+    halves.out.zero_()
+    halves.forward(store.table, logits, x, add=add, half="begin")
+    torch.cuda.synchronize()
+    assert float(halves.out.abs().max()) == 0.0          # nothing of the second half has run
+    got = halves.forward(store.table, logits, x, add=add, half="end")
+    torch.cuda.synchronize()
+    assert torch.equal(whole.ids, halves.ids) and torch.equal(whole.weights.view(torch.int32), halves.weights.view(torch.int32))
+    assert torch.equal(want.view(torch.int32), got.view(torch.int32))
