@@ -749,10 +749,10 @@ __global__ __launch_bounds__(512, MINW) void down_iq2s_pos_kernel(const uint64_t
     // flag, the plan (the wave's slot; the slots' presence and weights for the combine), the slot's h and the tables.
     // A wave past slot k - 1 reads that slot's data and drops it: no branch, and no load waits on another.
     const int skipv = skip ? *skip : 0;
+    const int ent = e0 + min(wave, k - 1);
+    uint64_t blob = plan_ptr[ent];   // (asked for first: loads come back in order, and the weights' request waits for this one)
     TablePieces<2048, 512> tp;
     table_request(iq2s_grid, tp);
-    const int ent = e0 + min(wave, k - 1);
-    uint64_t blob = plan_ptr[ent];
     const int ci = e0 + min((int) threadIdx.x & 7, k - 1);
     const uint64_t c_ptr = plan_ptr[ci];
     const float c_w = plan_w[ci];
