@@ -1527,6 +1527,9 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
 }
+// (The kernel is compiled for 6 waves a SIMD - three workgroups of up to 8 waves a compute unit, what is launched - not 8:
+// with the head's prologue in it the kernel needs 73 registers, and at 64 it spilled 36 bytes a lane to scratch memory:
+// 6.8 MB written and read back a launch, 2.1 us of the layer.)
 // one token: the tile-streaming form, launched with the workgroups the chip holds at once (asked of the runtime once a
 // shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
 // tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
@@ -1543,8 +1546,8 @@ int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hip
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0, m = 0;
-        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gate_up_iq2s_tiles_kernel<NW, 8, false>, 64 * NW, 0));
-        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, gate_up_iq2s_tiles_kernel<NW, 8, true>, 64 * NW, 0));
+        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gate_up_iq2s_tiles_kernel<NW, 6, false>, 64 * NW, 0));
+        MAYA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&m, gate_up_iq2s_tiles_kernel<NW, 6, true>, 64 * NW, 0));
         n = m < n ? m : n;
         per_cu = n > 3 ? 3 : n > 0 ? n : 1;
     }
@@ -1552,10 +1555,10 @@ int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hip
     const int wgs = per_cu * st.n_cu;
     const unsigned walkers = (unsigned) (wgs < n_tiles ? wgs : n_tiles);
     if (hd) {   // workgroup 0 routes, the others walk the tiles
-        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, (const void*) hd->logits,
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 6, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, (const void*) hd->logits,
                            (const void*) hd->table, hd->x, st.cb.iq2s, a.skip, hd->n_expert, hd->x_dtype, a.k, a, hd->out);
     } else {
-        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 8, false>), dim3(walkers), dim3(64 * NW), 0, s, (const void*) a.plan_ptr,
+        hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 6, false>), dim3(walkers), dim3(64 * NW), 0, s, (const void*) a.plan_ptr,
                            (const void*) a.x.q, (const void*) a.x.d, st.cb.iq2s, a.skip, 0, 0, a.k, a, LayerHead{});
     }
     MAYA_LAUNCHED("gate_up_iq2s_tiles_kernel");
