@@ -229,6 +229,13 @@ int maya_moe_route_tiered(const struct maya_router* router, const float* logits,
                           void* stream);
 /* Copies every planned entry with a fetch source into its slot: moe_fetch (glm_fast.hpp:468-469, glm_fast.cu:4688-4704). */
 int maya_moe_fetch(const uint64_t* fetch_src, const uint64_t* plan_ptr, int n_entries, size_t blob_bytes, void* stream);
+/* The copy of a prefetch list: moe_prefetch (glm_fast.hpp:473-474, glm_fast.cu:4619-4627, 7105-7123) - *pf_n entries (a
+ * DEVICE count, read by the kernel; clamped to max_entries) of blob_bytes each from pf_src[i] (HBM or mapped host memory)
+ * to pf_dst[i]; a null source or slot is skipped.  n_workgroups: how many workgroups copy (the call is meant for a side
+ * stream beside the layer's kernels, and every compute unit it holds is one they wait for); 0 = half the compute units,
+ * the reference's default.  Which experts to prefetch, and their slots, stay the engine's decision. */
+int maya_moe_prefetch(const uint64_t* pf_src, const uint64_t* pf_dst, const int32_t* pf_n, int max_entries, size_t blob_bytes,
+                      int n_workgroups, void* stream);
 /* tab[keys[i]] = vals[i], the engine's edits between tokens: tab_update (glm_fast.cu:7745-7754); n_words = the array's
  * length (a key outside it is ignored). */
 int maya_moe_tab_update(uint64_t* tab, int n_words, const int32_t* keys, const uint64_t* vals, int n, void* stream);

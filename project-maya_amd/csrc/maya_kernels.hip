@@ -2239,6 +2239,20 @@ int maya_moe_fetch(const uint64_t* fetch_src, const uint64_t* plan_ptr, int n_en
     return MAYA_OK;
 }
 
+int maya_moe_prefetch(const uint64_t* pf_src, const uint64_t* pf_dst, const int32_t* pf_n, int max_entries, size_t blob_bytes,
+                      int n_workgroups, void* stream) {
+    DeviceState* st;
+    if (const int rc = current_state(&st)) return rc;
+    if (!pf_src || !pf_dst || !pf_n) return fail(MAYA_E_ARG, "prefetch: null pointer");
+    if (max_entries <= 0 || max_entries > 65535 || blob_bytes == 0 || n_workgroups < 0 || n_workgroups > 65535)
+        return fail(MAYA_E_SHAPE, "prefetch: up to %d entries of %zu bytes by %d workgroups", max_entries, blob_bytes, n_workgroups);
+    // (0: half the compute units, the reference's default)
+    const unsigned wgs = n_workgroups > 0 ? (unsigned) n_workgroups : (unsigned) std::max(1, st->n_cu / 2);
+    hipLaunchKernelGGL(prefetch_kernel, dim3(wgs), dim3(256), 0, as_stream(stream), pf_src, pf_dst, pf_n, max_entries, blob_bytes);
+    MAYA_LAUNCHED("prefetch_kernel");
+    return MAYA_OK;
+}
+
 int maya_moe_tab_update(uint64_t* tab, int n_words, const int32_t* keys, const uint64_t* vals, int n, void* stream) {
     DeviceState* st;
     if (const int rc = current_state(&st)) return rc;

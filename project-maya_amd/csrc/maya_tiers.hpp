@@ -2,7 +2,7 @@
 // (include/strata/kernels/glm_fast.hpp:284-296) and the plan part of moe_route_kernel that reads them
 // (src/kernels/cuda/glm_fast.cu:4262-4375), the fetch of moe_fetch_kernel (glm_fast.cu:4688-4704) and tab_update
 // (glm_fast.cu:7745-7754).  The request ring to the host, the CPU lane, the prefetch of the next layer and the disk tier
-// stay the engine's: an expert in neither table is reported in the miss mask and left out of the plan.
+// stay the engine's (the prefetch LIST's copy is here: prefetch_kernel): an expert in neither table is reported in the miss mask and left out of the plan.
 #pragma once
 
 namespace maya {
@@ -189,6 +189,28 @@ __global__ __launch_bounds__(256) void fetch_kernel(const uint64_t* __restrict__
         for (size_t i = (n16 << 4) + i0; i < n; i += step) dst[i] = src[i];
     } else {
         for (size_t i = i0; i < n; i += step) dst[i] = src[i];
+    }
+}
+
+// The prefetch list's copy (moe_prefetch_kernel, glm_fast.cu:4619-4627): *n_list entries - the count is the device's, read
+// here - of n bytes each from src[i] to dst[i], by however many workgroups the caller grants (it runs beside the main
+// stream's kernels: every compute unit it holds is one they wait for).  Entry after entry, the workgroups striding
+// through each; a null source or slot is skipped.
+__global__ __launch_bounds__(256) void prefetch_kernel(const uint64_t* __restrict__ src_list, const uint64_t* __restrict__ dst_list,
+                                                       const int32_t* __restrict__ n_list, int max_entries, size_t n) {
+    const int cnt = min(max(*n_list, 0), max_entries);
+    const size_t i0 = (size_t) blockIdx.x * 256 + threadIdx.x, step = (size_t) gridDim.x * 256;
+    for (int e = 0; e < cnt; ++e) {
+        const uint8_t* src = (const uint8_t*) src_list[e];
+        uint8_t* dst = (uint8_t*) dst_list[e];
+        if (src == nullptr || dst == nullptr) continue;
+        if ((((uintptr_t) src | (uintptr_t) dst) & 15) == 0) {
+            const size_t n16 = n >> 4;
+            for (size_t i = i0; i < n16; i += step) ((uint4*) dst)[i] = ((const uint4*) src)[i];
+            for (size_t i = (n16 << 4) + i0; i < n; i += step) dst[i] = src[i];
+        } else {
+            for (size_t i = i0; i < n; i += step) dst[i] = src[i];
+        }
     }
 }
 

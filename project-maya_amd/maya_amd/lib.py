@@ -22,7 +22,7 @@ EXPORTS = [
     "maya_moe_tab_update",
     "maya_dequant_rows_packed", "maya_moe_down_rounds_h", "maya_mv_supported", "maya_mv", "maya_moe_layer_decode_static",
     "maya_moe_layer_decode_shared", "maya_moe_route_window_ok", "maya_moe_route_window", "maya_moe_layer_decode_begin",
-    "maya_moe_layer_decode_end",
+    "maya_moe_layer_decode_end", "maya_moe_prefetch",
 ]
 
 
@@ -103,6 +103,7 @@ def load():
     L.maya_moe_route_tiered.argtypes = [vp, vp, i32, i32, i32, i32, C.POINTER(Residency), i32, vp, vp, vp, vp]
     L.maya_moe_fetch.argtypes = [vp, vp, i32, sz, vp]
     L.maya_moe_tab_update.argtypes = [vp, i32, vp, vp, i32, vp]
+    L.maya_moe_prefetch.argtypes = [vp, vp, vp, i32, sz, i32, vp]
     L.maya_moe_group.argtypes = [vp, i32, vp, vp, vp, vp, vp]
     L.maya_moe_gate_up.argtypes = [C.POINTER(Args), vp]
     L.maya_moe_down.argtypes = [C.POINTER(Args), vp]
@@ -296,6 +297,13 @@ class Tiers:
 
     def update(self, keys, vals, stream=None):
         check(load().maya_moe_tab_update(_p(self.tab), self.tab.numel(), _p(keys), _p(vals), keys.numel(), _stream(stream)))
+
+
+def prefetch(pf_src, pf_dst, pf_n, blob_bytes, n_workgroups=0, stream=None):
+    """Copies the first *pf_n (a device int32) entries of the list: blob_bytes from pf_src[i] to pf_dst[i] (maya_moe_prefetch)."""
+    assert pf_src.dtype == torch.int64 and pf_dst.dtype == torch.int64 and pf_n.dtype == torch.int32
+    check(load().maya_moe_prefetch(_p(pf_src), _p(pf_dst), _p(pf_n), min(pf_src.numel(), pf_dst.numel()), blob_bytes, n_workgroups,
+                                   _stream(stream)))
 
 
 def plan(ids, expert_table, stream=None):

@@ -174,3 +174,45 @@ def test_a_layer_whose_experts_arrive_through_the_tiers(lib, gt, dt, n_embd, n_f
     out = layer.forward(table, None, x, router=router, routed=(ids, w))
     torch.cuda.synchronize()
     assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("nbytes,src_off,dst_off,pinned,count,wgs", ((4096, 0, 0, False, 3, 0), (100000, 0, 0, True, 6, 4), (65537, 2, 2, False, 9, 1),
+                                                                    (12345, 2, 6, True, 2, 7), (3 << 20, 0, 0, True, 4, 0), (4096, 0, 0, False, 0, 0)))
+def test_prefetch_copies_the_counted_entries_of_the_list(lib, nbytes, src_off, dst_off, pinned, count, wgs):
+    """maya_moe_prefetch: the first *pf_n entries of the list (a device count; past the list's length it is clamped), a null
+    source or slot skipped, nothing else written - from HBM and from mapped host memory, aligned and not, by 1 ... n workgroups."""
+    n = 6
+    stride = (nbytes + 511) & ~255
+    g = torch.Generator().manual_seed(nbytes + count)
+    host = torch.randint(0, 256, (n * stride + 256,), dtype=torch.uint8, generator=g)
+    if pinned:
+        ram = torch.empty(n * stride + 256, dtype=torch.uint8, pin_memory=True)
+        ram.copy_(host)
+    else:
+        ram = host.cuda()
+    slots = torch.full((n * stride + 256,), 0xEE, dtype=torch.uint8, device="cuda")
+    src = torch.zeros(n, dtype=torch.int64)
+    dst = torch.zeros(n, dtype=torch.int64)
+    sbase, dbase = ram.data_ptr() + (-ram.data_ptr()) % 256, slots.data_ptr() + (-slots.data_ptr()) % 256
+    for e in range(n):
+        src[e] = sbase + e * stride + src_off
+        dst[e] = dbase + (n - 1 - e) * stride + dst_off      # entry e -> slot n-1-e
+    src[1] = 0                                              # an entry without a source
+    dst[4] = 0                                              # ... and one without a slot
+    pf_n = torch.tensor([count], dtype=torch.int32, device="cuda")
+    lib.prefetch(src.cuda(), dst.cuda(), pf_n, nbytes, n_workgroups=wgs)
+    torch.cuda.synchronize()
+    got = slots.cpu().numpy()
+    want = np.full_like(got, 0xEE)
+    h = host.numpy()
+    so, do = sbase - ram.data_ptr(), dbase - slots.data_ptr()
+    for e in range(min(count, n)):
+        if e in (1, 4):
+            continue
+        a = do + (n - 1 - e) * stride + dst_off
+        b = so + e * stride + src_off
+        want[a:a + nbytes] = h[b:b + nbytes]
+    assert np.array_equal(got, want)
+    L = lib.load()
+    assert L.maya_moe_prefetch(None, dst.cuda().data_ptr(), pf_n.data_ptr(), n, nbytes, 0, None) == 3
+    assert L.maya_moe_prefetch(src.cuda().data_ptr(), dst.cuda().data_ptr(), pf_n.data_ptr(), 0, nbytes, 0, None) == 2
