@@ -498,17 +498,21 @@ struct LayerHead {
     int32_t* ids;            // [k]
     float* weights;          // [k]
     uint64_t* plan;          // [k]
+    float w_scale;           // the sigmoid router's weight scale and normalisation
+    int norm;
 };
 // The leading arguments are what the kernel asks of memory first; as plain pointers and integers at the head of the
 // argument list they arrive in scalar registers with the dispatch (a structure passed by value is read from memory
 // first).  HEAD: p0 = the logits [n_expert], p1 = the table [n_expert] of blob addresses (0 = absent), p2 = x [n_embd] of
-// x_dtype; else p0 = the plan's blob addresses (a.plan_ptr), p1 = the codes of x (a.x.q), p2 = their scales (a.x.d).
+// dtype `mode & 255`, bias = the sigmoid router's (`mode >> 8` = 1: the sigmoid router) or NULL; else p0 = the plan's blob
+// addresses (a.plan_ptr), p1 = the codes of x (a.x.q), p2 = their scales (a.x.d).
 template <int NW, int MINW, bool HEAD>
 __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_kernel(const void* __restrict__ p0, const void* __restrict__ p1,
                                                                                       const void* __restrict__ p2,
                                                                                       const uint64_t* __restrict__ iq2s_grid,
+                                                                                      const float* __restrict__ bias,
                                                                                       const int32_t* __restrict__ skip, int n_expert,
-                                                                                      int x_dtype, int n_ent, maya_moe_args a,
+                                                                                      int mode, int n_ent, maya_moe_args a,
                                                                                       LayerHead hd) {
     constexpr int NU = 32 * NW;  // sub-blocks a row
     __shared__ __align__(16) int lds[kFastLdsWords];
@@ -535,7 +539,9 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
         const float* logits = (const float*) p0;
         const uint64_t* table = (const uint64_t*) p1;
         const bool picker = t >= 64 * (NW - 1);
-        float lv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int x_dtype = mode & 255;
+        const bool sigm = (mode >> 8) != 0;
+        float lv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
         uint64_t tab[4] = {0ull, 0ull, 0ull, 0ull};
         if (picker) {
 #pragma unroll
@@ -543,6 +549,7 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
                 const int e = 64 * r + lane;
                 lv[r] = e < ne ? logits[e] : -INFINITY;
                 tab[r] = e < ne ? table[e] : 0ull;
+                if (bias) bv[r] = e < ne ? bias[e] : 0.0f;
             }
         }
         table_request(iq2s_grid, tp);   // (behind the picker's loads: loads come back in the order they were asked for)
@@ -551,7 +558,13 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
             int id;
             float w;
             uint64_t ptr;
-            route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+            if (sigm) {
+                float p[4], sc[4];
+                const bool fin = sigmoid_scores(lv, bv, bias != nullptr, ne, p, sc);
+                route_wave_sigmoid(p, sc, fin, tab, ne, n_ent, hd.norm, hd.w_scale, id, w, ptr);
+            } else {
+                route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+            }
             if (lane < n_ent) {
                 hd.ids[lane] = id;
                 hd.weights[lane] = w;
@@ -568,7 +581,17 @@ __global__ __launch_bounds__(NW > 4 ? 512 : 256, MINW) void gate_up_iq2s_tiles_k
             for (int r = 0; r < 4; ++r) s_tab[64 * r + lane] = tab[r];
             int id;
             uint64_t ptr;
-            if (route_wave_order_only(lv, ne, n_ent, s_lv, id)) {
+            if (sigm) {
+                // the scores are the exact router's own keys: any strictly descending order of the picks is its order
+                float p[4], sc[4];
+                const bool fin = sigmoid_scores(lv, bv, bias != nullptr, ne, p, sc);
+                if (route_wave_order_only(sc, fin, ne, n_ent, s_lv, 0.0f, INFINITY, id)) {
+                    ptr = s_tab[lane < n_ent ? id : 0];
+                } else {
+                    float w;
+                    route_wave_sigmoid(p, sc, fin, tab, ne, n_ent, hd.norm, hd.w_scale, id, w, ptr);
+                }
+            } else if (route_wave_order_only(lv, true, ne, n_ent, s_lv, 1e-6f, 60.0f, id)) {
                 ptr = s_tab[lane < n_ent ? id : 0];
             } else {
                 float w;

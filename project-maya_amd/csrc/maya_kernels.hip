@@ -846,11 +846,13 @@ __device__ __forceinline__ void route_wave_softmax(const float (&lv)[4], const u
 // shows as a negative gap), and holds the k-th pick against the upper end of the (k + 1)-th pick's bucket, above which
 // nothing unpicked can lie.  One wave, k < n_expert <= 256, k + 1 <= 64; s_lv [256] floats of LDS scratch; lane i < k
 // gets slot i's expert.
-__device__ __forceinline__ bool route_wave_order_only(const float (&lv)[4], int n_expert, int k, float* s_lv, int& my_id) {
+// (The sigmoid router picks by the score p + bias itself, so its keys ARE the exact router's: margin 0 - any strictly
+// descending order is the router's - and no range to keep; `fin` then says that no logit and no score is non-finite.)
+__device__ __forceinline__ bool route_wave_order_only(const float (&lv)[4], bool fin, int n_expert, int k, float* s_lv, float margin,
+                                                      float range, int& my_id) {
     const int lane = threadIdx.x & 63;
     constexpr int kNone = (int) 0x80000000;
     int k0, k1, k2, k3;
-    bool fin = true;
     {
         int key[4];
 #pragma unroll
@@ -878,9 +880,68 @@ __device__ __forceinline__ bool route_wave_order_only(const float (&lv)[4], int 
     const float ub = __int_as_float(ub_key >= 0 ? ub_key : ub_key ^ 0x7fffffff);   // the bucket's upper end
     const float nxt = __shfl_down(lane == k ? ub : val, 1, kWave);
     const float first = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(val), 0));
-    const bool apart = lane >= k || (val - nxt > 1e-6f && first - nxt <= 60.0f);
+    const bool apart = lane >= k || (val - nxt > margin && first - nxt <= range);
     my_id = id;
     return __all(fin && apart) != 0;
+}
+
+// The sigmoid router on ONE wave, nothing but registers (route_token_sigmoid's arithmetic; up to 256 experts, 4 a lane:
+// lv / bv / tab of experts L, L + 64, ...; bv all zero without a bias).  sc: the lane's four scores p + bias as the
+// caller already made them with sigmoid_scores (the same instructions, so the same bits).  Lane i < k returns slot i; a
+// row with a non-finite logit or score returns id -1, weight 0, no blob.
+__device__ __forceinline__ bool sigmoid_scores(const float (&lv)[4], const float (&bv)[4], bool has_bias, int n_expert, float (&p)[4],
+                                               float (&sc)[4]) {
+    const int lane = threadIdx.x & 63;
+    bool fin = true;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const bool have = 64 * r + lane < n_expert;
+        const float le = have ? lv[r] : 0.0f;
+        p[r] = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf(-le)));
+        sc[r] = has_bias ? __fadd_rn(p[r], bv[r]) : p[r];
+        fin = fin && (!have || (isfinite(le) && isfinite(sc[r])));
+    }
+    return fin;
+}
+__device__ __forceinline__ void route_wave_sigmoid(const float (&p)[4], const float (&sc)[4], bool fin, const uint64_t (&tab)[4], int n_expert,
+                                                   int k, int norm, float w_scale, int& my_id, float& my_w, uint64_t& my_ptr) {
+    const int lane = threadIdx.x & 63;
+    constexpr int kNone = (int) 0x80000000;
+    const bool bad = __any(!fin) != 0;
+    // (named copies: a select among array elements invites the compiler to index the array in memory)
+    const uint64_t t0 = tab[0], t1 = tab[1], t2 = tab[2], t3 = tab[3];
+    const float p0 = p[0], p1 = p[1], p2 = p[2], p3 = p[3];
+    int k0 = lane < n_expert ? float_order_key(sc[0]) : kNone, k1 = 64 + lane < n_expert ? float_order_key(sc[1]) : kNone;
+    int k2 = 128 + lane < n_expert ? float_order_key(sc[2]) : kNone, k3 = 192 + lane < n_expert ? float_order_key(sc[3]) : kNone;
+    int id = 0;
+    float pw = 0.0f;
+    uint64_t ptr = 0ull;
+    for (int i = 0; i < k; ++i) {
+        const int top = wave_max_i32(max(max(k0, k1), max(k2, k3)));
+        unsigned long long b = __ballot(k0 == top);
+        int q = 0;
+        if (b == 0ull) b = __ballot(k1 == top), q = 1;
+        if (b == 0ull) b = __ballot(k2 == top), q = 2;
+        if (b == 0ull) b = __ballot(k3 == top), q = 3;
+        const int at = __builtin_amdgcn_readfirstlane(__builtin_ctzll(b));
+        const bool hit = lane == at;
+        k0 = hit && q == 0 ? kNone : k0;
+        k1 = hit && q == 1 ? kNone : k1;
+        k2 = hit && q == 2 ? kNone : k2;
+        k3 = hit && q == 3 ? kNone : k3;
+        const float pq = q == 0 ? p0 : q == 1 ? p1 : q == 2 ? p2 : p3;
+        const uint64_t tq = q == 0 ? t0 : q == 1 ? t1 : q == 2 ? t2 : t3;
+        const float pv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pq), at));
+        const uint32_t plo = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) tq, at);
+        const uint32_t phi = (uint32_t) __builtin_amdgcn_readlane((int) (uint32_t) (tq >> 32), at);
+        if (lane == i) id = 64 * q + at, pw = pv, ptr = ((uint64_t) phi << 32) | plo;
+    }
+    double s = 0.0;
+    for (int i = 0; i < k; ++i) s += (double) __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pw), i));
+    const float inv = (float) (norm == 0 ? 1.0 : norm == 2 ? 1.0 / (s + 1e-20) : 1.0 / fmax(s, 6.103515625e-05));
+    my_id = bad ? -1 : id;
+    my_w = bad ? 0.0f : (float) ((double) pw * (double) inv * (double) w_scale);
+    my_ptr = bad ? 0ull : ptr;
 }
 
 __global__ __launch_bounds__(256) void router_kernel(const float* __restrict__ logits, int n_expert, int k, RouterSpec r,
@@ -1538,7 +1599,8 @@ struct LayerHeadIn {
     const float* logits;
     const uint64_t* table;
     const void* x;
-    int n_expert, x_dtype;
+    const float* bias;   // the sigmoid router's, or NULL
+    int n_expert, x_dtype, sigmoid;
     LayerHead out;
 };
 template <int NW>
@@ -1556,20 +1618,21 @@ int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hip
     const unsigned walkers = (unsigned) (wgs < n_tiles ? wgs : n_tiles);
     if (hd) {   // workgroup 0 routes, the others walk the tiles
         hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 6, true>), dim3(walkers + 1), dim3(64 * NW), 0, s, (const void*) hd->logits,
-                           (const void*) hd->table, hd->x, st.cb.iq2s, a.skip, hd->n_expert, hd->x_dtype, a.k, a, hd->out);
+                           (const void*) hd->table, hd->x, st.cb.iq2s, hd->bias, a.skip, hd->n_expert, hd->x_dtype | (hd->sigmoid << 8), a.k, a,
+                           hd->out);
     } else {
         hipLaunchKernelGGL((gate_up_iq2s_tiles_kernel<NW, 6, false>), dim3(walkers), dim3(64 * NW), 0, s, (const void*) a.plan_ptr,
-                           (const void*) a.x.q, (const void*) a.x.d, st.cb.iq2s, a.skip, 0, 0, a.k, a, LayerHead{});
+                           (const void*) a.x.q, (const void*) a.x.d, st.cb.iq2s, (const float*) nullptr, a.skip, 0, 0, a.k, a, LayerHead{});
     }
     MAYA_LAUNCHED("gate_up_iq2s_tiles_kernel");
     return MAYA_OK;
 }
-// The single-token IQ2_S layer whose head rides in the gate/up launch (gate_up_iq2s_tiles_kernel<.., true>): the softmax
+// The single-token IQ2_S layer whose head rides in the gate/up launch (gate_up_iq2s_tiles_kernel<.., true>): either
 // router over up to 256 experts with more experts than slots, x aligned for 16-byte loads, the stream packing's shapes.
 static bool layer_head_in_gate_up_ok(const maya_moe_args& a, const RouterSpec& rs, const float* logits, int n_expert, const void* x,
                                      int x_dtype) {
     const maya_moe_layout& l = a.layout;
-    return logits && a.n_tokens == 1 && rs.kind == MAYA_ROUTER_SOFTMAX && n_expert <= 256 && a.k < n_expert && x_dtype >= 0 &&
+    return logits && a.n_tokens == 1 && n_expert <= 256 && a.k < n_expert && x_dtype >= 0 &&
            x_dtype <= 2 && ((uintptr_t) x & 15) == 0 && l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM &&
            l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 && l.n_embd >= 2048 && l.n_embd <= 8192;
 }
@@ -2578,7 +2641,8 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
         // (the second half of a call made in two: the plan, the groups and h are in the workspace)
     } else if (layer_head_in_gate_up_ok(a, rs, logits, n_expert, x, x_dtype)) {
         // one token of IQ2_S experts: route, plan, Q8_K of x and gate/up in one launch
-        const LayerHeadIn hd{logits, expert_table, x, n_expert, x_dtype, LayerHead{ids, weights, w.plan_ptr}};
+        const LayerHeadIn hd{logits, expert_table, x, rs.bias, n_expert, x_dtype, rs.kind == MAYA_ROUTER_SIGMOID ? 1 : 0,
+                             LayerHead{ids, weights, w.plan_ptr, rs.w_scale, rs.norm}};
         if ((rc = launch_layer_gate_up_iq2s(a, hd, *st, as_stream(stream)))) return rc;
         gate_up_done = true;
     } else if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&

@@ -201,3 +201,65 @@ def test_the_layer_in_two_calls_is_the_layer(lib, gt, dt, n_embd, n_ff, ne, k, n
     torch.cuda.synchronize()
     assert torch.equal(whole.ids, halves.ids) and torch.equal(whole.weights.view(torch.int32), halves.weights.view(torch.int32))
     assert torch.equal(want.view(torch.int32), got.view(torch.int32))
+
+
+@pytest.mark.parametrize("norm,with_bias", ((1, True), (0, False), (2, True)))
+def test_sigmoid_router_in_the_gate_up_launch(lib, norm, with_bias):
+    """The sigmoid router (bias, weight scale, the three normalisations) with the head in the gate/up launch: ids, weights
+    and output bit for bit those of the three-launch layer (x unaligned) and of maya_moe_route_sigmoid, on random rows,
+    equal scores (equal logits with equal bias; a bias that makes different logits meet), saturated sigmoids (p = 1 for
+    many experts: ties at the top), scores a unit in the last place apart, and rows with NaN / Inf (refused: ids -1,
+    weights 0, the output just `add`)."""
+    n_embd, n_ff, ne, k = 2048, 512, 64, 6
+    blobs = make_experts(22, 22, n_embd, n_ff, ne, 321)
+    gguf_layout, _ = lib.layout(22, 22, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+    fused, plain = lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1), lib.MoeLayer(22, 22, n_embd, n_ff, ne, k, packing=1)
+    rng = np.random.default_rng(77 + norm)
+    bias = (rng.standard_normal(ne) * 0.1).astype(np.float32)
+    bias[[3, 9]] = 0.25
+    bias_d = dev(bias)
+    router = lib.Router(lib.ROUTER_SIGMOID, norm, bias_d.data_ptr() if with_bias else 0, 2.5)
+    rows = []
+    for trial in range(12):
+        base = rng.standard_normal(ne).astype(np.float32)
+        rows.append(base)
+        c = base.copy()
+        c[[3, 9, 20]] = np.float32(1.75)                                      # equal logits (3 and 9 with equal bias too)
+        rows.append(c)
+        rows.append((base * np.float32(30.0)).astype(np.float32))             # saturated: p = 1 (or 0) for most experts
+        c = base.copy()
+        top = np.argsort(-c)[:8]
+        v = np.float32(2.0)
+        for j in top:
+            c[j] = v
+            v = np.nextafter(v, np.float32(-np.inf))                          # neighbours in the last place
+        rows.append(c)
+        rows.append((np.round(base * 2) / 2).astype(np.float32))              # a coarse grid
+    c = rng.standard_normal(ne).astype(np.float32)
+    c[11] = np.float32(np.nan)
+    rows.append(c)
+    c = rng.standard_normal(ne).astype(np.float32)
+    c[5] = np.float32(np.inf)
+    rows.append(c)
+    rows = np.stack(rows).astype(np.float32)
+    want_ids, want_w = lib.route_sigmoid(dev(rows), bias_d if with_bias else None, k, 2.5, norm)
+    xa = torch.zeros(n_embd + 8, dtype=torch.float32, device="cuda")
+    x32 = torch.randn(n_embd, device="cuda")
+    add = torch.randn(1, n_embd, device="cuda")
+    x_al, x_un = xa[:n_embd].view(1, -1), xa[2:2 + n_embd].view(1, -1)
+    bad = 0
+    for i in range(rows.shape[0]):
+        lg = dev(rows[i:i + 1])
+        x_al.copy_(x32.view(1, -1))
+        out_f = fused.forward(store.table, lg, x_al, add=add, router=router).clone()
+        x_un.copy_(x32.view(1, -1))
+        out_p = plain.forward(store.table, lg, x_un, add=add, router=router)
+        ok = (torch.equal(fused.ids[0], want_ids[i]) and torch.equal(fused.weights[0].view(torch.int32), want_w[i].view(torch.int32))
+              and torch.equal(plain.ids[0], want_ids[i]) and torch.equal(out_f.view(torch.int32), out_p.view(torch.int32)))
+        if not ok:
+            bad += 1
+            print("row", i, fused.ids[0].tolist(), want_ids[i].tolist(), flush=True)
+    torch.cuda.synchronize()
+    assert bad == 0, bad
+    assert int(want_ids[-1, 0]) == -1 and int(want_ids[-2, 0]) == -1          # the refused rows were in the set
