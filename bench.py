@@ -32,9 +32,9 @@ IQ2_S = 22
 HBM_PEAK = 8.0e12
 PARITY_BAR = 1e-3
 # HBM bytes of one gate/up launch on this workload from rocprofv3's FETCH_SIZE and WRITE_SIZE (two runs, each scaled by
-# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 73,961.4 KiB read + 64.0 KiB written
+# what the counter reads for a plain device copy of known size: 2.000 and 1.000): 74,179.7 KiB read + 64.1 KiB written
 # (profiles/decode_iq2s_hbm_traffic_pmc.txt)
-GATE_UP_TRAFFIC_BYTES = int((73961.4 + 64.0) * 1024)
+GATE_UP_TRAFFIC_BYTES = int((74179.7 + 64.1) * 1024)
 
 
 def synth_experts_on_device(torch, n_expert, blob_bytes, seed):
