@@ -91,6 +91,31 @@ __device__ __forceinline__ void down_block_of_grid(int& row_block, int& token) {
     }
 }
 
+// The value of lane (lane ^ MASK), without address arithmetic: a DPP operand for masks 1, 2 (quad permutes) and 8 (a
+// rotation by 8 inside a row of 16 lanes), ds_swizzle for 4 and 16 (an LDS-crossbar exchange inside 32 lanes whose
+// pattern is an immediate), the gfx950 half-wave swap for 32.  (__shfl_xor costs four vector instructions of index
+// arithmetic per call before its ds_bpermute.)
+template <int MASK>
+__device__ __forceinline__ float xor_lane(float v) {
+    const int i = __float_as_int(v);
+    if constexpr (MASK == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0xB1, 0xf, 0xf, true));        // quad_perm [1,0,3,2]
+    else if constexpr (MASK == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, i, 0x128, 0xf, 0xf, true));  // row_ror:8
+    else if constexpr (MASK == 4) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x101F));                    // swap 4
+    else if constexpr (MASK == 16) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x401F));                   // swap 16
+    else {
+        static_assert(MASK == 32, "masks inside a wave");
+        const auto r = __builtin_amdgcn_permlane32_swap(i, i, false, false);   // r[0] = (lower, lower), r[1] = (upper, upper)
+        return __int_as_float((threadIdx.x & 32) ? r[0] : r[1]);
+    }
+}
+// v + the value of lane ^ 32 (both halves get lower + upper, the order __shfl_xor's form adds them in)
+__device__ __forceinline__ float add_other_half(float v) {
+    const int i = __float_as_int(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(i, i, false, false);
+    return __int_as_float(r[0]) + __int_as_float(r[1]);
+}
+
 // Q8_K rounding of a 256-value block held by 8 consecutive lanes, 32 values a lane: the arithmetic of the reference's
 // quantize_q8_K_kernel (src/kernels/cuda/quantize_act.cu:161-207) and codes, bit for bit, 4 codes a word in the order
 // of v.  The block's scale comes from the signed value at the FIRST largest magnitude.  Its magnitude is the largest

@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include "maya_host.h"
+#include "maya_dev.hpp"
 
 namespace maya {
 
@@ -76,14 +77,22 @@ __global__ __launch_bounds__(256) void exl3_inner_kernel(const uint32_t* __restr
 // Stage h < 64 pairs lane L with lane L ^ h (the lower index adds, the upper takes lower - upper), stage 64 pairs the
 // lane's own two values: the butterflies, their order and every rounding are the reference's
 // (src/kernels/cpu/exl3_ref.cpp:61-75), so the same bits.
+// The partner's value comes through a DPP operand, a swizzle or the half-wave swap (xor_lane), not through __shfl_xor's
+// LDS-routed permute: six exchanges a value, each of which was an LDS round trip.
+template <int H>
+__device__ __forceinline__ void had128_stage(float& v0, float& v1, int lane) {
+    const float p0 = xor_lane<H>(v0), p1 = xor_lane<H>(v1);
+    const bool upper = (lane & H) != 0;
+    v0 = upper ? __fsub_rn(p0, v0) : __fadd_rn(v0, p0);
+    v1 = upper ? __fsub_rn(p1, v1) : __fadd_rn(v1, p1);
+}
 __device__ __forceinline__ void had128_wave(float& v0, float& v1, int lane) {
-#pragma unroll
-    for (int h = 1; h < 64; h <<= 1) {
-        const float p0 = __shfl_xor(v0, h, 64), p1 = __shfl_xor(v1, h, 64);
-        const bool upper = (lane & h) != 0;
-        v0 = upper ? __fsub_rn(p0, v0) : __fadd_rn(v0, p0);
-        v1 = upper ? __fsub_rn(p1, v1) : __fadd_rn(v1, p1);
-    }
+    had128_stage<1>(v0, v1, lane);
+    had128_stage<2>(v0, v1, lane);
+    had128_stage<4>(v0, v1, lane);
+    had128_stage<8>(v0, v1, lane);
+    had128_stage<16>(v0, v1, lane);
+    had128_stage<32>(v0, v1, lane);
     const float a = v0, c = v1;
     v0 = __fadd_rn(a, c);
     v1 = __fsub_rn(a, c);
@@ -128,12 +137,31 @@ __device__ __forceinline__ void rotate_in(const float* __restrict__ x, const uin
                                           __half* xr) {
     (void) tmp;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int b = wave; b < (k >> 7); b += kExThreads / 64) {
-        const int i0 = b * 128 + lane;
-        float v0 = __fmul_rn(x[i0], f16_bits_to_f32(suh[i0])), v1 = __fmul_rn(x[i0 + 64], f16_bits_to_f32(suh[i0 + 64]));
-        had128_wave(v0, v1, lane);
-        xr[PAIRED ? paired_pos(i0) : i0] = __float2half_rn(v0);
-        xr[PAIRED ? paired_pos(i0 + 64) : i0 + 64] = __float2half_rn(v1);
+    const int nb = k >> 7;
+    // a wave's blocks three at a time: their loads go out together (one block a pass of the loop is one trip to memory a
+    // pass: the compiler waits for a pass's loads before it issues the next pass's)
+    constexpr int kAtOnce = 3, kWaves = kExThreads / 64;
+    for (int b0 = wave; b0 < nb; b0 += kAtOnce * kWaves) {
+        float xa[kAtOnce], xb[kAtOnce];
+        uint16_t sa[kAtOnce], sb[kAtOnce];
+#pragma unroll
+        for (int u = 0; u < kAtOnce; ++u) {
+            const int b = b0 + u * kWaves;
+            const int i0 = (b < nb ? b : b0) * 128 + lane;   // (past the end: the first block again, its result dropped)
+            xa[u] = x[i0], xb[u] = x[i0 + 64];
+            sa[u] = suh[i0], sb[u] = suh[i0 + 64];
+        }
+#pragma unroll
+        for (int u = 0; u < kAtOnce; ++u) {
+            const int b = b0 + u * kWaves;
+            if (b < nb) {
+                const int i0 = b * 128 + lane;
+                float v0 = __fmul_rn(xa[u], f16_bits_to_f32(sa[u])), v1 = __fmul_rn(xb[u], f16_bits_to_f32(sb[u]));
+                had128_wave(v0, v1, lane);
+                xr[PAIRED ? paired_pos(i0) : i0] = __float2half_rn(v0);
+                xr[PAIRED ? paired_pos(i0 + 64) : i0 + 64] = __float2half_rn(v1);
+            }
+        }
     }
     __syncthreads();
 }
