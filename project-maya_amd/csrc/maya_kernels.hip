@@ -1588,12 +1588,6 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
 }
-// (The kernel is compiled for 6 waves a SIMD - three workgroups of up to 8 waves a compute unit, what is launched - not 8:
-// with the head's prologue in it the kernel needs 73 registers, and at 64 it spilled 36 bytes a lane to scratch memory:
-// 6.8 MB written and read back a launch, 2.1 us of the layer.)
-// one token: the tile-streaming form, launched with the workgroups the chip holds at once (asked of the runtime once a
-// shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
-// tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
 // the head's inputs when it rides in the gate/up launch, and where its results go
 struct LayerHeadIn {
     const float* logits;
@@ -1603,6 +1597,14 @@ struct LayerHeadIn {
     int n_expert, x_dtype, sigmoid;
     LayerHead out;
 };
+// One token: the tile-streaming form, launched with the workgroups the chip holds at once (asked of the runtime once a
+// shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
+// tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
+// The kernel is compiled for 6 waves a SIMD - three workgroups of up to 8 waves a compute unit, what is launched - not 8:
+// with the head's prologue in it the kernel needs 73-77 registers, and at 64 it spilled 36 bytes a lane to scratch
+// memory: 6.8 MB written and read back a launch, 2.1 us of the layer.  Windows keep gate_up_iq2s_pos_kernel: the tile
+// stream with the resident workgroups shared out among the tokens (a token's codes in a workgroup's registers) was built
+// and is slower there (configs[2]: 260 us against 234).
 template <int NW>
 int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hipStream_t s, const LayerHeadIn* hd = nullptr) {
     static int per_cu = 0;
