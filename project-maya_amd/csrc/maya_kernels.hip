@@ -1017,6 +1017,45 @@ struct GroupLds {
 __device__ __forceinline__ void group_entries(GroupLds& g, int n, uint64_t* __restrict__ grp_ptr, int32_t* __restrict__ grp_start,
                                               int32_t* __restrict__ grp_ent, int32_t* __restrict__ n_groups) {
     const int e = threadIdx.x;
+    if (n <= 64) {
+        // Up to 64 entries: one wave, registers only.  A lane learns which lanes hold its blob (n reads of a lane's value),
+        // and everything else is a count of bits: its group's leader (the first such lane), its rank in the group, the
+        // groups before its own (leaders below its leader), the entries before its group (lanes whose leader is below its
+        // own).  The same groups, order and members as the general form below, value for value.
+        if (e >= 64) return;
+        const uint64_t ptr = e < n ? g.ptr[e] : 0ull;
+        const uint32_t plo = (uint32_t) ptr, phi = (uint32_t) (ptr >> 32);
+        unsigned long long same = 0ull;
+        for (int f = 0; f < n; ++f) {
+            const uint32_t flo = (uint32_t) __builtin_amdgcn_readlane((int) plo, f), fhi = (uint32_t) __builtin_amdgcn_readlane((int) phi, f);
+            if (flo == plo && fhi == phi) same |= 1ull << f;
+        }
+        const bool valid = ptr != 0ull;
+        if (!valid) same = 0ull;
+        const int leader = valid ? __builtin_ctzll(same) : -1;
+        const unsigned long long below = (1ull << e) - 1ull;
+        const int rank = __popcll(same & below);
+        const unsigned long long leaders = __ballot(leader == e);
+        const int gi = valid ? __popcll(leaders & ((1ull << leader) - 1ull)) : -1;
+        const int ng = __popcll(leaders);
+        int start = 0;
+        for (int f = 0; f < n; ++f) {
+            const int lf = __builtin_amdgcn_readlane(leader, f);
+            start += (lf >= 0 && lf < leader) ? 1 : 0;
+        }
+        const int total = __popcll(__ballot(valid));
+        if (leader == e) {
+            grp_ptr[gi] = ptr;
+            grp_start[gi] = start;
+        }
+        if (e == 0) {
+            grp_start[ng] = total;
+            *n_groups = ng;
+        }
+        if (valid) grp_ent[start + rank] = e;
+        if (e >= total && e < n) grp_ent[e] = -1;
+        return;
+    }
     g.count[e] = 0;
     int leader = -1;
     if (e < n && g.ptr[e] != 0ull) {
