@@ -195,7 +195,7 @@ def single_q4k(K, W):
             "config": {"workload": "configs[0]: one expert GLU, gate/up [2048x7168] + down [7168x2048] quantized to Q4_K from "
                                    "N(0,0.02), 1 token F32 N(0,1); 16 such experts rotate over the steps",
                        "algorithmic_bytes_per_step": nbytes},
-            "roofline": hbm_roofline("layer (layer_head_kernel + gate_up_q4k_pos_kernel + down_q4k_pos_kernel)", nbytes, sec, TRAFFIC_BYTES["single_q4k"]),
+            "roofline": hbm_roofline("layer (gate_up_q4k_pos_kernel with the head in the same launch + down_q4k_pos_kernel)", nbytes, sec, TRAFFIC_BYTES["single_q4k"]),
             # for bench.py's parity leg (the CPU path's expert on the same bytes, after the timed region)
             "_parity": {"kind": "expert", "type": lib.Q4_K, "n_embd": E, "n_ff": FF, "blob": pool[:bb], "x": x, "out": out0}}
 

@@ -476,6 +476,146 @@ struct LayerHead {
     float w_scale;           // the sigmoid router's weight scale and normalisation
     int norm;
 };
+// the head's inputs when it rides in the gate/up launch, and where its results go
+struct LayerHeadIn {
+    const float* logits;
+    const uint64_t* table;
+    const void* x;
+    const float* bias;   // the sigmoid router's, or NULL
+    int n_expert, x_dtype, sigmoid;
+    LayerHead out;
+};
+// The head of a one-token layer inside a gate/up launch whose workgroups are a (gate row, up row) pair's 2 * 32 NW
+// positions, grid (row blocks + 1, k): called by every thread once.  The workgroup (last column, 0) is the exact router
+// (ids, weights, plan: hd.out); the rest of that column leaves.  Every other workgroup picks the experts on its last
+// wave (up lanes only) from the ORDER of the logits - the exact router on the same wave when two of them are too close to
+// call - while the waves with gate lanes round their positions' x to Q8_K in registers (a 256-value block is 8 lanes: the
+// lane of position u holds the values o0 .. o0 + 15 and o1 .. o1 + 15 of x, o0 < o1 inside one block) and hand codes and
+// scale to the up lanes through LDS.  y: the position's 32 codes in that order, d: its block's scale, blob: the expert of
+// slot blockIdx.y.  False: the thread has nothing more to do in this launch.
+template <int NW>
+__device__ __forceinline__ bool head_in_gate_up(const LayerHeadIn& hd, int n_ent, const int32_t* skip, bool is_up, int u, int o0, int o1,
+                                                int (&y)[8], float& d, uint64_t& blob) {
+    constexpr int NU = 32 * NW;
+    __shared__ uint64_t s_blob[MAYA_MAX_K];
+    __shared__ float s_lv[256];
+    __shared__ uint64_t s_tab[256];
+    __shared__ int s_y[9][NU];
+    const int t = threadIdx.x, lane = t & 63, ne = hd.n_expert;
+    const bool picker = t >= 64 * (NW - 1), sigm = hd.sigmoid != 0;
+    float lv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint64_t tab[4] = {0ull, 0ull, 0ull, 0ull};
+    if (picker) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int x = 64 * r + lane;
+            lv[r] = x < ne ? hd.logits[x] : -INFINITY;
+            tab[r] = x < ne ? hd.table[x] : 0ull;
+            if (hd.bias) bv[r] = x < ne ? hd.bias[x] : 0.0f;
+        }
+    }
+    if (blockIdx.x == gridDim.x - 1) {   // the router (it looks at no skip flag, like the head kernel)
+        if (blockIdx.y != 0 || !picker) return false;
+        int id;
+        float w;
+        uint64_t ptr;
+        if (sigm) {
+            float pr[4], sc[4];
+            const bool fin = sigmoid_scores(lv, bv, hd.bias != nullptr, ne, pr, sc);
+            route_wave_sigmoid(pr, sc, fin, tab, ne, n_ent, hd.out.norm, hd.out.w_scale, id, w, ptr);
+        } else {
+            route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+        }
+        if (lane < n_ent) {
+            hd.out.ids[lane] = id;
+            hd.out.weights[lane] = w;
+            hd.out.plan[lane] = ptr;
+        }
+        return false;
+    }
+    if (skip && *skip) return false;
+    if (picker) {
+        __builtin_amdgcn_s_setprio(3);   // the workgroup waits for this wave: it goes first on its SIMD
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_tab[64 * r + lane] = tab[r];
+        int id;
+        uint64_t ptr;
+        if (sigm) {
+            // the scores are the exact router's own keys: any strictly descending order of the picks is its order
+            float pr[4], sc[4];
+            const bool fin = sigmoid_scores(lv, bv, hd.bias != nullptr, ne, pr, sc);
+            if (route_wave_order_only(sc, fin, ne, n_ent, s_lv, 0.0f, INFINITY, id)) {
+                ptr = s_tab[lane < n_ent ? id : 0];
+            } else {
+                float w;
+                route_wave_sigmoid(pr, sc, fin, tab, ne, n_ent, hd.out.norm, hd.out.w_scale, id, w, ptr);
+            }
+        } else if (route_wave_order_only(lv, true, ne, n_ent, s_lv, 1e-6f, 60.0f, id)) {
+            ptr = s_tab[lane < n_ent ? id : 0];
+        } else {
+            float w;
+            route_wave_softmax(lv, tab, ne, n_ent, id, w, ptr);
+        }
+        if (lane < n_ent) s_blob[lane] = ptr;
+        __builtin_amdgcn_s_setprio(0);
+    }
+    float v[32];
+    if (!is_up) {
+        if (hd.x_dtype == MAYA_DT_F32) {
+            const float4 *xa = (const float4*) ((const float*) hd.x + o0), *xb = (const float4*) ((const float*) hd.x + o1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 lo = xa[i], hi = xb[i];
+                v[4 * i] = lo.x, v[4 * i + 1] = lo.y, v[4 * i + 2] = lo.z, v[4 * i + 3] = lo.w;
+                v[16 + 4 * i] = hi.x, v[16 + 4 * i + 1] = hi.y, v[16 + 4 * i + 2] = hi.z, v[16 + 4 * i + 3] = hi.w;
+            }
+        } else {
+            const uint4 *xa = (const uint4*) ((const uint16_t*) hd.x + o0), *xb = (const uint4*) ((const uint16_t*) hd.x + o1);
+            uint32_t w4[16];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const uint4 lo = xa[i], hi = xb[i];
+                w4[4 * i] = lo.x, w4[4 * i + 1] = lo.y, w4[4 * i + 2] = lo.z, w4[4 * i + 3] = lo.w;
+                w4[8 + 4 * i] = hi.x, w4[8 + 4 * i + 1] = hi.y, w4[8 + 4 * i + 2] = hi.z, w4[8 + 4 * i + 3] = hi.w;
+            }
+            if (hd.x_dtype == MAYA_DT_BF16) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    v[2 * j] = __uint_as_float(w4[j] << 16);
+                    v[2 * j + 1] = __uint_as_float(w4[j] & 0xffff0000u);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    v[2 * j] = f16_bits_to_f32((uint16_t) (w4[j] & 0xffffu));
+                    v[2 * j + 1] = f16_bits_to_f32((uint16_t) (w4[j] >> 16));
+                }
+            }
+        }
+    }
+    d = 0.0f;
+    // (a wave with a gate lane rounds: the block's 8 lanes are all gate lanes or all up lanes, NU being a multiple of 8)
+    if (64 * (t >> 6) < NU) {
+        q8k_round_lane32(v, [&](int i) { return i < 16 ? (o0 & 255) + i : (o1 & 255) + i - 16; }, y, d);
+        if (!is_up) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s_y[i][u] = y[i];
+            s_y[8][u] = __float_as_int(d);
+        }
+    }
+    __syncthreads();
+    if (is_up) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = s_y[i][u];
+        d = __int_as_float(s_y[8][u]);
+    }
+    const uint64_t bl = s_blob[blockIdx.y];
+    const uint32_t lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) bl);
+    const uint32_t hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (bl >> 32));
+    blob = ((uint64_t) hi << 32) | lo;
+    return blob != 0ull;
+}
+
 // The leading arguments are what the kernel asks of memory first; as plain pointers and integers at the head of the
 // argument list they arrive in scalar registers with the dispatch (a structure passed by value is read from memory
 // first).  HEAD: p0 = the logits [n_expert], p1 = the table [n_expert] of blob addresses (0 = absent), p2 = x [n_embd] of

@@ -84,30 +84,37 @@ __device__ __forceinline__ int sum32_codes(const int (&y)[8]) {
 
 // ---- gate/up, n_embd = 1024 NW: a workgroup of NW waves = the 2 * 32 NW sub-block positions of a (gate row, up row) pair;
 // grid (n_ff / ROWS, entries); entry e = token e / k, slot e % k.  Rows in batches of 8 (two quads), a quad ahead.
-template <int NW, int ROWS, int MINW>
-__global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1s_pos_kernel(maya_moe_args a, Codebooks cb) {
+// HEAD (one token): the layer's head rides in this launch (head_in_gate_up) - grid (n_ff / ROWS + 1, k).
+template <int NW, int ROWS, int MINW, bool HEAD = false>
+__global__ __launch_bounds__(64 * NW, MINW) void gate_up_iq1s_pos_kernel(maya_moe_args a, Codebooks cb, LayerHeadIn hd) {
     static_assert(ROWS % 8 == 0, "a batch is two quads");
     constexpr int NU = 32 * NW;
     __shared__ __align__(16) int lds[kFast1LdsWords];
     __shared__ float part[2][2 * NW][8];
-    if (a.skip && *a.skip) return;
-    const int e = blockIdx.y;
-    const uint64_t blob = a.plan_ptr[e];
-    if (blob == 0ull) return;
-    stage_iq1s_table<64 * NW>(lds, cb);
-    const uint2* grid = (const uint2*) lds;
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
     const int u = is_up ? t - NU : t;
-    const int tok = e / a.k;
+    const int e = blockIdx.y;
+    uint64_t blob;
     int y[8];
-    {
+    float dy8;
+    if constexpr (HEAD) {
+        float d;
+        if (!head_in_gate_up<NW>(hd, a.k, a.skip, is_up, u, 32 * u, 32 * u + 16, y, d, blob)) return;
+        dy8 = d * 0.125f;
+    } else {
+        if (a.skip && *a.skip) return;
+        blob = a.plan_ptr[e];
+        if (blob == 0ull) return;
+        const int tok = e / a.k;
         const int4* q = (const int4*) (a.x.q + (size_t) tok * (32 * NU));
         const int4 ya = q[2 * u], yb = q[2 * u + 1];
         y[0] = ya.x, y[1] = ya.y, y[2] = ya.z, y[3] = ya.w, y[4] = yb.x, y[5] = yb.y, y[6] = yb.z, y[7] = yb.w;
+        dy8 = a.x.d[(size_t) tok * NU + u] * 0.125f;
     }
+    stage_iq1s_table<64 * NW>(lds, cb);
+    const uint2* grid = (const uint2*) lds;
     const int sy = sum32_codes(y);
-    const float dy8 = a.x.d[(size_t) tok * NU + u] * 0.125f;
     constexpr uint32_t qb = NU / 8 * 50 * 4;  // bytes of a quad of rows
     const int n_ff = a.layout.n_ff, r0 = blockIdx.x * ROWS;
     const __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob + a.layout.gate_off, (uint32_t) (a.layout.down_off - a.layout.gate_off));

@@ -63,25 +63,42 @@ __device__ __forceinline__ float pos_q4k_value(const PosQ4K& p, const u32x4 hdr,
 // grid (n_ff / ROWS, entries); entry e = token e / k, slot e % k.  Rows in batches of 8, one row ahead in registers.
 // AHEAD (8 rows): all of a lane's rows are requested up front - the launches of a few entries, whose workgroups do not fill
 // the chip and would otherwise run at the memory's latency a row.
-template <int NW, int ROWS, int MINW, bool AHEAD = false>
-__global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe_args a) {
+// HEAD (one token): the layer's head rides in this launch (head_in_gate_up) - grid (n_ff / ROWS + 1, k).
+template <int NW, int ROWS, int MINW, bool AHEAD = false, bool HEAD = false>
+__global__ __launch_bounds__(64 * NW, MINW) void gate_up_q4k_pos_kernel(maya_moe_args a, LayerHeadIn hd) {
     static_assert(ROWS % 8 == 0, "rows come in batches of 8");
     static_assert(!AHEAD || ROWS == 8, "every row up front: one batch");
     constexpr int NU = 32 * NW;
     __shared__ float part[2][2 * NW][8];
-    if (a.skip && *a.skip) return;
-    // (a window's entries in the order of grp_ent where one is given: the entries of an expert side by side; -1 ends it)
-    const int e = (a.grp_ent && !a.grp_ptr) ? a.grp_ent[blockIdx.y] : (int) blockIdx.y;
-    if (e < 0) return;
-    const uint64_t blob = a.plan_ptr[e];
-    if (blob == 0ull) return;
     const int t = threadIdx.x, lane = t & 63, hw = t >> 5;
     const bool is_up = t >= NU;
     const int u = is_up ? t - NU : t;
-    const int tok = e / a.k;
     PosQ4K p;
     pos_q4k_init(p, u, is_up ? (uint32_t) (a.layout.up_off - a.layout.gate_off) : 0u);
-    pos_q4k_codes(p, u, a.x.q + (size_t) tok * (32 * NU), a.x.d + (size_t) tok * NU, a.x.bsums + (size_t) tok * (2 * NU));
+    int e;
+    uint64_t blob;
+    if constexpr (HEAD) {
+        // position u holds the block's values v0 .. v0 + 15 (against the low nibbles) and v0 + 32 .. v0 + 47 (the high ones)
+        const int v0 = 256 * (u >> 3) + 64 * ((u & 7) >> 1) + 16 * (u & 1);
+        int y[8];
+        float d;
+        e = (int) blockIdx.y;
+        if (!head_in_gate_up<NW>(hd, a.k, a.skip, is_up, u, v0, v0 + 32, y, d, blob)) return;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p.ylo[i] = y[i], p.yhi[i] = y[4 + i];
+        p.dx = d;
+        p.slo = dot4(0x01010101, p.ylo[0], dot4(0x01010101, p.ylo[1], dot4(0x01010101, p.ylo[2], dot4(0x01010101, p.ylo[3], 0))));
+        p.shi = dot4(0x01010101, p.yhi[0], dot4(0x01010101, p.yhi[1], dot4(0x01010101, p.yhi[2], dot4(0x01010101, p.yhi[3], 0))));
+    } else {
+        if (a.skip && *a.skip) return;
+        // (a window's entries in the order of grp_ent where one is given: the entries of an expert side by side; -1 ends it)
+        e = (a.grp_ent && !a.grp_ptr) ? a.grp_ent[blockIdx.y] : (int) blockIdx.y;
+        if (e < 0) return;
+        blob = a.plan_ptr[e];
+        if (blob == 0ull) return;
+        const int tok = e / a.k;
+        pos_q4k_codes(p, u, a.x.q + (size_t) tok * (32 * NU), a.x.d + (size_t) tok * NU, a.x.bsums + (size_t) tok * (2 * NU));
+    }
     constexpr uint32_t rb = NU / 8 * 144;   // bytes of a row
     const int n_ff = a.layout.n_ff, r0 = blockIdx.x * ROWS;
     const __amdgpu_buffer_rsrc_t rs = weight_rsrc(blob + a.layout.gate_off, (uint32_t) (a.layout.down_off - a.layout.gate_off));

@@ -1627,15 +1627,6 @@ int launch_gate_up_iq2s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
     MAYA_LAUNCHED("gate_up_iq2s_pos_kernel");
     return MAYA_OK;
 }
-// the head's inputs when it rides in the gate/up launch, and where its results go
-struct LayerHeadIn {
-    const float* logits;
-    const uint64_t* table;
-    const void* x;
-    const float* bias;   // the sigmoid router's, or NULL
-    int n_expert, x_dtype, sigmoid;
-    LayerHead out;
-};
 // One token: the tile-streaming form, launched with the workgroups the chip holds at once (asked of the runtime once a
 // shape), at most three a compute unit: measured on 7168 x 2048, top-8, 768 workgroups 18.5 us, 1024 (all resident, two
 // tiles each) 20.1 us, 512 20.4 us, 256 24.1 us - a workgroup's cold start is paid per workgroup, latency hiding per wave.
@@ -1668,14 +1659,22 @@ int launch_gate_up_iq2s_tiles(const maya_moe_args& a, const DeviceState& st, hip
     MAYA_LAUNCHED("gate_up_iq2s_tiles_kernel");
     return MAYA_OK;
 }
-// The single-token IQ2_S layer whose head rides in the gate/up launch (gate_up_iq2s_tiles_kernel<.., true>): either
-// router over up to 256 experts with more experts than slots, x aligned for 16-byte loads, the stream packing's shapes.
+// The single-token layer whose head rides in the gate/up launch (gate_up_iq2s_tiles_kernel<.., true>,
+// gate_up_q4k_pos_kernel<.., true>): either router over up to 256 experts with more experts than slots, x aligned for
+// 16-byte loads, IQ2_S, Q4_K or IQ1_S gate/up rows in the stream packing's shapes.  (IQ1_M keeps its head launch: its
+// gate/up kernel with the head in it was 6.3 us slower a launch than without, more than the 4.8 us head launch it replaces;
+// IQ1_S gains 1.4 us a layer, Q4_K 0.6, and the one-expert Q4_K layer of few workgroups 2.7 of 16.)
+bool gate_up_q4k_pos_ok(const maya_moe_args& a);
+bool gate_up_iq1s_pos_ok(const maya_moe_args& a);
 static bool layer_head_in_gate_up_ok(const maya_moe_args& a, const RouterSpec& rs, const float* logits, int n_expert, const void* x,
                                      int x_dtype) {
     const maya_moe_layout& l = a.layout;
-    return logits && a.n_tokens == 1 && n_expert <= 256 && a.k < n_expert && x_dtype >= 0 &&
-           x_dtype <= 2 && ((uintptr_t) x & 15) == 0 && l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM &&
-           l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 && l.n_embd >= 2048 && l.n_embd <= 8192;
+    if (!(logits && a.n_tokens == 1 && n_expert <= 256 && a.k < n_expert && x_dtype >= 0 && x_dtype <= 2 && ((uintptr_t) x & 15) == 0))
+        return false;
+    if (l.gate_type == kQ4_K) return gate_up_q4k_pos_ok(a);
+    if (l.gate_type == kIQ1_S) return gate_up_iq1s_pos_ok(a);
+    return l.gate_type == kIQ2_S && l.up_type == kIQ2_S && l.packing == MAYA_PACK_STREAM && l.n_ff % 16 == 0 && l.n_embd % 1024 == 0 &&
+           l.n_embd >= 2048 && l.n_embd <= 8192;
 }
 static int launch_layer_gate_up_iq2s(const maya_moe_args& a, const LayerHeadIn& hd, const DeviceState& st, hipStream_t s) {
     switch (a.layout.n_embd / 1024) {
@@ -1777,9 +1776,11 @@ bool down_iq1s_pos_ok(const maya_moe_args& a) {
     return (l.down_type == kIQ1_S || l.down_type == kIQ1_M) && l.packing == MAYA_PACK_STREAM && a.k <= 8 &&
            (l.n_ff == 1024 || l.n_ff == 1536 || l.n_ff == 2048) && l.n_embd % 16 == 0 && (l.down_off & 15) == 0;
 }
-int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s) {
-    const dim3 grid((unsigned) (a.layout.n_ff / 16), (unsigned) (a.n_tokens * a.k));
+int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipStream_t s, const LayerHeadIn* hd = nullptr) {
+    // (IQ1_S with the head in the launch: one more column, whose first workgroup is the router)
+    const dim3 grid((unsigned) (a.layout.n_ff / 16) + (hd ? 1u : 0u), (unsigned) (a.n_tokens * a.k));
     if (a.layout.gate_type == kIQ1_M) {
+        if (hd) return fail(MAYA_E_UNSUPPORTED, "gate_up: the IQ1_M rows take no head in their launch");
         switch (a.layout.n_embd / 1024) {
             case 2: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<2, 16, 8>), grid, dim3(128), 0, s, a, st.cb); break;
             case 3: hipLaunchKernelGGL((gate_up_iq1m_pos_kernel<3, 16, 8>), grid, dim3(192), 0, s, a, st.cb); break;
@@ -1792,15 +1793,20 @@ int launch_gate_up_iq1s_pos(const maya_moe_args& a, const DeviceState& st, hipSt
         MAYA_LAUNCHED("gate_up_iq1m_pos_kernel");
         return MAYA_OK;
     }
+    const LayerHeadIn h = hd ? *hd : LayerHeadIn{};
+#define MAYA_IQ1(NWV)                                                                                                          \
+    if (hd) hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<NWV, 16, 6, true>), grid, dim3(64 * NWV), 0, s, a, st.cb, h);             \
+    else hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a, st.cb, h);
     switch (a.layout.n_embd / 1024) {
-        case 2: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<2, 16, 8>), grid, dim3(128), 0, s, a, st.cb); break;
-        case 3: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<3, 16, 8>), grid, dim3(192), 0, s, a, st.cb); break;
-        case 5: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<5, 16, 8>), grid, dim3(320), 0, s, a, st.cb); break;
-        case 4: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<4, 16, 8>), grid, dim3(256), 0, s, a, st.cb); break;
-        case 6: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<6, 16, 8>), grid, dim3(384), 0, s, a, st.cb); break;
-        case 7: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<7, 16, 8>), grid, dim3(448), 0, s, a, st.cb); break;
-        default: hipLaunchKernelGGL((gate_up_iq1s_pos_kernel<8, 16, 8>), grid, dim3(512), 0, s, a, st.cb); break;
+        case 2: MAYA_IQ1(2) break;
+        case 3: MAYA_IQ1(3) break;
+        case 4: MAYA_IQ1(4) break;
+        case 5: MAYA_IQ1(5) break;
+        case 6: MAYA_IQ1(6) break;
+        case 7: MAYA_IQ1(7) break;
+        default: MAYA_IQ1(8) break;
     }
+#undef MAYA_IQ1
     MAYA_LAUNCHED("gate_up_iq1s_pos_kernel");
     return MAYA_OK;
 }
@@ -1854,14 +1860,18 @@ bool down_q4k_pos_ok(const maya_moe_args& a) {
     return l.down_type == kQ4_K && l.packing == MAYA_PACK_STREAM && a.k <= 8 && down_pos_nff_ok(l.n_ff) && l.n_embd % 16 == 0 &&
            (l.down_off & 15) == 0;
 }
-int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s) {
+int launch_gate_up_q4k_pos(const maya_moe_args& a, hipStream_t s, const LayerHeadIn* hd = nullptr) {
     // 16 rows a workgroup, 8 - all requested up front - when the call has so few entries that 16 would leave compute units idle
     const bool small = (long long) (a.layout.n_ff / 16) * a.n_tokens * a.k < 512;
     const int rows = small ? 8 : 16;
-    const dim3 grid((unsigned) (a.layout.n_ff / rows), (unsigned) (a.n_tokens * a.k));
-#define MAYA_Q4(NWV)                                                                                              \
-    if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 4, true>), grid, dim3(64 * NWV), 0, s, a);    \
-    else hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a);
+    // (with the head in the launch: one more column, whose first workgroup is the router)
+    const dim3 grid((unsigned) (a.layout.n_ff / rows) + (hd ? 1u : 0u), (unsigned) (a.n_tokens * a.k));
+    const LayerHeadIn h = hd ? *hd : LayerHeadIn{};
+#define MAYA_Q4(NWV)                                                                                                       \
+    if (hd && small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 4, true, true>), grid, dim3(64 * NWV), 0, s, a, h);   \
+    else if (hd) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 6, false, true>), grid, dim3(64 * NWV), 0, s, a, h);     \
+    else if (small) hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 8, 4, true>), grid, dim3(64 * NWV), 0, s, a, h);          \
+    else hipLaunchKernelGGL((gate_up_q4k_pos_kernel<NWV, 16, 8>), grid, dim3(64 * NWV), 0, s, a, h);
     switch (a.layout.n_embd / 1024) {
         case 2: MAYA_Q4(2) break;
         case 3: MAYA_Q4(3) break;
@@ -2681,10 +2691,14 @@ static int layer_decode_core(const maya_moe_layout* l, const uint64_t* expert_ta
     if (!head) {
         // (the second half of a call made in two: the plan, the groups and h are in the workspace)
     } else if (layer_head_in_gate_up_ok(a, rs, logits, n_expert, x, x_dtype)) {
-        // one token of IQ2_S experts: route, plan, Q8_K of x and gate/up in one launch
+        // one token of IQ2_S, Q4_K or IQ1_S experts: route, plan, Q8_K of x and gate/up in one launch
         const LayerHeadIn hd{logits, expert_table, x, rs.bias, n_expert, x_dtype, rs.kind == MAYA_ROUTER_SIGMOID ? 1 : 0,
                              LayerHead{ids, weights, w.plan_ptr, rs.w_scale, rs.norm}};
-        if ((rc = launch_layer_gate_up_iq2s(a, hd, *st, as_stream(stream)))) return rc;
+        hipStream_t s = as_stream(stream);
+        if ((rc = l->gate_type == kQ4_K   ? launch_gate_up_q4k_pos(a, s, &hd)
+                  : l->gate_type == kIQ2_S ? launch_layer_gate_up_iq2s(a, hd, *st, s)
+                                           : launch_gate_up_iq1s_pos(a, *st, s, &hd)))
+            return rc;
         gate_up_done = true;
     } else if (logits && q8k_act(l->gate_type) && n_expert <= MAYA_MAX_EXPERTS && x_dtype >= 0 && x_dtype <= 2 && n_tokens > 1 &&
         n_tokens <= kWindowHeadTokens && maya_moe_route_window_ok(router, n_tokens, n_expert, k)) {

@@ -1,4 +1,4 @@
-"""GPU parity of the single-token IQ2_S layer whose head rides in the gate/up launch: every gate/up workgroup picks the
+"""GPU parity of the single-token layer whose head rides in the gate/up launch (IQ2_S first, the other types below): every gate/up workgroup picks the
 token's experts from the ORDER of the logits and rounds x itself, so the cases here are the ones where the order of the
 logits and the order of the rounded probabilities can differ (ties, near ties, probabilities in the sub-normal range,
 NaN / Inf) - the layer must give the ids, weights and output, bit for bit, of the layer that routes with the exact
@@ -263,3 +263,59 @@ def test_sigmoid_router_in_the_gate_up_launch(lib, norm, with_bias):
     torch.cuda.synchronize()
     assert bad == 0, bad
     assert int(want_ids[-1, 0]) == -1 and int(want_ids[-2, 0]) == -1          # the refused rows were in the set
+
+
+@pytest.mark.parametrize("ty,n_embd,n_ff,ne,k", ((12, 2048, 512, 40, 8), (12, 2048, 2048, 12, 8), (12, 3072, 512, 9, 4), (12, 7168, 256, 6, 1),
+                                                   (19, 2048, 512, 40, 8), (19, 3072, 256, 9, 4), (19, 5120, 256, 7, 2)))
+def test_other_types_head_in_the_gate_up_launch(lib, oracle, ty, n_embd, n_ff, ne, k):
+    """The same for Q4_K and IQ1_S experts (their position-mapped gate/up kernels with the head in them): for Q4_K
+    the 8-row launch of few entries and the 16-row one; row lengths whose middle wave holds gate and up lanes (3072,
+    5120); one slot (k = 1); F32, BF16 and F16 x; edge logits; the sigmoid router.  ids, weights and output bit for bit
+    those of the three-launch layer, and the CPU path's within 1e-3."""
+    blobs = make_experts(ty, ty, n_embd, n_ff, ne, 500 + ne)
+    gguf_layout, _ = lib.layout(ty, ty, n_embd, n_ff)
+    store = lib.ExpertStore(blobs, pack_layout=gguf_layout)
+    fused, plain = lib.MoeLayer(ty, ty, n_embd, n_ff, ne, k, packing=1), lib.MoeLayer(ty, ty, n_embd, n_ff, ne, k, packing=1)
+    rng = np.random.default_rng(n_embd + ne)
+    x32 = rng.standard_normal(n_embd).astype(np.float32)
+    x32[256:512] = 0.0
+    x32[600], x32[700] = 9.0, -9.0
+    rows = [rng.standard_normal(ne).astype(np.float32) for _ in range(6)]
+    c = rows[0].copy()
+    c[[1, 4]] = np.float32(2.5)                                   # a tie at the top
+    rows.append(c)
+    c = rows[1].copy()
+    order = np.argsort(-c)
+    c[order[k]] = c[order[k - 1]]                                 # a tie at the cut
+    rows.append(c)
+    c = rows[2].copy()
+    c[order[0]] = np.nextafter(c[order[1]], np.float32(10))       # one unit in the last place apart
+    rows.append(c)
+    rows.append(np.zeros(ne, dtype=np.float32))
+    c = rows[3].copy()
+    c[2] = np.float32(np.nan)
+    rows.append(c)
+    bias = dev((rng.standard_normal(ne) * 0.1).astype(np.float32))
+    routers = (None, lib.Router(lib.ROUTER_SIGMOID, 1, bias.data_ptr(), 2.5))
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        xa = torch.zeros(n_embd + 16, dtype=dtype, device="cuda")
+        off = 8 // xa.element_size()
+        x_al, x_un = xa[:n_embd].view(1, n_embd), xa[off:off + n_embd].view(1, n_embd)
+        for router in routers:
+            for i, lg in enumerate(rows):
+                print("case", n_embd, n_ff, dtype, router is not None, i, flush=True)
+                logits = dev(lg.reshape(1, ne))
+                x_al.copy_(torch.from_numpy(x32).to(dtype).view(1, -1))
+                out_f = fused.forward(store.table, logits, x_al, router=router).clone()
+                ids_f, w_f = fused.ids.clone(), fused.weights.clone()
+                x_un.copy_(torch.from_numpy(x32).to(dtype).view(1, -1))
+                out_p = plain.forward(store.table, logits, x_un, router=router).clone()
+                torch.cuda.synchronize()
+                assert torch.equal(ids_f, plain.ids), (i, ids_f, plain.ids)
+                assert torch.equal(w_f.view(torch.int32), plain.weights.view(torch.int32)), i
+                assert torch.equal(out_f.view(torch.int32), out_p.view(torch.int32)), i
+    lg = rows[0].reshape(1, ne)
+    xin = torch.from_numpy(x32)
+    out = fused.forward(store.table, dev(lg), xin.cuda().view(1, -1)).cpu().numpy()
+    wi, ww, wout = oracle_layer(oracle, ty, ty, blobs, k, n_embd, n_ff, lg, x32.reshape(1, -1))
+    assert np.array_equal(fused.ids.cpu().numpy(), wi) and rel_l2(out[0], wout[0]) <= 1e-3
