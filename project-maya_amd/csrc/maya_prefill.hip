@@ -573,9 +573,12 @@ __device__ __forceinline__ void pf_tile(const PfGemm& a, uint8_t* b0, uint8_t* b
                 for (int c = 0; c < 4; ++c) q[c] = qn[c];
             }
         }
-        // super-block sb + 1 has landed once only this iteration's copies (of sb + 2) may still be in flight
+        // super-block sb + 1 has landed once only the wave's youngest NMT operations may still be in flight: this
+        // iteration's copies (of sb + 2), or - in the last steps, which copy nothing - some of the five weight loads
+        // issued above; a wave that holds no weight rows has nothing younger than its last copies then and waits for all
         // (a bare barrier: __syncthreads() would first wait for every memory operation of the wave, these copies included)
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NMT) : "memory");
+        if (sb + 2 < nsb || wave_on) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NMT) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
     for (int sb = 0; sb < nsb; sb += 3) {
         step(sb, b0, b2);
